@@ -1,0 +1,255 @@
+// extern "C" surface of libhingetree_hip.so (declared in include/hingetree_hip.h) and the host-only pieces.
+#include <cmath>
+#include <limits>
+
+#include "common.hpp"
+
+namespace ht {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string &msg) { g_last_error = msg; }
+int fail(int code, const std::string &msg) {
+  g_last_error = msg;
+  return code;
+}
+
+// Shape rules and messages of hingetree.cpp:66-94 that can be decided from sizes alone.
+int make_dims(const ht_forest_shape *s, ForestDims *d) {
+  if (!s) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null shape.");
+  if (s->dtype != HT_F32 && s->dtype != HT_F64)
+    return fail(HT_ERR_INVALID_ARGUMENT,
+                "Error: Unsupported data type. Only torch.float32 and torch.float64 are supported.");
+  if (s->kind != HT_TREE && s->kind != HT_FERN) return fail(HT_ERR_INVALID_ARGUMENT, "Error: unknown tree kind.");
+  if (s->depth < 0 || s->depth > 31)  // 32-bit leaf keys, HingeTreeCommon.h:51,138
+    return fail(HT_ERR_RUNTIME,
+                "Error: The tree depth exceeds compile-time constraints or the number of thresholds is incorrect for "
+                "the tree depth (tree depth = " + std::to_string((long long)s->depth) + ").");
+  if (s->B < 0 || s->F < 0 || s->K < 0 || s->T < 0 || s->M < 0)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  const long long V = s->kind == HT_FERN ? s->depth : ((1LL << s->depth) - 1), L = 1LL << s->depth;
+  const long long lim = 0x7fffffffLL;
+  if (s->F > lim || s->K > lim || s->T > lim || s->M > lim || V > lim || L > lim || L * s->M > lim)
+    return fail(HT_ERR_RUNTIME, "Error: a tensor dimension exceeds the 32-bit limits of this build.");
+  if (s->depth > 0 && V == 0) return fail(HT_ERR_RUNTIME, "Error: inconsistent tree shape.");
+  d->S = s->B * s->K;
+  d->FK = s->F * s->K;
+  d->F = int(s->F);
+  d->K = int(s->K);
+  d->T = int(s->T);
+  d->depth = int(s->depth);
+  d->V = int(V);
+  d->L = int(L);
+  d->M = int(s->M);
+  return HT_OK;
+}
+
+// ---- threshold consistency (host memory) -----------------------------------------------------------------------
+// A vertex that re-tests a feature already tested by an ancestor must keep its threshold on the side of the ancestor's
+// threshold that its path came from (HingeTreeCommon.h:211-287).
+template <typename Real>
+static bool tree_consistent(const Real *thr, const int64_t *ord, int64_t V) {
+  for (int64_t i = V - 1; i > 0; --i) {
+    int64_t child = i;
+    while (child > 0) {
+      const int64_t up = (child - 1) >> 1;
+      if (ord[up] == ord[i]) {
+        const bool from_right = (child & 1) == 0;  // right children have even heap indices
+        if (from_right ? thr[i] < thr[up] : thr[i] > thr[up]) return false;
+      }
+      child = up;
+    }
+  }
+  return true;
+}
+
+template <typename Real>
+static bool tree_repair(Real *thr, const int64_t *ord, int64_t V) {
+  bool changed = false;
+  const Real inf = std::numeric_limits<Real>::infinity();
+  for (int64_t i = 1; i < V; ++i) {
+    Real lower = -inf, upper = inf;
+    int64_t child = i;
+    while (child > 0) {
+      const int64_t up = (child - 1) >> 1;
+      if (ord[up] == ord[i]) {
+        if ((child & 1) == 0)
+          lower = std::max(lower, thr[up]);
+        else
+          upper = std::min(upper, thr[up]);
+      }
+      child = up;
+    }
+    if (thr[i] < lower || thr[i] > upper) {
+      if (!std::isfinite(lower))
+        thr[i] = upper - Real(1);
+      else if (!std::isfinite(upper))
+        thr[i] = lower + Real(1);
+      else
+        thr[i] = Real(0.5) * (lower + upper);
+      changed = true;
+    }
+  }
+  return changed;
+}
+
+}  // namespace ht
+
+using namespace ht;
+
+extern "C" {
+
+const char *ht_last_error(void) { return g_last_error.c_str(); }
+int ht_abi_version(void) { return 1; }
+
+int ht_ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, void *stream) {
+  if (!minmax || (n > 0 && !ord)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return ordinal_range(ord, n, minmax, static_cast<hipStream_t>(stream));
+}
+
+size_t ht_forest_forward_workspace(const ht_forest_shape *) { return 0; }
+
+int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
+                      void *out, void *, size_t, void *stream) {
+  ForestDims d;
+  int rc = make_dims(s, &d);
+  if (rc != HT_OK) return rc;
+  if (d.S > 0 && d.T > 0 && (!x || !thr || !ord || !w || !out))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool fern = s->kind == HT_FERN;
+  if (s->dtype == HT_F32)
+    return forest_forward<float>(d, fern, (const float *)x, (const float *)thr, ord, (const float *)w, (float *)out, st);
+  return forest_forward<double>(d, fern, (const double *)x, (const double *)thr, ord, (const double *)w, (double *)out,
+                                st);
+}
+
+size_t ht_forest_backward_workspace(const ht_forest_shape *s, int mode, int, int, int) {
+  ForestDims d;
+  if (make_dims(s, &d) != HT_OK) return 0;
+  return s->dtype == HT_F32 ? forest_backward_workspace<float>(d, mode) : forest_backward_workspace<double>(d, mode);
+}
+
+int ht_forest_backward(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
+                       const void *gout, void *dx, void *dthr, void *dw, int mode, void *workspace,
+                       size_t workspace_bytes, void *stream) {
+  ForestDims d;
+  int rc = make_dims(s, &d);
+  if (rc != HT_OK) return rc;
+  if (mode != HT_BACKWARD_ATOMIC && mode != HT_BACKWARD_DETERMINISTIC)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: unknown backward mode.");
+  if (d.S > 0 && d.T > 0 && (!x || !thr || !ord || !w || !gout))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool fern = s->kind == HT_FERN;
+  if (s->dtype == HT_F32)
+    return forest_backward<float>(d, fern, (const float *)x, (const float *)thr, ord, (const float *)w,
+                                  (const float *)gout, (float *)dx, (float *)dthr, (float *)dw, mode, workspace,
+                                  workspace_bytes, st);
+  return forest_backward<double>(d, fern, (const double *)x, (const double *)thr, ord, (const double *)w,
+                                 (const double *)gout, (double *)dx, (double *)dthr, (double *)dw, mode, workspace,
+                                 workspace_bytes, st);
+}
+
+size_t ht_forest_maps_workspace(const ht_forest_shape *) { return 0; }
+
+int ht_forest_maps(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, int64_t *leafmap,
+                   void *margins, int64_t *ordinals, int64_t *reach, void *, size_t, void *stream) {
+  ForestDims d;
+  int rc = make_dims(s, &d);
+  if (rc != HT_OK) return rc;
+  if (d.S > 0 && d.T > 0 && (!x || !thr || !ord)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool fern = s->kind == HT_FERN;
+  if (s->dtype == HT_F32)
+    return forest_maps<float>(d, fern, (const float *)x, (const float *)thr, ord, leafmap, (float *)margins, ordinals,
+                              reach, st);
+  return forest_maps<double>(d, fern, (const double *)x, (const double *)thr, ord, leafmap, (double *)margins, ordinals,
+                             reach, st);
+}
+
+static int check_conv(const ht_conv_shape *s) {
+  if (!s) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null shape.");
+  if (s->dtype != HT_F32 && s->dtype != HT_F64)
+    return fail(HT_ERR_INVALID_ARGUMENT,
+                "Error: Unsupported data type. Only torch.float32 and torch.float64 are supported.");
+  if (s->depth < 0 || s->depth > 31)
+    return fail(HT_ERR_RUNTIME,
+                "Error: The tree depth exceeds compile-time constraints or the number of thresholds is incorrect for "
+                "the tree depth (tree depth = " + std::to_string((long long)s->depth) + ").");
+  if (s->B < 0 || s->C < 0 || s->Cout < 0 || s->M < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if ((1LL << s->depth) * s->M > 0x7fffffffLL || s->C > 0x7fffffffLL)
+    return fail(HT_ERR_RUNTIME, "Error: a tensor dimension exceeds the 32-bit limits of this build.");
+  return HT_OK;
+}
+
+int ht_conv_output_size(const ht_conv_shape *s, int64_t *out_size) {
+  int rc = check_conv(s);
+  if (rc != HT_OK) return rc;
+  return conv_output_size(*s, out_size);
+}
+
+int ht_conv_forward(const ht_conv_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w, void *out,
+                    void *stream) {
+  int rc = check_conv(s);
+  if (rc != HT_OK) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (s->dtype == HT_F32)
+    return conv_forward<float>(*s, (const float *)x, (const float *)thr, ord, (const float *)w, (float *)out, st);
+  return conv_forward<double>(*s, (const double *)x, (const double *)thr, ord, (const double *)w, (double *)out, st);
+}
+
+int ht_conv_backward(const ht_conv_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
+                     const void *gout, void *dx, void *dthr, void *dw, void *stream) {
+  int rc = check_conv(s);
+  if (rc != HT_OK) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (s->dtype == HT_F32)
+    return conv_backward<float>(*s, (const float *)x, (const float *)thr, ord, (const float *)w, (const float *)gout,
+                                (float *)dx, (float *)dthr, (float *)dw, st);
+  return conv_backward<double>(*s, (const double *)x, (const double *)thr, ord, (const double *)w, (const double *)gout,
+                               (double *)dx, (double *)dthr, (double *)dw, st);
+}
+
+static int thresholds_common(int64_t T, int64_t depth, int32_t dtype, int32_t kind, int64_t *V) {
+  if (dtype != HT_F32 && dtype != HT_F64)
+    return fail(HT_ERR_INVALID_ARGUMENT,
+                "Error: Unsupported data type. Only torch.float32 and torch.float64 are supported.");
+  if (T < 0 || depth < 0 || depth > 31) return fail(HT_ERR_RUNTIME, "Error: invalid tree shape.");
+  *V = kind == HT_FERN ? depth : ((int64_t(1) << depth) - 1);
+  return HT_OK;
+}
+
+int ht_check_thresholds(const void *thr, const int64_t *ord, int64_t T, int64_t depth, int32_t dtype, int32_t kind,
+                        uint8_t *flags) {
+  int64_t V;
+  int rc = thresholds_common(T, depth, dtype, kind, &V);
+  if (rc != HT_OK) return rc;
+  for (int64_t t = 0; t < T; ++t) {
+    if (kind == HT_FERN)
+      flags[t] = 1;
+    else if (dtype == HT_F32)
+      flags[t] = tree_consistent<float>((const float *)thr + t * V, ord + t * V, V);
+    else
+      flags[t] = tree_consistent<double>((const double *)thr + t * V, ord + t * V, V);
+  }
+  return HT_OK;
+}
+
+int ht_fix_thresholds(void *thr, const int64_t *ord, int64_t T, int64_t depth, int32_t dtype, int32_t kind,
+                      uint8_t *flags) {
+  int64_t V;
+  int rc = thresholds_common(T, depth, dtype, kind, &V);
+  if (rc != HT_OK) return rc;
+  for (int64_t t = 0; t < T; ++t) {
+    if (kind == HT_FERN)
+      flags[t] = 0;
+    else if (dtype == HT_F32)
+      flags[t] = tree_repair<float>((float *)thr + t * V, ord + t * V, V);
+    else
+      flags[t] = tree_repair<double>((double *)thr + t * V, ord + t * V, V);
+  }
+  return HT_OK;
+}
+
+}  // extern "C"

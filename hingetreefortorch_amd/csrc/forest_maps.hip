@@ -1,0 +1,158 @@
+// Leaf map, margin map, reachability, ordinal range and the zero-fill helper.
+#include "forest_tile.hpp"
+
+namespace ht {
+namespace {
+
+// Same tile walk as the forward; each (sample, tree) pair writes its observables directly.
+template <typename Real, bool FERN, int BT, bool XLDS>
+__global__ __launch_bounds__(kForestThreads) void maps_kernel(ForestDims d, const Real *__restrict__ x,
+                                                              const Real *__restrict__ thr,
+                                                              const int64_t *__restrict__ ord, int64_t *leafmap,
+                                                              Real *margins, int64_t *ordinals,
+                                                              unsigned long long *reach, int trees_per_block) {
+  constexpr int NT = kForestThreads;
+  constexpr int TC = NT / BT;
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *xs = reinterpret_cast<Real *>(smem);
+  const long long s0 = (long long)blockIdx.x * BT;
+  if (XLDS) {
+    load_tile<Real, BT, NT>(xs, x, d, s0);
+    __syncthreads();
+  }
+  const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
+  const long long s = s0 + j;
+  if (s >= d.S) return;
+  const long long b = s / d.K, k = s % d.K;
+  const long long xbase = b * d.FK + k;
+  const int t_begin = blockIdx.y * trees_per_block;
+  const int t_end = min(d.T, t_begin + trees_per_block);
+  for (int t = t_begin + tt; t < t_end; t += TC) {
+    const Real *th = thr + (long long)t * d.V;
+    const int64_t *od = ord + (long long)t * d.V;
+    auto node = [&](uint32_t at, Real &tv, int &ov) { tv = th[at]; ov = clamp_ordinal(od[at], d.F); };
+    WalkResult<Real> r;
+    if (XLDS)
+      r = walk<Real, FERN>(d.depth, node, [&](int f) { return xs[f * BT + j]; });
+    else
+      r = walk<Real, FERN>(d.depth, node, [&](int f) { return x[xbase + (long long)f * d.K]; });
+    const long long at = (b * d.T + t) * d.K + k;
+    if (leafmap) leafmap[at] = (int64_t)r.key;
+    if (margins) margins[at] = r.margin;
+    if (ordinals) ordinals[at] = od[r.vertex];
+    if (reach) atomicAdd(reach + (long long)t * d.L + r.key, 1ull);
+  }
+}
+
+template <typename Real, bool FERN, int BT, bool XLDS>
+int launch_maps(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap, Real *margins,
+                int64_t *ordinals, int64_t *reach, hipStream_t stream) {
+  constexpr int TC = kForestThreads / BT;
+  const size_t lds = XLDS ? size_t(d.F) * BT * sizeof(Real) : 0;
+  const long long tiles = (d.S + BT - 1) / BT;
+  const int passes = (d.T + TC - 1) / TC;
+  long long want = tiles >= 512 ? 1 : (512 + tiles - 1) / tiles;
+  const int split = int(want < passes ? want : passes);
+  const int trees_per_block = ((passes + split - 1) / split) * TC;
+  const int gy = (d.T + trees_per_block - 1) / trees_per_block;
+  if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
+  auto kernel = maps_kernel<Real, FERN, BT, XLDS>;
+  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   int(lds)));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, thr, ord,
+                     leafmap, margins, ordinals, reinterpret_cast<unsigned long long *>(reach), trees_per_block);
+  HT_LAUNCH_CHECK("forest maps");
+  return HT_OK;
+}
+
+template <typename Real, bool FERN>
+int dispatch_maps(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap,
+                  Real *margins, int64_t *ordinals, int64_t *reach, hipStream_t stream) {
+  switch (pick_tile<Real>(d.F, 1024)) {
+    case 64: return launch_maps<Real, FERN, 64, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
+    case 32: return launch_maps<Real, FERN, 32, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
+    case 16: return launch_maps<Real, FERN, 16, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
+    case 8: return launch_maps<Real, FERN, 8, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
+    default: return launch_maps<Real, FERN, 64, false>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
+  }
+}
+
+__global__ void zero_kernel(uint32_t *p, size_t words) {
+  for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < words; i += size_t(gridDim.x) * blockDim.x)
+    p[i] = 0u;
+}
+
+__global__ void zero_tail_kernel(unsigned char *p, size_t bytes) {
+  if (threadIdx.x < bytes) p[threadIdx.x] = 0;
+}
+
+__global__ void minmax_init_kernel(long long *mm) {
+  mm[0] = 0x7fffffffffffffffLL;
+  mm[1] = -0x7fffffffffffffffLL - 1;
+}
+
+__global__ __launch_bounds__(256) void minmax_kernel(const long long *__restrict__ v, long long n, long long *mm) {
+  long long lo = 0x7fffffffffffffffLL, hi = -0x7fffffffffffffffLL - 1;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+    const long long a = v[i];
+    lo = a < lo ? a : lo;
+    hi = a > hi ? a : hi;
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const long long lo2 = __shfl_xor(lo, off, kWave), hi2 = __shfl_xor(hi, off, kWave);
+    lo = lo2 < lo ? lo2 : lo;
+    hi = hi2 > hi ? hi2 : hi;
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    atomicMin(mm, lo);
+    atomicMax(mm + 1, hi);
+  }
+}
+
+}  // namespace
+
+int zero_fill(void *p, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return HT_OK;
+  const size_t words = bytes / 4, tail = bytes % 4;
+  if (words) {
+    size_t blocks = (words + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, static_cast<uint32_t *>(p), words);
+    HT_LAUNCH_CHECK("zero fill");
+  }
+  if (tail) {
+    hipLaunchKernelGGL(zero_tail_kernel, dim3(1), dim3(4), 0, stream, static_cast<unsigned char *>(p) + words * 4, tail);
+    HT_LAUNCH_CHECK("zero fill tail");
+  }
+  return HT_OK;
+}
+
+int ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, hipStream_t stream) {
+  hipLaunchKernelGGL(minmax_init_kernel, dim3(1), dim3(1), 0, stream, reinterpret_cast<long long *>(minmax));
+  HT_LAUNCH_CHECK("ordinal range init");
+  if (n > 0) {
+    long long blocks = (n + 255) / 256;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(minmax_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                       reinterpret_cast<const long long *>(ord), (long long)n, reinterpret_cast<long long *>(minmax));
+    HT_LAUNCH_CHECK("ordinal range");
+  }
+  return HT_OK;
+}
+
+template <typename Real>
+int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap,
+                Real *margins, int64_t *ordinals, int64_t *reach, hipStream_t stream) {
+  int rc;
+  if (reach && (rc = zero_fill(reach, size_t(d.T) * d.L * sizeof(int64_t), stream)) != HT_OK) return rc;
+  if (d.S == 0 || d.T == 0) return HT_OK;
+  return fern ? dispatch_maps<Real, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream)
+              : dispatch_maps<Real, false>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
+}
+
+template int forest_maps<float>(const ForestDims &, bool, const float *, const float *, const int64_t *, int64_t *,
+                                float *, int64_t *, int64_t *, hipStream_t);
+template int forest_maps<double>(const ForestDims &, bool, const double *, const double *, const int64_t *, int64_t *,
+                                 double *, int64_t *, int64_t *, hipStream_t);
+
+}  // namespace ht

@@ -1,0 +1,39 @@
+// Sample tile shared by the forest kernels.
+//
+// A workgroup owns BT consecutive samples (a sample is one (batch row, inner position) pair) and keeps all F features
+// of them in LDS, feature major: xs[f * BT + j]. With lane = sample, a gather of *different* features by different
+// lanes touches bank (j mod 32) only, so the data-dependent reads of the walk never conflict.
+#pragma once
+#include "common.hpp"
+#include "walk.hpp"
+
+namespace ht {
+
+// Largest tile width whose feature-major copy fits the LDS budget left after `reserve` bytes; 0 if even 8 do not fit.
+template <typename Real>
+static inline int pick_tile(int F, size_t reserve) {
+  const int candidates[4] = {64, 32, 16, 8};
+  for (int bt : candidates)
+    if (size_t(F) * bt * sizeof(Real) + reserve <= size_t(kLdsBytes)) return bt;
+  return 0;
+}
+
+// Cooperative load of the tile starting at sample s0. NT must be a multiple of BT, so a thread always serves the
+// same sample j and only its feature index advances.
+template <typename Real, int BT, int NT>
+__device__ __forceinline__ void load_tile(Real *xs, const Real *__restrict__ x, const ForestDims &d, long long s0) {
+  const int j = threadIdx.x % BT;
+  const long long s = s0 + j;
+  const bool live = s < d.S;
+  const long long base = live ? (s / d.K) * d.FK + (s % d.K) : 0;
+  for (int f = threadIdx.x / BT; f < d.F; f += NT / BT)
+    xs[f * BT + j] = live ? x[base + (long long)f * d.K] : Real(0);
+}
+
+// Flat offset of element (sample s, tree t, output m) of the [B, T, K, M] output / upstream-gradient tensors.
+__device__ __forceinline__ long long out_offset(const ForestDims &d, long long s, int t, int m) {
+  const long long b = s / d.K, k = s % d.K;
+  return ((b * d.T + t) * d.K + k) * d.M + m;
+}
+
+}  // namespace ht

@@ -1,0 +1,129 @@
+"""Autograd functions with the reference's public names (HingeTree/_HingeTree.py:92-186, 370-506).
+
+`HingeTree`, `HingeFern` and the six convolution functions keep the reference's `apply` signatures, static helper
+methods and the rule that `torch.use_deterministic_algorithms(True)` selects the deterministic backward
+(_HingeTree.py:24-30,103-106). The convolutions have no deterministic backward in the reference either and raise the
+same RuntimeError under that switch (_HingeTree.py:384-385).
+"""
+import torch
+
+from . import hingetree_cpp as _ops
+
+
+def _is_deterministic():
+    if hasattr(torch, "are_deterministic_algorithms_enabled"):
+        return torch.are_deterministic_algorithms_enabled()
+    if hasattr(torch, "is_deterministic"):
+        return torch.is_deterministic()
+    raise RuntimeError("Unable to query torch deterministic mode.")
+
+
+class _ForestFunction(torch.autograd.Function):
+    """forward(ctx, inData, inThresholds, inOrdinals, inWeights); gradients for data, thresholds and weights."""
+    _prefix = None  # "tree" | "fern"
+
+    @classmethod
+    def _op(cls, name):
+        return getattr(_ops, f"{cls._prefix}_{name}")
+
+    @staticmethod
+    def _forward(cls, ctx, inData, inThresholds, inOrdinals, inWeights):
+        ctx.save_for_backward(inData, inThresholds, inOrdinals, inWeights)
+        return cls._op("forward")(inData, inThresholds, inOrdinals, inWeights)
+
+    @staticmethod
+    def _backward(cls, ctx, outDataGrad):
+        inData, inThresholds, inOrdinals, inWeights = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        op = cls._op("backward_deterministic" if _is_deterministic() else "backward")
+        grads = op(inData, need[0], inThresholds, need[1], inOrdinals, need[2], inWeights, need[3],
+                   outDataGrad.contiguous())
+        return tuple(grads)
+
+    # static helpers of the reference classes
+    @classmethod
+    def check_thresholds(cls, inThresholds, inOrdinals, inWeights):
+        return cls._op("check_thresholds")(inThresholds, inOrdinals, inWeights)
+
+    @classmethod
+    def fix_thresholds(cls, inThresholds, inOrdinals, inWeights):
+        return cls._op("fix_thresholds")(inThresholds, inOrdinals, inWeights)
+
+    @classmethod
+    def reachability(cls, inData, inThresholds, inOrdinals, inWeights):
+        return cls._op("reachability")(inData, inThresholds, inOrdinals, inWeights)
+
+    @classmethod
+    def leafmap(cls, inData, inThresholds, inOrdinals, inWeights):
+        return cls._op("leafmap")(inData, inThresholds, inOrdinals, inWeights)
+
+    @classmethod
+    def marginmap(cls, inData, inThresholds, inOrdinals, inWeights):
+        return cls._op("marginmap")(inData, inThresholds, inOrdinals, inWeights)
+
+    @classmethod
+    def speedtest(cls, inData):
+        return cls._op("speedtest")(inData, _is_deterministic())
+
+    @classmethod
+    def init_medians(cls, inData, inThresholds, inOrdinals, inWeights):
+        return cls._op("init_medians")(inData, inThresholds, inOrdinals, inWeights)
+
+
+class HingeTree(_ForestFunction):
+    _prefix = "tree"
+
+    @staticmethod
+    def forward(ctx, inData, inThresholds, inOrdinals, inWeights):
+        return _ForestFunction._forward(HingeTree, ctx, inData, inThresholds, inOrdinals, inWeights)
+
+    @staticmethod
+    def backward(ctx, outDataGrad):
+        return _ForestFunction._backward(HingeTree, ctx, outDataGrad)
+
+    @staticmethod
+    def init_greedy(inData, inLabels, inThresholds, inOrdinals, inWeights):
+        return _ops.tree_init_greedy(inData, inLabels, inThresholds, inOrdinals, inWeights)
+
+
+class HingeFern(_ForestFunction):
+    _prefix = "fern"
+
+    @staticmethod
+    def forward(ctx, inData, inThresholds, inOrdinals, inWeights):
+        return _ForestFunction._forward(HingeFern, ctx, inData, inThresholds, inOrdinals, inWeights)
+
+    @staticmethod
+    def backward(ctx, outDataGrad):
+        return _ForestFunction._backward(HingeFern, ctx, outDataGrad)
+
+
+def _conv_function(name, prefix, nd, label):
+    fwd = getattr(_ops, f"{prefix}_conv{nd}d_forward")
+    bwd = getattr(_ops, f"{prefix}_conv{nd}d_backward")
+
+    def forward(ctx, inData, inThresholds, inOrdinals, inWeights, kernelSize, stride, padding, dilation):
+        ctx.save_for_backward(inData, inThresholds, inOrdinals, inWeights)
+        ctx.kernelSize, ctx.stride, ctx.padding, ctx.dilation = kernelSize, stride, padding, dilation
+        return fwd(inData, inThresholds, inOrdinals, inWeights, kernelSize, stride, padding, dilation)
+
+    def backward(ctx, outDataGrad):
+        if _is_deterministic() and outDataGrad.device.type != "cpu":
+            raise RuntimeError(f"No deterministic implementation of backpropagation for hinge {label} convolution on "
+                               "GPUs.")
+        inData, inThresholds, inOrdinals, inWeights = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        grads = bwd(inData, need[0], inThresholds, need[1], inOrdinals, need[2], inWeights, need[3],
+                    outDataGrad.contiguous(), ctx.kernelSize, ctx.stride, ctx.padding, ctx.dilation)
+        return tuple(grads) + (None, None, None, None)
+
+    return type(name, (torch.autograd.Function,), {"forward": staticmethod(forward), "backward": staticmethod(backward),
+                                                   "__doc__": f"{nd}-d hinge {label} convolution."})
+
+
+HingeTreeConv1d = _conv_function("HingeTreeConv1d", "tree", 1, "tree")
+HingeTreeConv2d = _conv_function("HingeTreeConv2d", "tree", 2, "tree")
+HingeTreeConv3d = _conv_function("HingeTreeConv3d", "tree", 3, "tree")
+HingeFernConv1d = _conv_function("HingeFernConv1d", "fern", 1, "fern")
+HingeFernConv2d = _conv_function("HingeFernConv2d", "fern", 2, "fern")
+HingeFernConv3d = _conv_function("HingeFernConv3d", "fern", 3, "fern")

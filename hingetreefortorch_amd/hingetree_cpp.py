@@ -1,0 +1,457 @@
+"""Host-side mirror of the reference's `hingetree_cpp` operator module (hingetree.cpp:1962-2031) on top of the C ABI.
+
+Same function names, positional signatures, validation order, error types and messages as the reference's dispatchers
+(hingetree.cpp:648-1358, 1736-1926) for the forest / fern / convolution path; tensors are validated here, outputs and
+scratch come from torch's caching allocator, and the kernels are enqueued on torch's current stream of the input's
+device. This build has a single back-end, the HIP library: CPU tensors are rejected (except by the threshold helpers,
+which the reference also keeps on the CPU), and operators outside the path raise.
+"""
+import ctypes
+import time
+import weakref
+
+import torch
+
+from . import _lib as L
+
+__all__ = []  # filled at the bottom
+
+
+def _invalid(msg):
+    raise ValueError(msg)
+
+
+def _runtime(msg):
+    raise RuntimeError(msg)
+
+
+_DT = {torch.float32: L.HT_F32, torch.float64: L.HT_F64}
+
+
+def _prod(xs):
+    r = 1
+    for v in xs:
+        r *= int(v)
+    return r
+
+
+def _ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _compute_depth(leaves):
+    # HingeTreeCommon.h:55-65,141-151: -1 unless the leaf count is a positive power of two
+    if leaves <= 0 or (leaves & (leaves - 1)) != 0:
+        return -1
+    return leaves.bit_length() - 1
+
+
+def _depth_error(depth):
+    _runtime("Error: The tree depth exceeds compile-time constraints or the number of thresholds is incorrect for the "
+             f"tree depth (tree depth = {depth}).")
+
+
+def _require_gpu(t):
+    if t.device.type != "cuda":
+        _runtime("Error: this build of hingetree_cpp has no CPU back-end (its only back-end is the HIP library for "
+                 "MI355X); move the tensors to a ROCm device.")
+
+
+# ---- ordinal range check ------------------------------------------------------------------------------------------
+# The reference reduces inOrdinals to its min and max and reads them back on every call (hingetree.cpp:91,
+# hingetree_gpu.cu:445). The same check runs here, but its verdict is remembered per tensor object and version
+# counter, so a module's fixed `ordinals` parameter costs one device->host read in its lifetime rather than one per
+# call. (Writes through `.data` do not advance the version counter; the kernels therefore also clamp every ordinal
+# into range, so a stale verdict can give wrong numbers but never an out-of-bounds access.)
+_range_ok = {}  # id(tensor) -> (weakref, version, bound) with the proven fact 0 <= ordinals < bound
+
+
+def _validate_ordinals(ordinals, limit):
+    key = id(ordinals)
+    hit = _range_ok.get(key)
+    if hit is not None and hit[0]() is ordinals and hit[1] == ordinals._version and hit[2] <= limit:
+        return
+    bound = 0
+    if ordinals.numel() > 0:
+        mm = torch.empty(2, dtype=torch.int64, device=ordinals.device)
+        with torch.cuda.device(ordinals.device):
+            L.check(L.load().ht_ordinal_range(_ptr(ordinals), ordinals.numel(), _ptr(mm), _stream(ordinals.device)))
+        lo, hi = mm.cpu().tolist()
+        if lo < 0 or hi >= limit:
+            _runtime("Error: An ordinal value is either negative or larger than or equal to the number of channels.")
+        bound = hi + 1
+    try:
+        ref = weakref.ref(ordinals, lambda _r, k=key: _range_ok.pop(k, None))
+    except TypeError:
+        return
+    _range_ok[key] = (ref, ordinals._version, bound)
+
+
+# ---- forest / fern ------------------------------------------------------------------------------------------------
+def _common_checks(tensors, ordinals, with_grad):
+    data = tensors[0]
+    if any(t.dtype != data.dtype for t in tensors) or ordinals.dtype != torch.int64:
+        if with_grad:
+            _invalid("Error: inData, inThresholds, inWeights, outDataGrad are expected to share the same torch real "
+                     "number data type. inOrdinals is expected to be type torch.int64.")
+        _invalid("Error: inData, inThresholds, inWeights are expected to share the same torch real number data type. "
+                 "inOrdinals is expected to be type torch.int64.")
+    if any(t.device != data.device for t in tensors) or ordinals.device != data.device:
+        _invalid("Error: All tensors are expected to be on the same device.")
+    if not all(t.is_contiguous() for t in tensors) or not ordinals.is_contiguous():
+        _invalid("Error: All tensors are expected to be contiguous.")
+    if data.dtype not in _DT:
+        _invalid("Error: Unsupported data type. Only torch.float32 and torch.float64 are supported.")
+
+
+def _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights, outDataGrad=None):
+    """Shape rules of hingetree_cpu_forward / _backward (hingetree.cpp:66-94,164-222) -> ForestShape."""
+    if inData.dim() < 2 or inThresholds.dim() != 2 or inOrdinals.dim() != 2 or inWeights.dim() < 2 or \
+            (outDataGrad is not None and outDataGrad.dim() < 2):
+        _invalid("Error: inData, inWeights must have at least 2 dimensions. inThresholds and inOrdinals must have 2 "
+                 "dimensions.")
+    if inThresholds.shape != inOrdinals.shape or inWeights.shape[0] != inThresholds.shape[0]:
+        _invalid("Error: inThresholds and inOrdinals must be the same shape. inWeights.shape[0] must be the same as "
+                 "inThresholds.shape[0].")
+    leaves = inWeights.shape[1]
+    depth = _compute_depth(leaves)
+    want = depth if kind == L.HT_FERN else (1 << depth) - 1 if depth >= 0 else None
+    if depth > 31 or depth < 0 or inThresholds.shape[1] != want:
+        _depth_error(depth)
+    _require_gpu(inData)
+    _validate_ordinals(inOrdinals, inData.shape[1])
+    shape = L.ForestShape(inData.shape[0], inData.shape[1], _prod(inData.shape[2:]), inWeights.shape[0], depth,
+                          _prod(inWeights.shape[2:]), _DT[inData.dtype], kind)
+    out_sizes = [inData.shape[0], inWeights.shape[0]] + list(inData.shape[2:]) + list(inWeights.shape[2:])
+    if outDataGrad is not None and list(outDataGrad.shape) != out_sizes:
+        _invalid(f"Error: outDataGrad.shape does not match the expected shape ({list(outDataGrad.shape)} != "
+                 f"{out_sizes}).")
+    return shape, out_sizes
+
+
+def _forward(kind, inData, inThresholds, inOrdinals, inWeights):
+    _common_checks([inData, inThresholds, inWeights], inOrdinals, False)
+    shape, out_sizes = _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights)
+    with torch.cuda.device(inData.device):
+        out = torch.empty(out_sizes, dtype=inData.dtype, device=inData.device)
+        lib = L.load()
+        L.check(lib.ht_forest_forward(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals),
+                                      _ptr(inWeights), _ptr(out), None, 0, _stream(inData.device)))
+    return out
+
+
+def _backward(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad, inWeights,
+              bInWeightsGrad, outDataGrad):
+    _common_checks([inData, inThresholds, inWeights, outDataGrad], inOrdinals, True)
+    if bInOrdinalsGrad:  # hingetree.cpp:159-162
+        _runtime("Error: Gradient on inOrdinals is requested, but inOrdinals never has a gradient.")
+    shape, _ = _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights, outDataGrad)
+    with torch.cuda.device(inData.device):
+        dx = torch.empty_like(inData) if bInDataGrad else None
+        dthr = torch.empty_like(inThresholds) if bInThresholdsGrad else None
+        dw = torch.empty_like(inWeights) if bInWeightsGrad else None
+        lib = L.load()
+        nbytes = lib.ht_forest_backward_workspace(ctypes.byref(shape), mode, int(bool(bInDataGrad)),
+                                                  int(bool(bInThresholdsGrad)), int(bool(bInWeightsGrad)))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=inData.device) if nbytes else None
+        L.check(lib.ht_forest_backward(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals),
+                                       _ptr(inWeights), _ptr(outDataGrad), _ptr(dx), _ptr(dthr), _ptr(dw), mode, _ptr(ws),
+                                       nbytes, _stream(inData.device)))
+        if ws is not None:
+            ws.record_stream(torch.cuda.current_stream(inData.device))
+    return [dx, dthr, None, dw]
+
+
+def _maps(kind, inData, inThresholds, inOrdinals, inWeights, want):
+    _common_checks([inData, inThresholds, inWeights], inOrdinals, False)
+    shape, out_sizes = _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights)
+    map_sizes = [inData.shape[0], inWeights.shape[0]] + list(inData.shape[2:])
+    dev = inData.device
+    with torch.cuda.device(dev):
+        leaf = torch.empty(map_sizes, dtype=torch.int64, device=dev) if want == "leaf" else None
+        margins = torch.empty(map_sizes, dtype=inData.dtype, device=dev) if want == "margin" else None
+        ordinals = torch.empty(map_sizes, dtype=torch.int64, device=dev) if want == "margin" else None
+        reach = torch.empty(list(inWeights.shape[:2]), dtype=torch.int64, device=dev) if want == "reach" else None
+        L.check(L.load().ht_forest_maps(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals),
+                                        _ptr(leaf), _ptr(margins), _ptr(ordinals), _ptr(reach), None, 0, _stream(dev)))
+    if want == "leaf":
+        return leaf
+    if want == "margin":
+        return [margins, ordinals]
+    return reach
+
+
+def _thresholds(kind, fix, inThresholds, inOrdinals, inWeights):
+    # hingetree.cpp:930-1076 (dispatch) and :513-581 (shape rules)
+    if inOrdinals.dtype != torch.int64 or inThresholds.dtype != inWeights.dtype:
+        _invalid("Error: inThresholds, inWeights are expected to share the same torch real number data type. inOrdinals "
+                 "is expected to be type torch.int64.")
+    if inThresholds.device.type != "cpu" or inOrdinals.device != inThresholds.device or \
+            inWeights.device != inThresholds.device:
+        _invalid("Error: All tensors are expected to be on the CPU.")
+    if not (inThresholds.is_contiguous() and inOrdinals.is_contiguous() and inWeights.is_contiguous()):
+        _invalid("Error: All tensors are expected to be contiguous.")
+    if inThresholds.dtype not in _DT:
+        _invalid("Error: Unsupported data type. Only torch.float32 and torch.float64 are supported.")
+    if inThresholds.dim() != 2 or inOrdinals.dim() != 2 or inWeights.dim() < 2:
+        _invalid("Error: inWeights must have at least 2 dimensions. inThresholds and inOrdinals must have 2 dimensions.")
+    if inThresholds.shape != inOrdinals.shape or inWeights.shape[0] != inThresholds.shape[0]:
+        _invalid("Error: inThresholds and inOrdinals must be the same shape. inWeights.shape[0] must be the same as "
+                 "inThresholds.shape[0].")
+    depth = _compute_depth(inWeights.shape[1])
+    want = depth if kind == L.HT_FERN else (1 << depth) - 1 if depth >= 0 else None
+    if depth > 31 or depth < 0 or inThresholds.shape[1] != want:
+        _depth_error(depth)
+    T = inThresholds.shape[0]
+    flags = (ctypes.c_uint8 * max(T, 1))()
+    fn = L.load().ht_fix_thresholds if fix else L.load().ht_check_thresholds
+    L.check(fn(_ptr(inThresholds), _ptr(inOrdinals), T, depth, _DT[inThresholds.dtype], kind, flags))
+    return [bool(flags[i]) for i in range(T)]
+
+
+def _speedtest(kind, inData, bDeterministic):
+    """hingetree.cpp:1361-1438: T in {1,2,..,512} x depth in 1..12, 100 forwards then 100 backwards each, wall clock.
+    Unlike the reference this synchronises the device around each timed loop, so it reports execution time."""
+    if inData.dim() < 2:
+        _invalid("Error: inData tensor expected to have at least 2 dimensions (i.e. [batch_size, num_channels, ...]).")
+    name = "hingefern" if kind == L.HT_FERN else "hingetree"
+    num_batches, tree_steps, max_depth = 100, 10, 12
+    timings = torch.zeros([4, tree_steps * max_depth], dtype=torch.float32)
+    fwd = fern_forward if kind == L.HT_FERN else tree_forward
+    if bDeterministic:
+        bwd, bwd_name = (fern_backward_deterministic if kind == L.HT_FERN else tree_backward_deterministic), \
+            name + "_backward_deterministic"
+    else:
+        bwd, bwd_name = (fern_backward if kind == L.HT_FERN else tree_backward), name + "_backward"
+    opts = dict(dtype=inData.dtype, device=inData.device)
+    t = 0
+    for step in range(tree_steps):
+        trees = 1 << step
+        for depth in range(1, max_depth + 1):
+            nodes = depth if kind == L.HT_FERN else (1 << depth) - 1
+            thr = torch.rand([trees, nodes], **opts) * 6.0 - 3.0
+            w = torch.randn([trees, 1 << depth], **opts)
+            ordn = torch.randint(0, inData.shape[1], [trees, nodes], dtype=torch.int64, device=inData.device)
+            timings[0, t], timings[1, t] = trees, depth
+            torch.cuda.synchronize(inData.device)
+            t0 = time.perf_counter()
+            for _ in range(num_batches):
+                out = fwd(inData, thr, ordn, w)
+            torch.cuda.synchronize(inData.device)
+            avg = (time.perf_counter() - t0) * 1e3 / num_batches
+            timings[2, t] = avg
+            print(f"{name}_forward: numBatches = {num_batches}, numTrees = {trees}, depth = {depth}: {avg} ms per batch.",
+                  flush=True)
+            gout = torch.ones_like(out)
+            torch.cuda.synchronize(inData.device)
+            t0 = time.perf_counter()
+            for _ in range(num_batches):
+                bwd(inData, True, thr, True, ordn, False, w, True, gout)
+            torch.cuda.synchronize(inData.device)
+            avg = (time.perf_counter() - t0) * 1e3 / num_batches
+            timings[3, t] = avg
+            print(f"{bwd_name}: numBatches = {num_batches}, numTrees = {trees}, depth = {depth}: {avg} ms per batch.",
+                  flush=True)
+            t += 1
+    return timings
+
+
+def tree_forward(inData, inThresholds, inOrdinals, inWeights):
+    return _forward(L.HT_TREE, inData, inThresholds, inOrdinals, inWeights)
+
+
+def fern_forward(inData, inThresholds, inOrdinals, inWeights):
+    return _forward(L.HT_FERN, inData, inThresholds, inOrdinals, inWeights)
+
+
+def tree_backward(inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad, inWeights,
+                  bInWeightsGrad, outDataGrad):
+    return _backward(L.HT_TREE, L.HT_BACKWARD_ATOMIC, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals,
+                     bInOrdinalsGrad, inWeights, bInWeightsGrad, outDataGrad)
+
+
+def tree_backward_deterministic(inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad,
+                                inWeights, bInWeightsGrad, outDataGrad):
+    return _backward(L.HT_TREE, L.HT_BACKWARD_DETERMINISTIC, inData, bInDataGrad, inThresholds, bInThresholdsGrad,
+                     inOrdinals, bInOrdinalsGrad, inWeights, bInWeightsGrad, outDataGrad)
+
+
+def fern_backward(inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad, inWeights,
+                  bInWeightsGrad, outDataGrad):
+    return _backward(L.HT_FERN, L.HT_BACKWARD_ATOMIC, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals,
+                     bInOrdinalsGrad, inWeights, bInWeightsGrad, outDataGrad)
+
+
+def fern_backward_deterministic(inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad,
+                                inWeights, bInWeightsGrad, outDataGrad):
+    return _backward(L.HT_FERN, L.HT_BACKWARD_DETERMINISTIC, inData, bInDataGrad, inThresholds, bInThresholdsGrad,
+                     inOrdinals, bInOrdinalsGrad, inWeights, bInWeightsGrad, outDataGrad)
+
+
+def tree_check_thresholds(inThresholds, inOrdinals, inWeights):
+    return _thresholds(L.HT_TREE, False, inThresholds, inOrdinals, inWeights)
+
+
+def tree_fix_thresholds(inThresholds, inOrdinals, inWeights):
+    return _thresholds(L.HT_TREE, True, inThresholds, inOrdinals, inWeights)
+
+
+def fern_check_thresholds(inThresholds, inOrdinals, inWeights):
+    return _thresholds(L.HT_FERN, False, inThresholds, inOrdinals, inWeights)
+
+
+def fern_fix_thresholds(inThresholds, inOrdinals, inWeights):
+    return _thresholds(L.HT_FERN, True, inThresholds, inOrdinals, inWeights)
+
+
+def tree_reachability(inData, inThresholds, inOrdinals, inWeights):
+    return _maps(L.HT_TREE, inData, inThresholds, inOrdinals, inWeights, "reach")
+
+
+def tree_leafmap(inData, inThresholds, inOrdinals, inWeights):
+    return _maps(L.HT_TREE, inData, inThresholds, inOrdinals, inWeights, "leaf")
+
+
+def tree_marginmap(inData, inThresholds, inOrdinals, inWeights):
+    return _maps(L.HT_TREE, inData, inThresholds, inOrdinals, inWeights, "margin")
+
+
+def fern_reachability(inData, inThresholds, inOrdinals, inWeights):
+    return _maps(L.HT_FERN, inData, inThresholds, inOrdinals, inWeights, "reach")
+
+
+def fern_leafmap(inData, inThresholds, inOrdinals, inWeights):
+    return _maps(L.HT_FERN, inData, inThresholds, inOrdinals, inWeights, "leaf")
+
+
+def fern_marginmap(inData, inThresholds, inOrdinals, inWeights):
+    return _maps(L.HT_FERN, inData, inThresholds, inOrdinals, inWeights, "margin")
+
+
+def tree_speedtest(inData, bDeterministic):
+    return _speedtest(L.HT_TREE, inData, bDeterministic)
+
+
+def fern_speedtest(inData, bDeterministic):
+    return _speedtest(L.HT_FERN, inData, bDeterministic)
+
+
+# ---- convolution --------------------------------------------------------------------------------------------------
+def _conv_shape(kind, nd, inData, inThresholds, inOrdinals, inWeights, kernelSize, stride, padding, dilation,
+                outDataGrad=None):
+    """Rules of hingetree_conv_cpu_forward / _backward (hingetree_conv.cpp:58-122,240-332)."""
+    kernelSize, stride, padding, dilation = list(kernelSize), list(stride), list(padding), list(dilation)
+    if len(kernelSize) != nd or len(stride) != nd or len(padding) != nd or len(dilation) != nd:
+        _invalid(f"Error: kernel, stride, padding, dilation all expected to have {nd} dimensions.")
+    if inData.dim() != nd + 2 or inThresholds.dim() != 3 or inOrdinals.dim() != 3 or inWeights.dim() < 3:
+        _invalid(f"Error: inData expected to have {nd + 2} dimensions. inThresholds, inOrdinals expected to have 3 "
+                 "dimensions. inWeights expected to be less than 3 dimensions.")
+    if inThresholds.shape != inOrdinals.shape or inWeights.shape[0] != inThresholds.shape[0]:
+        _invalid("Error: inThresholds and inOrdinals must be the same shape. inWeights.shape[0] must be the same as "
+                 "inThresholds.shape[0].")
+    if inWeights.shape[1] == 0:
+        _invalid("Error: inWeights.shape[1] is expected to divide inData.shape[1].")
+    groups = inData.shape[1] // inWeights.shape[1]
+    if groups * inWeights.shape[1] != inData.shape[1]:
+        _invalid("Error: inWeights.shape[1] is expected to divide inData.shape[1].")
+    if groups == 0 or inWeights.shape[0] % groups != 0:
+        _invalid("inData.shape[1]//inWeights.shape[1] is expected to divide output channels.")
+    if groups != 1 or inThresholds.shape[1] != inData.shape[1]:
+        # the reference indexes grouped convolutions inconsistently (hingetree_conv.cpp:125 vs :202-206), so only
+        # groups == 1 has a defined result
+        _runtime("Error: grouped hinge tree convolution (inData.shape[1] != inWeights.shape[1]) is not supported.")
+    shape = L.ConvShape()
+    shape.B, shape.C, shape.Cout = inData.shape[0], inData.shape[1], inWeights.shape[0]
+    shape.M = _prod(inWeights.shape[3:])
+    shape.dtype, shape.kind, shape.nd = _DT[inData.dtype], kind, nd
+    for d in range(nd):
+        shape.size[d], shape.kernel[d], shape.stride[d] = inData.shape[2 + d], kernelSize[d], stride[d]
+        shape.padding[d], shape.dilation[d] = padding[d], dilation[d]
+    depth = _compute_depth(inWeights.shape[2])
+    shape.depth = max(depth, 0)
+    osz = (ctypes.c_int64 * L.HT_MAX_CONV_DIMS)()
+    L.check(L.load().ht_conv_output_size(ctypes.byref(shape), osz))  # "Unable to convert image patches to matrix."
+    _require_gpu(inData)
+    _validate_ordinals(inOrdinals, _prod(kernelSize))
+    want = depth if kind == L.HT_FERN else (1 << depth) - 1 if depth >= 0 else None
+    if depth > 31 or depth < 0 or inThresholds.shape[2] != want:
+        _depth_error(depth)
+    out_sizes = [inData.shape[0], inWeights.shape[0]] + [int(osz[d]) for d in range(nd)] + list(inWeights.shape[3:])
+    if outDataGrad is not None and list(outDataGrad.shape) != out_sizes:
+        _invalid(f"Error: outDataGrad.shape does not match the expected shape ({list(outDataGrad.shape)} != "
+                 f"{out_sizes}).")
+    return shape, out_sizes
+
+
+def _conv_forward(kind, nd, inData, inThresholds, inOrdinals, inWeights, kernelSize, stride, padding, dilation):
+    _common_checks([inData, inThresholds, inWeights], inOrdinals, False)
+    shape, out_sizes = _conv_shape(kind, nd, inData, inThresholds, inOrdinals, inWeights, kernelSize, stride, padding,
+                                   dilation)
+    with torch.cuda.device(inData.device):
+        out = torch.empty(out_sizes, dtype=inData.dtype, device=inData.device)
+        L.check(L.load().ht_conv_forward(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals),
+                                         _ptr(inWeights), _ptr(out), _stream(inData.device)))
+    return out
+
+
+def _conv_backward(kind, nd, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad,
+                   inWeights, bInWeightsGrad, outDataGrad, kernelSize, stride, padding, dilation):
+    _common_checks([inData, inThresholds, inWeights, outDataGrad], inOrdinals, True)
+    if bInOrdinalsGrad:  # hingetree_conv.cpp:235-238
+        _runtime("Error: Gradient on inOrdinals is requested, but inOrdinals never has a gradient.")
+    shape, _ = _conv_shape(kind, nd, inData, inThresholds, inOrdinals, inWeights, kernelSize, stride, padding, dilation,
+                           outDataGrad)
+    with torch.cuda.device(inData.device):
+        dx = torch.empty_like(inData) if bInDataGrad else None
+        dthr = torch.empty_like(inThresholds) if bInThresholdsGrad else None
+        dw = torch.empty_like(inWeights) if bInWeightsGrad else None
+        L.check(L.load().ht_conv_backward(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals),
+                                          _ptr(inWeights), _ptr(outDataGrad), _ptr(dx), _ptr(dthr), _ptr(dw),
+                                          _stream(inData.device)))
+    return [dx, dthr, None, dw]
+
+
+def _make_conv(kind, nd):
+    def forward(inData, inThresholds, inOrdinals, inWeights, kernelSize, stride, padding, dilation):
+        return _conv_forward(kind, nd, inData, inThresholds, inOrdinals, inWeights, kernelSize, stride, padding, dilation)
+
+    def backward(inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad, inWeights,
+                 bInWeightsGrad, outDataGrad, kernelSize, stride, padding, dilation):
+        return _conv_backward(kind, nd, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad,
+                              inWeights, bInWeightsGrad, outDataGrad, kernelSize, stride, padding, dilation)
+
+    return forward, backward
+
+
+tree_conv1d_forward, tree_conv1d_backward = _make_conv(L.HT_TREE, 1)
+tree_conv2d_forward, tree_conv2d_backward = _make_conv(L.HT_TREE, 2)
+tree_conv3d_forward, tree_conv3d_backward = _make_conv(L.HT_TREE, 3)
+fern_conv1d_forward, fern_conv1d_backward = _make_conv(L.HT_FERN, 1)
+fern_conv2d_forward, fern_conv2d_backward = _make_conv(L.HT_FERN, 2)
+fern_conv3d_forward, fern_conv3d_backward = _make_conv(L.HT_FERN, 3)
+
+
+# ---- operators of the reference module that lie outside this build's path -------------------------------------------
+def _outside(name):
+    def stub(*_args, **_kwargs):
+        raise RuntimeError(f"Error: hingetree_cpp.{name} is not part of this build (forest / fern / convolution "
+                           "forward+backward path only).")
+
+    stub.__name__ = name
+    return stub
+
+
+for _name in ["sparse_tree_backward", "sparse_fern_backward", "tree_init_medians", "tree_init_greedy",
+              "fern_init_medians", "trie_forward", "trie_backward", "trie_init_medians", "tree_fused_linear_forward",
+              "tree_fused_linear_backward", "sparse_tree_fused_linear_backward", "fern_fused_linear_forward",
+              "fern_fused_linear_backward", "sparse_fern_fused_linear_backward", "tree_fusion_forward",
+              "tree_fusion_backward", "fern_fusion_forward", "fern_fusion_backward", "tree_fusion_fused_linear_forward",
+              "tree_fusion_fused_linear_backward", "fern_fusion_fused_linear_forward",
+              "fern_fusion_fused_linear_backward", "contract", "expand"]:
+    globals()[_name] = _outside(_name)
+
+__all__ = [n for n in list(globals()) if n.split("_")[0] in ("tree", "fern", "sparse", "trie", "contract", "expand")]

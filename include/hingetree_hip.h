@@ -1,0 +1,108 @@
+/*
+ * hingetree_hip.h -- C ABI of the MI355X (gfx950) hinge forest / hinge fern library (libhingetree_hip.so).
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream (passed as void*, 0 = the null stream).
+ * Nothing here allocates device memory: outputs and scratch ("workspace") are supplied by the caller, whose size
+ * requirement is answered by the matching *_workspace query. All kernels are enqueued on `stream` and the call
+ * returns without synchronising. Tensors are dense, row-major, and must not alias.
+ *
+ * Return value: HT_OK, or an error code with a message retrievable through ht_last_error() (thread local).
+ * HT_ERR_INVALID_ARGUMENT corresponds to the reference's std::invalid_argument (Python ValueError) and HT_ERR_RUNTIME
+ * to its std::runtime_error (Python RuntimeError), hingetree_error.h:38-49.
+ *
+ * Shapes (reference notation, hingetree.cpp:87-135):
+ *   x    [B, F, K]   real          K = product of trailing data dims
+ *   thr  [T, V]      real          V = 2^depth - 1 (tree, heap order) or depth (fern)
+ *   ord  [T, V]      int64         0 <= ord < F  (validated by the caller, see ht_ordinal_range)
+ *   w    [T, L, M]   real          L = 2^depth, M = product of trailing weight dims
+ *   out  [B, T, K, M]
+ */
+#ifndef HINGETREE_HIP_H
+#define HINGETREE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { HT_OK = 0, HT_ERR_INVALID_ARGUMENT = 1, HT_ERR_RUNTIME = 2, HT_ERR_HIP = 3 };
+enum { HT_F32 = 0, HT_F64 = 1 };
+enum { HT_TREE = 0, HT_FERN = 1 };
+/* backward accumulation modes */
+enum { HT_BACKWARD_ATOMIC = 0, HT_BACKWARD_DETERMINISTIC = 1 };
+
+typedef struct ht_forest_shape {
+  int64_t B, F, K, T, depth, M;
+  int32_t dtype; /* HT_F32 | HT_F64 */
+  int32_t kind;  /* HT_TREE | HT_FERN */
+} ht_forest_shape;
+
+#define HT_MAX_CONV_DIMS 3
+typedef struct ht_conv_shape {
+  int64_t B, C, Cout, depth, M;
+  int32_t dtype, kind;
+  int32_t nd; /* 1, 2 or 3 spatial dims */
+  int64_t size[HT_MAX_CONV_DIMS], kernel[HT_MAX_CONV_DIMS], stride[HT_MAX_CONV_DIMS], padding[HT_MAX_CONV_DIMS],
+      dilation[HT_MAX_CONV_DIMS];
+} ht_conv_shape;
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *ht_last_error(void);
+/* ABI version of this header; bumped on any signature change. */
+int ht_abi_version(void);
+
+/* Device-side min and max of n int64 ordinals -> minmax[0], minmax[1] (device memory, 2 x int64).
+ * Replaces the reference's per-call `inOrdinals.min()/.max()` range check (hingetree.cpp:91, hingetree_gpu.cu:445):
+ * the caller reads the two values back and raises the reference's error. */
+int ht_ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, void *stream);
+
+/* out[b,t,k,m] = |margin| * w[t,leaf,m].
+ * Replaces hingetree_gpu_forward / hingefern forward (hingetree.cpp:45,648-693; hingetree_gpu.cu:416-498). */
+size_t ht_forest_forward_workspace(const ht_forest_shape *s);
+int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
+                      void *out, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Gradients of the above w.r.t. x, thr and w; any of dx/dthr/dw may be NULL (not requested). The library clears the
+ * requested buffers itself and then accumulates into them.
+ * mode HT_BACKWARD_ATOMIC replaces hingetree_gpu_backward (hingetree.cpp:48,695-740; hingetree_gpu.cu:619-730);
+ * mode HT_BACKWARD_DETERMINISTIC replaces hingetree_gpu_backward_deterministic (hingetree.cpp:51,742-787;
+ * hingetree_gpu.cu:500-617) and is bit-reproducible run to run. */
+size_t ht_forest_backward_workspace(const ht_forest_shape *s, int mode, int need_dx, int need_dthr, int need_dw);
+int ht_forest_backward(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
+                       const void *gout, void *dx, void *dthr, void *dw, int mode, void *workspace,
+                       size_t workspace_bytes, void *stream);
+
+/* Per-(b,t,k) leaf key / signed margin + selected ordinal / per-(t,leaf) visit counts; any output may be NULL.
+ * Replaces hingetree_gpu_leafmap, _marginmap, _reachability (hingetree.cpp:54-60; hingetree_gpu.cu:732-933), which
+ * return the leaf map and the counts as int64 on the GPU. */
+size_t ht_forest_maps_workspace(const ht_forest_shape *s);
+int ht_forest_maps(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, int64_t *leafmap,
+                   void *margins, int64_t *ordinals, int64_t *reach, void *workspace, size_t workspace_bytes,
+                   void *stream);
+
+/* Convolutional variant, groups == 1: one tree per (out channel, in channel) over the prod(kernel) taps of that in
+ * channel's patch, summed over in channels; the patch gather happens inside the walk (no im2col buffer).
+ *   x [B, C, *size]   thr/ord [Cout, C, V]   w [Cout, C, L, M]   out [B, Cout, *out_size, M]
+ * Replaces hingetree_conv_gpu_forward / _backward (hingetree_conv.cpp:31-47; hingetree_conv_gpu.cu:214-618) and the
+ * ImageToMatrix extraction kernels they launch (ImageToMatrix_gpu.cu:132-239). */
+int ht_conv_output_size(const ht_conv_shape *s, int64_t *out_size /* [nd] */);
+int ht_conv_forward(const ht_conv_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w, void *out,
+                    void *stream);
+int ht_conv_backward(const ht_conv_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
+                     const void *gout, void *dx, void *dthr, void *dw, void *stream);
+
+/* Host-side (CPU pointers) threshold consistency, in place for _fix. One flag byte per tree is written to `flags`
+ * (check: 1 = consistent; fix: 1 = changed). Ferns are always consistent and never change.
+ * Replaces hingetree_cpu_check_thresholds / _fix_thresholds (hingetree.cpp:513-581, HingeTreeCommon.h:211-287); the
+ * reference keeps these on the CPU as well (hingetree.cpp:936,1010). */
+int ht_check_thresholds(const void *thr, const int64_t *ord, int64_t T, int64_t depth, int32_t dtype, int32_t kind,
+                        uint8_t *flags);
+int ht_fix_thresholds(void *thr, const int64_t *ord, int64_t T, int64_t depth, int32_t dtype, int32_t kind,
+                      uint8_t *flags);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HINGETREE_HIP_H */

@@ -1,0 +1,155 @@
+"""GPU parity of the forest / fern operators against the CPU oracle (through the C ABI via the operator layer).
+
+Bars: leaf keys, selected ordinals, signed margins and forward outputs bit-exact; gradients within 1e-5 (fp32,
+relative to the largest reference entry of the tensor; the summation order differs from the serial CPU loop) and
+1e-12 (fp64); deterministic mode bit-identical run to run, and its dX / dW bit-identical to the CPU order.
+"""
+import itertools
+
+import pytest
+import torch
+
+from conftest import make_forest, rel_err
+from oracle import hinge_oracle as ho
+import hingetree_cpp as ops
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # B, F, Kd, T, D, Md
+    (7, 11, [], 5, 1, []),
+    (33, 20, [], 9, 3, [1]),
+    (100, 1000, [], 100, 7, [1]),          # the reference's CPU-runnable configuration
+    (65, 64, [], 40, 6, [10]),
+    (19, 13, [3, 2], 6, 4, [2, 3]),
+    (5, 7, [70], 3, 5, [4]),
+    (130, 300, [], 35, 10, [3]),
+    (4, 5000, [], 3, 4, [2]),              # feature count too large for an LDS tile of 8 float64 rows
+]
+
+
+def _gpu(dev, *ts):
+    return [t.to(dev) for t in ts]
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("case", CASES, ids=[f"c{i}" for i in range(len(CASES))])
+def test_forward_and_maps_bit_exact(dev, case, dtype, fern):
+    B, F, Kd, T, D, Md = case
+    x, thr, ordn, w, _ = make_forest(B, F, Kd, T, D, Md, fern, dtype)
+    ref_out = ho.forward(x, thr, ordn, w, fern)
+    ref_leaf, ref_margin, ref_sel, ref_reach = ho.maps(x, thr, ordn, w, fern)
+    gx, gthr, gord, gw = _gpu(dev, x, thr, ordn, w)
+    pre = "fern_" if fern else "tree_"
+    out = getattr(ops, pre + "forward")(gx, gthr, gord, gw)
+    assert out.shape == ref_out.shape and out.dtype == dtype
+    assert torch.equal(out.cpu(), ref_out)
+    leaf = getattr(ops, pre + "leafmap")(gx, gthr, gord, gw)
+    assert leaf.dtype == torch.int64 and torch.equal(leaf.cpu(), ref_leaf.to(torch.int64))
+    margins, sel = getattr(ops, pre + "marginmap")(gx, gthr, gord, gw)
+    assert torch.equal(margins.cpu(), ref_margin) and torch.equal(sel.cpu(), ref_sel)
+    reach = getattr(ops, pre + "reachability")(gx, gthr, gord, gw)
+    assert reach.dtype == torch.int64 and torch.equal(reach.cpu(), ref_reach.to(torch.int64))
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("case", CASES, ids=[f"c{i}" for i in range(len(CASES))])
+def test_backward_atomic(dev, case, dtype, fern):
+    B, F, Kd, T, D, Md = case
+    x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype)
+    rdx, rdthr, rdw = ho.backward(x, thr, ordn, w, gout, fern=fern)
+    gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
+    pre = "fern_" if fern else "tree_"
+    dx, dthr, dord, dw = getattr(ops, pre + "backward")(gx, True, gthr, True, gord, False, gw, True, gg)
+    assert dord is None
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    assert rel_err(dx.cpu(), rdx) <= tol
+    assert rel_err(dthr.cpu(), rdthr) <= tol
+    assert rel_err(dw.cpu(), rdw) <= tol
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("case", CASES, ids=[f"c{i}" for i in range(len(CASES))])
+def test_backward_deterministic(dev, case, dtype, fern):
+    B, F, Kd, T, D, Md = case
+    x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype)
+    rdx, rdthr, rdw = ho.backward(x, thr, ordn, w, gout, fern=fern)
+    gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
+    fn = getattr(ops, ("fern_" if fern else "tree_") + "backward_deterministic")
+    runs = [fn(gx, True, gthr, True, gord, False, gw, True, gg) for _ in range(3)]
+    for r in runs[1:]:
+        for a, b in zip(r, runs[0]):
+            assert (a is None and b is None) or torch.equal(a, b)
+    dx, dthr, _, dw = runs[0]
+    # dX and dW add their terms in the CPU loop's order: identical bits
+    assert torch.equal(dx.cpu(), rdx)
+    assert torch.equal(dw.cpu(), rdw)
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    assert rel_err(dthr.cpu(), rdthr) <= tol
+
+
+@pytest.mark.parametrize("need", list(itertools.product([False, True], repeat=3)))
+def test_backward_need_subsets(dev, need):
+    x, thr, ordn, w, gout = make_forest(21, 9, [], 4, 3, [2], False, torch.float32)
+    ref = ho.backward(x, thr, ordn, w, gout, need=need)
+    gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
+    for fn in (ops.tree_backward, ops.tree_backward_deterministic):
+        got = fn(gx, need[0], gthr, need[1], gord, False, gw, need[2], gg)
+        assert len(got) == 4 and got[2] is None
+        for g, r in zip((got[0], got[1], got[3]), ref):
+            assert (g is None) == (r is None)
+            if g is not None:
+                assert rel_err(g.cpu(), r) <= 1e-5
+
+
+def test_degenerate_inputs(dev):
+    """margin == 0 goes left with zero output and zero dX/dThr; NaN goes left; +-inf thresholds pin the leaf."""
+    F, T, D = 6, 4, 3
+    x, thr, ordn, w, gout = make_forest(16, F, [], T, D, [2], False, torch.float32, seed=3)
+    x[0, :] = thr[0, 0]                       # exact tie at the root of tree 0 for sample 0
+    x[1, 2] = float("nan")
+    thr[1, :] = float("-inf")                 # always right -> leaf 2^D - 1
+    thr[2, :] = float("inf")                  # always left  -> leaf 0
+    ref_out = ho.forward(x, thr, ordn, w)
+    ref_leaf, ref_margin, ref_sel, _ = ho.maps(x, thr, ordn, w)
+    assert (ref_leaf[:, 1] == 2 ** D - 1).all() and (ref_leaf[:, 2] == 0).all()
+    gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
+    out = ops.tree_forward(gx, gthr, gord, gw).cpu()
+    same = (out == ref_out) | (out.isnan() & ref_out.isnan())
+    assert same.all()
+    assert torch.equal(ops.tree_leafmap(gx, gthr, gord, gw).cpu(), ref_leaf.to(torch.int64))
+    m, s = ops.tree_marginmap(gx, gthr, gord, gw)
+    m = m.cpu()
+    assert ((m == ref_margin) | (m.isnan() & ref_margin.isnan())).all() and torch.equal(s.cpu(), ref_sel)
+
+
+def test_errors(dev):
+    x, thr, ordn, w, gout = [t.to(dev) for t in make_forest(8, 5, [], 3, 2, [], False, torch.float32)]
+    with pytest.raises(ValueError):
+        ops.tree_forward(x.double(), thr, ordn, w)
+    with pytest.raises(ValueError):
+        ops.tree_forward(x, thr, ordn.int(), w)
+    with pytest.raises(ValueError):
+        ops.tree_forward(x.cpu(), thr, ordn, w)
+    with pytest.raises(ValueError):
+        ops.tree_forward(x.t(), thr, ordn, w)
+    with pytest.raises(ValueError):
+        ops.tree_forward(x, thr[:2], ordn, w)
+    with pytest.raises(RuntimeError, match="tree depth = 2"):
+        ops.tree_forward(x, thr[:, :2].contiguous(), ordn[:, :2].contiguous(), w)
+    with pytest.raises(RuntimeError, match="tree depth = -1"):
+        ops.tree_forward(x, thr, ordn, w[:, :3].contiguous())
+    bad = ordn.clone()
+    bad[0, 0] = 5
+    with pytest.raises(RuntimeError, match="ordinal"):
+        ops.tree_forward(x, thr, bad, w)
+    bad[0, 0] = -1
+    with pytest.raises(RuntimeError, match="ordinal"):
+        ops.tree_forward(x, thr, bad, w)
+    with pytest.raises(RuntimeError, match="never has a gradient"):
+        ops.tree_backward(x, True, thr, True, ordn, True, w, True, gout)
+    with pytest.raises(ValueError, match="outDataGrad.shape"):
+        ops.tree_backward(x, True, thr, True, ordn, False, w, True, gout[:4].contiguous())
