@@ -1,0 +1,86 @@
+"""Writes tests/golden/*.npz from the reference's own CPU build (oracle/_ref/hingetree_cpp.so, made by
+`make -C oracle ref` from the sources under /root/reference). Run in the authoring container only:
+
+    python tests/golden/make_golden.py
+
+Each file holds seeded inputs and the reference's outputs for one small case; tests compare the oracle (CPU) and the
+HIP path (GPU) against them. The fixtures are data only.
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+sys.path.insert(0, os.path.dirname(HERE))
+
+from conftest import make_conv, make_forest  # noqa: E402
+from oracle import hinge_oracle as ho  # noqa: E402
+
+FOREST_CASES = {
+    # name: (B, F, Kd, T, D, Md, fern, dtype, x_dist)
+    "tree_f32_plain": (12, 16, [], 6, 4, [], False, torch.float32, "normal"),
+    "tree_f32_m10": (9, 20, [], 5, 5, [10], False, torch.float32, "uniform"),
+    "tree_f32_inner": (4, 6, [3, 2], 3, 3, [2, 2], False, torch.float32, "normal"),
+    "tree_f64_m3": (8, 10, [], 4, 6, [3], False, torch.float64, "normal"),
+    "fern_f32_m1": (12, 16, [], 6, 5, [1], True, torch.float32, "normal"),
+    "fern_f64_inner": (3, 7, [5], 4, 4, [2], True, torch.float64, "normal"),
+}
+
+CONV_CASES = {
+    # name: (B, C, Cout, size, D, Md, kernel, stride, padding, dilation, fern, dtype)
+    "conv1d_tree": (2, 3, 4, [11], 3, [], [3], [2], [1], [1], False, torch.float32),
+    "conv2d_tree": (2, 3, 4, [7, 6], 3, [], [3, 3], [1, 1], [1, 1], [1, 1], False, torch.float32),
+    "conv2d_tree_m3_dil": (1, 2, 3, [9, 8], 2, [3], [3, 2], [2, 1], [2, 0], [2, 2], False, torch.float64),
+    "conv3d_fern": (1, 2, 2, [5, 4, 6], 3, [2], [2, 2, 3], [1, 2, 1], [0, 1, 1], [1, 1, 1], True, torch.float32),
+}
+
+
+def main():
+    ref = ho.reference_module()
+    if ref is None:
+        raise SystemExit("oracle/_ref/hingetree_cpp.so is missing: run `make -C oracle ref` first")
+    for name, (B, F, Kd, T, D, Md, fern, dtype, dist) in FOREST_CASES.items():
+        x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype, seed=11, x_dist=dist)
+        pre = "fern_" if fern else "tree_"
+        if not fern:
+            getattr(ref, pre + "fix_thresholds")(thr, ordn, w)
+        out = getattr(ref, pre + "forward")(x, thr, ordn, w)
+        dx, dthr, _, dw = getattr(ref, pre + "backward")(x, True, thr, True, ordn, False, w, True, gout)
+        leaf = getattr(ref, pre + "leafmap")(x, thr, ordn, w)
+        margin, sel = getattr(ref, pre + "marginmap")(x, thr, ordn, w)
+        reach = getattr(ref, pre + "reachability")(x, thr, ordn, w)
+        np.savez_compressed(os.path.join(HERE, name + ".npz"), fern=np.int64(fern), x=x.numpy(), thr=thr.numpy(),
+                            ord=ordn.numpy(), w=w.numpy(), gout=gout.numpy(), out=out.numpy(), dx=dx.numpy(),
+                            dthr=dthr.numpy(), dw=dw.numpy(), leaf=leaf.numpy(), margin=margin.numpy(), sel=sel.numpy(),
+                            reach=reach.numpy())
+    for name, (B, C, Cout, size, D, Md, ker, st, pad, dil, fern, dtype) in CONV_CASES.items():
+        x, thr, ordn, w = make_conv(B, C, Cout, size, D, Md, ker, fern, dtype, seed=5)
+        nd = len(size)
+        pre = ("fern_" if fern else "tree_") + f"conv{nd}d_"
+        out = getattr(ref, pre + "forward")(x, thr, ordn, w, ker, st, pad, dil)
+        gout = torch.randn(out.shape, generator=torch.Generator().manual_seed(77), dtype=dtype)
+        dx, dthr, _, dw = getattr(ref, pre + "backward")(x, True, thr, True, ordn, False, w, True, gout, ker, st, pad, dil)
+        np.savez_compressed(os.path.join(HERE, name + ".npz"), fern=np.int64(fern), x=x.numpy(), thr=thr.numpy(),
+                            ord=ordn.numpy(), w=w.numpy(), gout=gout.numpy(), out=out.numpy(), dx=dx.numpy(),
+                            dthr=dthr.numpy(), dw=dw.numpy(), kernel=np.array(ker), stride=np.array(st),
+                            padding=np.array(pad), dilation=np.array(dil))
+    # threshold repair: inputs that need fixing, and the reference's in-place result
+    g = torch.Generator().manual_seed(3)
+    thr = 6.0 * torch.rand([12, 31], generator=g) - 3.0
+    ordn = torch.randint(0, 3, [12, 31], generator=g)
+    w = torch.randn([12, 32], generator=g)
+    before = thr.clone()
+    ok_before = ref.tree_check_thresholds(thr, ordn, w)
+    changed = ref.tree_fix_thresholds(thr, ordn, w)
+    ok_after = ref.tree_check_thresholds(thr, ordn, w)
+    np.savez_compressed(os.path.join(HERE, "fix_thresholds.npz"), before=before.numpy(), ord=ordn.numpy(), w=w.numpy(),
+                        after=thr.numpy(), ok_before=np.array(ok_before), changed=np.array(changed),
+                        ok_after=np.array(ok_after))
+    print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))
+
+
+if __name__ == "__main__":
+    main()

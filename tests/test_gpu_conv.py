@@ -1,0 +1,64 @@
+"""GPU parity of the convolutional operators against the CPU oracle: forward bit-exact (ascending-channel accumulation
+from +0, no contraction), gradients within 1e-5 (fp32) / 1e-12 (fp64) relative to the largest reference entry."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, make_conv, rel_err
+from oracle import hinge_oracle as ho
+import hingetree_cpp as ops
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # B, C, Cout, size, D, Md, kernel, stride, padding, dilation
+    (2, 3, 4, [19], 3, [], [3], [2], [1], [1]),
+    (3, 4, 5, [12, 13], 4, [], [3, 3], [1, 1], [1, 1], [1, 1]),
+    (2, 2, 3, [17, 15], 2, [3], [3, 2], [2, 1], [2, 0], [2, 2]),
+    (1, 16, 8, [20, 20], 6, [], [3, 3], [1, 1], [1, 1], [1, 1]),       # the benchmark's tree shape, small image
+    (2, 2, 2, [6, 5, 7], 3, [2], [2, 2, 3], [1, 2, 1], [0, 1, 1], [1, 1, 1]),
+    (1, 2, 2, [40, 9], 3, [20], [3, 3], [1, 1], [0, 0], [1, 1]),       # more than 16 outputs per leaf
+    (1, 1, 2, [30, 30], 12, [], [5, 5], [1, 1], [2, 2], [1, 1]),       # deep trees: accumulators leave LDS
+]
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("case", CASES, ids=[f"c{i}" for i in range(len(CASES))])
+def test_conv_parity(dev, case, dtype, fern):
+    B, C, Cout, size, D, Md, ker, st, pad, dil = case
+    x, thr, ordn, w = make_conv(B, C, Cout, size, D, Md, ker, fern, dtype)
+    ref = ho.conv_forward(x, thr, ordn, w, ker, st, pad, dil, fern)
+    gout = torch.randn(ref.shape, generator=torch.Generator().manual_seed(4), dtype=dtype)
+    rdx, rdthr, rdw = ho.conv_backward(x, thr, ordn, w, gout, ker, st, pad, dil, fern=fern)
+    gx, gthr, gord, gw, gg = [t.to(dev) for t in (x, thr, ordn, w, gout)]
+    pre = ("fern_" if fern else "tree_") + f"conv{len(size)}d_"
+    out = getattr(ops, pre + "forward")(gx, gthr, gord, gw, ker, st, pad, dil)
+    assert out.shape == ref.shape and torch.equal(out.cpu(), ref)
+    dx, dthr, dord, dw = getattr(ops, pre + "backward")(gx, True, gthr, True, gord, False, gw, True, gg, ker, st, pad, dil)
+    assert dord is None
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    assert rel_err(dx.cpu(), rdx) <= tol and rel_err(dthr.cpu(), rdthr) <= tol and rel_err(dw.cpu(), rdw) <= tol
+    only = getattr(ops, pre + "backward")(gx, False, gthr, True, gord, False, gw, False, gg, ker, st, pad, dil)
+    assert only[0] is None and only[3] is None and rel_err(only[1].cpu(), rdthr) <= tol
+
+
+GOLD = sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "conv*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLD, ids=[os.path.basename(p)[:-4] for p in GOLD])
+def test_conv_golden(dev, path):
+    z = np.load(path)
+    fern = bool(z["fern"])
+    x, thr, ordn, w, gout = (torch.from_numpy(z[k]).to(dev) for k in ("x", "thr", "ord", "w", "gout"))
+    geo = [z[k].tolist() for k in ("kernel", "stride", "padding", "dilation")]
+    pre = ("fern_" if fern else "tree_") + f"conv{len(geo[0])}d_"
+    out = getattr(ops, pre + "forward")(x, thr, ordn, w, *geo)
+    assert torch.equal(out.cpu(), torch.from_numpy(z["out"]))
+    dx, dthr, _, dw = getattr(ops, pre + "backward")(x, True, thr, True, ordn, False, w, True, gout, *geo)
+    tol = 1e-5 if x.dtype == torch.float32 else 1e-12
+    for got, key in ((dx, "dx"), (dthr, "dthr"), (dw, "dw")):
+        assert rel_err(got.cpu(), torch.from_numpy(z[key])) <= tol

@@ -115,7 +115,8 @@ def test_degenerate_inputs(dev):
     thr[2, :] = float("inf")                  # always left  -> leaf 0
     ref_out = ho.forward(x, thr, ordn, w)
     ref_leaf, ref_margin, ref_sel, _ = ho.maps(x, thr, ordn, w)
-    assert (ref_leaf[:, 1] == 2 ** D - 1).all() and (ref_leaf[:, 2] == 0).all()
+    keep = torch.arange(16) != 1              # the NaN sample goes left wherever its NaN feature is tested
+    assert (ref_leaf[keep, 1] == 2 ** D - 1).all() and (ref_leaf[:, 2] == 0).all()
     gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
     out = ops.tree_forward(gx, gthr, gord, gw).cpu()
     same = (out == ref_out) | (out.isnan() & ref_out.isnan())

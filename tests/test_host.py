@@ -1,0 +1,173 @@
+"""CPU-side checks of the product: the C-ABI library loads and exports what include/hingetree_hip.h declares, the
+operator layer validates like the reference's dispatchers, the host-side threshold logic matches the oracle and the
+golden vector, and the modules are constructed like the reference's."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, make_forest
+from oracle import hinge_oracle as ho
+from hingetreefortorch_amd import _lib
+import hingetree_cpp as ops
+import HingeTree
+import RandomHingeForest as RHF
+
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def test_library_exports_header_symbols():
+    header = open(os.path.join(ROOT, "include", "hingetree_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ht_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert _lib.load().ht_abi_version() == 1
+
+
+def test_no_fallback_when_library_missing(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", os.path.join(ROOT, "no_such_dir", "libhingetree_hip.so"))
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.load()
+
+
+def test_validation_order_on_cpu_tensors():
+    x, thr, ordn, w, gout = make_forest(8, 5, [], 3, 2, [], False, torch.float32)
+    with pytest.raises(ValueError, match="share the same torch real number data type"):
+        ops.tree_forward(x.double(), thr, ordn, w)
+    with pytest.raises(ValueError, match="torch.int64"):
+        ops.fern_forward(x, thr, ordn.int(), w)
+    with pytest.raises(ValueError, match="contiguous"):
+        ops.tree_forward(x.t(), thr, ordn, w)
+    with pytest.raises(ValueError, match="Unsupported data type"):
+        ops.tree_forward(x.half(), thr.half(), ordn, w.half())
+    with pytest.raises(ValueError, match="at least 2 dimensions"):
+        ops.tree_forward(x[0], thr, ordn, w)
+    with pytest.raises(ValueError, match="same shape"):
+        ops.tree_forward(x, thr[:2], ordn, w)
+    with pytest.raises(RuntimeError, match=r"tree depth = 2"):
+        ops.tree_forward(x, thr[:, :2].contiguous(), ordn[:, :2].contiguous(), w)
+    with pytest.raises(RuntimeError, match=r"tree depth = -1"):
+        ops.tree_forward(x, thr, ordn, w[:, :3].contiguous())
+    with pytest.raises(RuntimeError, match="never has a gradient"):
+        ops.tree_backward(x, True, thr, True, ordn, True, w, True, gout)
+    with pytest.raises(ValueError, match="outDataGrad are expected"):
+        ops.tree_backward(x, True, thr, True, ordn, False, w, True, gout.double())
+    # everything valid but on the CPU: this build has no CPU back-end and says so instead of computing elsewhere
+    with pytest.raises(RuntimeError, match="no CPU back-end"):
+        ops.tree_forward(x, thr, ordn, w)
+    with pytest.raises(RuntimeError, match="not part of this build"):
+        ops.tree_fused_linear_forward(x, thr, ordn, w, w, w)
+
+
+def test_conv_validation_on_cpu_tensors():
+    x = torch.randn(2, 3, 8, 8)
+    thr, ordn, w = torch.randn(4, 3, 7), torch.randint(0, 9, (4, 3, 7)), torch.randn(4, 3, 8)
+    with pytest.raises(ValueError, match="expected to have 2 dimensions"):
+        ops.tree_conv2d_forward(x, thr, ordn, w, [3], [1, 1], [0, 0], [1, 1])
+    with pytest.raises(ValueError, match="inData expected to have 4 dimensions"):
+        ops.tree_conv2d_forward(x[0], thr, ordn, w, [3, 3], [1, 1], [0, 0], [1, 1])
+    with pytest.raises(ValueError, match="expected to divide inData"):
+        ops.tree_conv2d_forward(x, thr[:, :2].contiguous(), ordn[:, :2].contiguous(), w[:, :2].contiguous(), [3, 3],
+                                [1, 1], [0, 0], [1, 1])
+    with pytest.raises(RuntimeError, match="Unable to convert image patches"):
+        ops.tree_conv2d_forward(x, thr, ordn, w, [9, 9], [1, 1], [0, 0], [1, 1])
+    with pytest.raises(RuntimeError, match="Unable to convert image patches"):
+        ops.tree_conv2d_forward(x, thr, ordn, w, [3, 3], [0, 1], [0, 0], [1, 1])
+    with pytest.raises(RuntimeError, match="no CPU back-end"):
+        ops.tree_conv2d_forward(x, thr, ordn, w, [3, 3], [1, 1], [0, 0], [1, 1])
+
+
+def test_conv_output_size_matches_torch():
+    lib = _lib.load()
+    for size, k, s, p, d in [([17, 9], [3, 2], [2, 1], [1, 0], [1, 3]), ([128, 128], [3, 3], [1, 1], [1, 1], [1, 1]),
+                             ([5, 6, 7], [2, 3, 2], [1, 2, 3], [0, 1, 2], [2, 1, 1])]:
+        shape = _lib.ConvShape()
+        shape.B, shape.C, shape.Cout, shape.depth, shape.M, shape.nd = 1, 1, 1, 2, 1, len(size)
+        for i in range(len(size)):
+            shape.size[i], shape.kernel[i], shape.stride[i], shape.padding[i], shape.dilation[i] = \
+                size[i], k[i], s[i], p[i], d[i]
+        out = (ctypes.c_int64 * 3)()
+        assert lib.ht_conv_output_size(ctypes.byref(shape), out) == 0
+        conv = {2: torch.nn.functional.conv2d, 3: torch.nn.functional.conv3d}[len(size)]
+        expect = conv(torch.zeros([1, 1] + size), torch.zeros([1, 1] + k), stride=s, padding=p, dilation=d).shape[2:]
+        assert list(out)[:len(size)] == list(expect)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_thresholds_match_oracle_and_golden(dtype):
+    z = np.load(os.path.join(GOLDEN, "fix_thresholds.npz"))
+    thr = torch.from_numpy(z["before"]).clone()
+    ordn, w = torch.from_numpy(z["ord"]), torch.from_numpy(z["w"])
+    assert ops.tree_check_thresholds(thr, ordn, w) == z["ok_before"].tolist()
+    assert ops.tree_fix_thresholds(thr, ordn, w) == z["changed"].tolist()
+    assert torch.equal(thr, torch.from_numpy(z["after"]))
+    assert ops.tree_check_thresholds(thr, ordn, w) == z["ok_after"].tolist()
+    g = torch.Generator().manual_seed(5)
+    thr = (6 * torch.rand([40, 127], generator=g) - 3).to(dtype)
+    ordn = torch.randint(0, 5, [40, 127], generator=g)
+    w = torch.zeros(40, 128, dtype=dtype)
+    a, b = thr.clone(), thr.clone()
+    assert ops.tree_check_thresholds(a, ordn, w) == ho.check_thresholds(b, ordn, w)
+    assert ops.tree_fix_thresholds(a, ordn, w) == ho.fix_thresholds(b, ordn, w)
+    assert torch.equal(a, b) and all(ops.tree_check_thresholds(a, ordn, w))
+    fthr, ford = thr[:, :7].contiguous(), ordn[:, :7].contiguous()
+    keep = fthr.clone()
+    assert ops.fern_check_thresholds(fthr, ford, w) == [True] * 40
+    assert ops.fern_fix_thresholds(fthr, ford, w) == [False] * 40 and torch.equal(fthr, keep)
+    with pytest.raises(ValueError, match="on the CPU"):
+        ops.tree_fix_thresholds(thr.to("meta"), ordn.to("meta"), w.to("meta"))
+
+
+def test_module_construction_follows_reference_draw_order():
+    torch.manual_seed(1234)
+    m = RHF.RandomHingeForest(20, 6, 4, extra_outputs=3)
+    torch.manual_seed(1234)
+    thr = 6.0 * torch.rand([6, 15]) - 3.0
+    ordn = torch.randint_like(thr, low=0, high=20, dtype=torch.long)
+    w = torch.randn([6, 16, 3])
+    ho.fix_thresholds(thr, ordn, w)
+    assert torch.equal(m.thresholds.data, thr) and torch.equal(m.ordinals.data, ordn) and torch.equal(m.weights.data, w)
+    assert m.ordinals.dtype == torch.int64 and not m.ordinals.requires_grad
+    assert m.thresholds.requires_grad and m.weights.requires_grad
+    assert all(m.check_thresholds())
+
+    assert RHF.RandomHingeForest(5, 3, 2).weights.shape == (3, 4)
+    assert RHF.RandomHingeForest(5, 3, 2, extra_outputs=1).weights.shape == (3, 4, 1)
+    assert RHF.RandomHingeForest(5, 3, 2, extra_outputs=[8, 8]).weights.shape == (3, 4, 8, 8)
+    assert RHF.RandomHingeFern(5, 3, 6).thresholds.shape == (3, 6)
+    seq = RHF.RandomHingeForest(10, 3, 3, init_type="sequential")
+    assert torch.equal(seq.ordinals.data.view(-1), torch.arange(21) % 10)
+    with pytest.raises(RuntimeError, match="Unknown init_type"):
+        RHF.RandomHingeForest(5, 3, 2, init_type="nope")
+    c = RHF.HingeTreeConv2d(3, 4, 2, 3, padding=1)
+    assert c.thresholds.shape == (4, 3, 3) and c.weights.shape == (4, 3, 4) and int(c.ordinals.max()) < 9
+    assert RHF.HingeTreeConv2d(3, 4, 2, (3, 2), extra_outputs=5).weights.shape == (4, 3, 4, 5)
+    assert RHF.HingeFernConv3d(2, 2, 4, 2).thresholds.shape == (2, 2, 4)   # the reference's constructor raises here
+    assert RHF.HingeTreeConv1d(2, 2, 3, 5).kernel_size == (5,)
+
+
+def test_state_dict_with_float_ordinals():
+    m = RHF.RandomHingeForest(9, 4, 3)
+    state = {k: v.clone() for k, v in m.state_dict().items()}
+    state["ordinals"] = state["ordinals"].float()    # old snapshots of the reference stored ordinals as floats
+    n = RHF.RandomHingeForest(9, 4, 3)
+    n.load_state_dict(state)
+    assert n.ordinals.dtype == torch.int64 and torch.equal(n.ordinals.data, m.ordinals.data)
+    assert torch.equal(n.thresholds.data, m.thresholds.data)
+
+
+def test_public_names():
+    for name in ["HingeTree", "HingeFern", "HingeTreeConv1d", "HingeTreeConv2d", "HingeTreeConv3d", "HingeFernConv1d",
+                 "HingeFernConv2d", "HingeFernConv3d"]:
+        assert issubclass(getattr(HingeTree, name), torch.autograd.Function)
+    for name in ["tree_forward", "tree_backward", "tree_backward_deterministic", "fern_forward", "fern_backward",
+                 "fern_backward_deterministic", "tree_conv2d_forward", "tree_conv2d_backward", "tree_leafmap",
+                 "tree_marginmap", "tree_reachability", "tree_speedtest", "tree_fix_thresholds", "fern_conv3d_backward"]:
+        assert callable(getattr(ops, name))
