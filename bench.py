@@ -1,0 +1,171 @@
+#!/usr/bin/env python3
+"""Headline benchmark: RandomHingeForest fp32 forward+backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c1] [--mode atomic|deterministic]
+
+One step = one forward (tree_forward) plus one backward (tree_backward, all three gradients requested, atomic mode)
+over one batch of synthetic input that is already resident in HBM, called through the C ABI on torch's current stream.
+The default workload is the configuration the metric is quoted on: x ~ N(0,1) [65536, 1024], 1000 trees, depth 10,
+extra_outputs = 10 (out [65536, 1000, 10]); thresholds ~ U(-3,3) made consistent like the module constructor does,
+ordinals ~ U{0..1023}, leaf weights ~ N(0,1), upstream gradient ~ N(0,1).
+
+Prints ONE JSON line. `value` is samples/s over the timed steps (wall clock between device synchronisations);
+`roofline` prices the dominant pass (backward) against the 8 TB/s HBM peak using the algorithmic bytes of that pass
+(every input read once, every output written once) and its duration measured with events on the launch stream;
+`cpu_baseline` is the single-threaded CPU oracle timed on a bounded slice of the same workload on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: (B, F, T, depth, M, kind, x distribution, description)
+    "c3": (65536, 1024, 1000, 10, 10, "tree", "normal",
+           "forest fp32 fwd+bwd, x~N(0,1) [65536,1024], T=1000, depth=10, extra_outputs=10"),
+    "c2": (65536, 1024, 1000, 10, 1, "fern", "normal",
+           "fern fp32 fwd+bwd, x~N(0,1) [65536,1024], T=1000, depth=10, extra_outputs=1"),
+    "c1": (100, 1000, 100, 7, 1, "tree", "uniform",
+           "forest fp32 fwd+bwd, x~U[0,1) [100,1000], T=100, depth=7, extra_outputs=1"),
+}
+
+
+def algorithmic_bytes(B, F, T, depth, M, kind):
+    """Compulsory traffic: every input read once, every output written once; ordinals at their int64 API width."""
+    V = depth if kind == "fern" else 2 ** depth - 1
+    L = 2 ** depth
+    x, thr, ordn, w, out = 4 * B * F, 4 * T * V, 8 * T * V, 4 * T * L * M, 4 * B * T * M
+    fwd = x + thr + ordn + w + out
+    bwd = x + thr + ordn + w + out + x + thr + w   # + gout read, dX, dThr, dW written
+    return fwd, bwd
+
+
+def make_inputs(torch, name, dev):
+    import hingetree_cpp as ops
+    B, F, T, depth, M, kind, dist, _ = WORKLOADS[name]
+    g = torch.Generator().manual_seed(6112)
+    V = depth if kind == "fern" else 2 ** depth - 1
+    thr = 6.0 * torch.rand([T, V], generator=g) - 3.0
+    ordn = torch.randint(0, F, [T, V], generator=g, dtype=torch.int64)
+    w = torch.randn([T, 2 ** depth, M], generator=g)
+    if kind == "tree":
+        ops.tree_fix_thresholds(thr, ordn, w)   # as the module constructor does (host side)
+    gg = torch.Generator(device=dev).manual_seed(6113)
+    if dist == "normal":
+        x = torch.randn([B, F], generator=gg, device=dev)
+    else:
+        x = torch.rand([B, F], generator=gg, device=dev)
+    gout = torch.randn([B, T, M], generator=gg, device=dev)
+    return x, thr.to(dev), ordn.to(dev), w.to(dev), gout
+
+
+def cpu_baseline(torch, name, x, thr, ordn, w, gout, budget_rows):
+    """Single-threaded CPU oracle (a port of the reference's CPU loops) on the first rows of the same batch."""
+    from oracle import hinge_oracle as ho
+    B, F, T, depth, M, kind, _, _ = WORKLOADS[name]
+    rows = min(B, budget_rows)
+    xs, gs = x[:rows].cpu().contiguous(), gout[:rows].cpu().contiguous()
+    tc, oc, wc = thr.cpu(), ordn.cpu(), w.cpu()
+    fern = kind == "fern"
+    ho.lib()
+    t0 = time.perf_counter()
+    ho.forward(xs, tc, oc, wc, fern)
+    t1 = time.perf_counter()
+    ho.backward(xs, tc, oc, wc, gs, fern=fern)
+    t2 = time.perf_counter()
+    return {"value": rows / (t2 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+            "sample": f"first {rows} of {B} rows of the same batch, all {T} trees; 1 forward + 1 backward "
+                      f"(3 gradients) = {t2 - t0:.2f} s (forward {t1 - t0:.2f} s), single thread",
+            "host_cores": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--mode", default="atomic", choices=["atomic", "deterministic"])
+    ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the batch timed on the CPU (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (the path needs no exchange between GPUs and nothing "
+                 "here shards it); use --gpus 1.")
+
+    import torch
+    import hingetree_cpp as ops
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP library is the only back-end.")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    name = args.workload
+    B, F, T, depth, M, kind, _, desc = WORKLOADS[name]
+    x, thr, ordn, w, gout = make_inputs(torch, name, dev)
+    fwd = ops.fern_forward if kind == "fern" else ops.tree_forward
+    if args.mode == "deterministic":
+        bwd = ops.fern_backward_deterministic if kind == "fern" else ops.tree_backward_deterministic
+    else:
+        bwd = ops.fern_backward if kind == "fern" else ops.tree_backward
+
+    def step():
+        out = fwd(x, thr, ordn, w)
+        grads = bwd(x, True, thr, True, ordn, False, w, True, gout)
+        return out, grads
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        ev[i][0].record()
+        out = fwd(x, thr, ordn, w)
+        ev[i][1].record()
+        grads = bwd(x, True, thr, True, ordn, False, w, True, gout)
+        ev[i][2].record()
+        del out, grads
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+
+    fwd_bytes, bwd_bytes = algorithmic_bytes(B, F, T, depth, M, kind)
+    achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    result = {
+        "metric": "fwd+bwd samples/s (forest B=65536,F=1024,T=1000,D=10) + % of HBM peak BW",
+        "value": B / (ms_per_step * 1e-3),
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{name}: {desc}", "backward_mode": args.mode, "B": B, "F": F, "T": T, "depth": depth,
+                   "extra_outputs": M},
+        "roofline": {"bound": "hbm", "kernel": f"{kind} backward ({args.mode})", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "algorithmic_bytes": bwd_bytes, "ms": bwd_ms},
+        "forward": {"ms": fwd_ms, "samples_per_s": B / (fwd_ms * 1e-3), "algorithmic_bytes": fwd_bytes,
+                    "hbm_frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "step_hbm_frac": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+    }
+    if args.cpu_rows > 0:
+        result["cpu_baseline"] = cpu_baseline(torch, name, x, thr, ordn, w, gout, args.cpu_rows)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
