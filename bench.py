@@ -92,7 +92,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--mode", default="atomic", choices=["atomic", "deterministic"])
-    ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the batch timed on the CPU (0 = skip)")
+    ap.add_argument("--cpu-rows", type=int, default=32768, help="rows of the batch timed on the CPU (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the path needs no exchange between GPUs and nothing "
