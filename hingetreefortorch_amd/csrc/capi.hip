@@ -21,7 +21,7 @@ int make_dims(const ht_forest_shape *s, ForestDims *d) {
     return fail(HT_ERR_INVALID_ARGUMENT,
                 "Error: Unsupported data type. Only torch.float32 and torch.float64 are supported.");
   if (s->kind != HT_TREE && s->kind != HT_FERN) return fail(HT_ERR_INVALID_ARGUMENT, "Error: unknown tree kind.");
-  if (s->depth < 0 || s->depth > 31)  // 32-bit leaf keys, HingeTreeCommon.h:51,138
+  if (s->depth < 1 || s->depth > 31)  // 32-bit leaf keys, HingeTreeCommon.h:51,138; a depth-0 walk reads no vertex
     return fail(HT_ERR_RUNTIME,
                 "Error: The tree depth exceeds compile-time constraints or the number of thresholds is incorrect for "
                 "the tree depth (tree depth = " + std::to_string((long long)s->depth) + ").");
@@ -107,10 +107,14 @@ int ht_ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, void *strea
   return ordinal_range(ord, n, minmax, static_cast<hipStream_t>(stream));
 }
 
-size_t ht_forest_forward_workspace(const ht_forest_shape *) { return 0; }
+size_t ht_forest_forward_workspace(const ht_forest_shape *s) {
+  ForestDims d;
+  if (make_dims(s, &d) != HT_OK) return 0;
+  return s->dtype == HT_F32 ? forest_forward_workspace<float>(d) : forest_forward_workspace<double>(d);
+}
 
 int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
-                      void *out, void *, size_t, void *stream) {
+                      void *out, void *workspace, size_t workspace_bytes, void *stream) {
   ForestDims d;
   int rc = make_dims(s, &d);
   if (rc != HT_OK) return rc;
@@ -119,15 +123,17 @@ int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, 
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool fern = s->kind == HT_FERN;
   if (s->dtype == HT_F32)
-    return forest_forward<float>(d, fern, (const float *)x, (const float *)thr, ord, (const float *)w, (float *)out, st);
+    return forest_forward<float>(d, fern, (const float *)x, (const float *)thr, ord, (const float *)w, (float *)out,
+                                 workspace, workspace_bytes, st);
   return forest_forward<double>(d, fern, (const double *)x, (const double *)thr, ord, (const double *)w, (double *)out,
-                                st);
+                                workspace, workspace_bytes, st);
 }
 
-size_t ht_forest_backward_workspace(const ht_forest_shape *s, int mode, int, int, int) {
+size_t ht_forest_backward_workspace(const ht_forest_shape *s, int mode, int need_dx, int need_dthr, int need_dw) {
   ForestDims d;
   if (make_dims(s, &d) != HT_OK) return 0;
-  return s->dtype == HT_F32 ? forest_backward_workspace<float>(d, mode) : forest_backward_workspace<double>(d, mode);
+  return s->dtype == HT_F32 ? forest_backward_workspace<float>(d, mode, need_dx != 0, need_dthr != 0, need_dw != 0)
+                            : forest_backward_workspace<double>(d, mode, need_dx != 0, need_dthr != 0, need_dw != 0);
 }
 
 int ht_forest_backward(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
@@ -151,10 +157,15 @@ int ht_forest_backward(const ht_forest_shape *s, const void *x, const void *thr,
                                  workspace_bytes, st);
 }
 
-size_t ht_forest_maps_workspace(const ht_forest_shape *) { return 0; }
+size_t ht_forest_maps_workspace(const ht_forest_shape *s) {
+  ForestDims d;
+  if (make_dims(s, &d) != HT_OK) return 0;
+  return s->dtype == HT_F32 ? forest_maps_workspace<float>(d) : forest_maps_workspace<double>(d);
+}
 
 int ht_forest_maps(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, int64_t *leafmap,
-                   void *margins, int64_t *ordinals, int64_t *reach, void *, size_t, void *stream) {
+                   void *margins, int64_t *ordinals, int64_t *reach, void *workspace, size_t workspace_bytes,
+                   void *stream) {
   ForestDims d;
   int rc = make_dims(s, &d);
   if (rc != HT_OK) return rc;
@@ -163,9 +174,9 @@ int ht_forest_maps(const ht_forest_shape *s, const void *x, const void *thr, con
   const bool fern = s->kind == HT_FERN;
   if (s->dtype == HT_F32)
     return forest_maps<float>(d, fern, (const float *)x, (const float *)thr, ord, leafmap, (float *)margins, ordinals,
-                              reach, st);
+                              reach, workspace, workspace_bytes, st);
   return forest_maps<double>(d, fern, (const double *)x, (const double *)thr, ord, leafmap, (double *)margins, ordinals,
-                             reach, st);
+                             reach, workspace, workspace_bytes, st);
 }
 
 static int check_conv(const ht_conv_shape *s) {

@@ -40,25 +40,55 @@ __host__ __device__ constexpr size_t align_up(size_t v, size_t a) { return (v + 
 constexpr int kWave = 64;
 constexpr int kLdsBytes = 160 * 1024;       // LDS per CU / per workgroup limit on gfx950
 constexpr int kForestThreads = 1024;        // workgroup size of the tile kernels
+constexpr int kNumCUs = 256;                // MI355X
+
+// n / d for n * d < 2^32 by multiply-high with ceil(2^32 / d) (d >= 1).
+struct FastDiv {
+  uint32_t inv;
+  uint32_t d;
+  FastDiv() : inv(0), d(1) {}
+  explicit FastDiv(int divisor) : inv(divisor <= 1 ? 0u : uint32_t(((1ull << 32) + divisor - 1) / divisor)), d(divisor) {}
+  __device__ __forceinline__ int div(int n) const { return d <= 1 ? n : int(__umulhi(uint32_t(n), inv)); }
+};
+
+// How a tile kernel spreads the trees over blockIdx.y: with few sample tiles the trees are split so that at least
+// ~2 workgroups per CU exist; `group` is the number of trees a workgroup handles per pass.
+static inline void split_trees(long long tiles, int T, int group, int *trees_per_block, int *grid_y) {
+  const int passes = (T + group - 1) / group;
+  const long long want = tiles >= 2 * kNumCUs ? 1 : (2 * kNumCUs + tiles - 1) / (tiles > 0 ? tiles : 1);
+  const int split = int(want < passes ? want : passes);
+  *trees_per_block = ((passes + split - 1) / (split > 0 ? split : 1)) * group;
+  *grid_y = (T + *trees_per_block - 1) / *trees_per_block;
+}
 
 // Validates a forest shape and derives ForestDims. Returns HT_OK or an error (message set).
 int make_dims(const ht_forest_shape *s, ForestDims *d);
 
 // ---- entry points implemented per translation unit -------------------------------------------------------------
+// Packed (threshold, ordinal) vertices: layout in walk.hpp (Node<Real>), T*V entries.
 template <typename Real>
-int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                   Real *out, hipStream_t stream);
+size_t packed_nodes_bytes(const ForestDims &d);
+template <typename Real>
+int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *dst, hipStream_t stream);
 
 template <typename Real>
-size_t forest_backward_workspace(const ForestDims &d, int mode);
+size_t forest_forward_workspace(const ForestDims &d);
+template <typename Real>
+int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
+                   Real *out, void *ws, size_t ws_bytes, hipStream_t stream);
+
+template <typename Real>
+size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw);
 template <typename Real>
 int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
                     const Real *gout, Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes,
                     hipStream_t stream);
 
 template <typename Real>
+size_t forest_maps_workspace(const ForestDims &d);
+template <typename Real>
 int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap,
-                Real *margins, int64_t *ordinals, int64_t *reach, hipStream_t stream);
+                Real *margins, int64_t *ordinals, int64_t *reach, void *ws, size_t ws_bytes, hipStream_t stream);
 
 template <typename Real>
 int conv_forward(const ht_conv_shape &s, const Real *x, const Real *thr, const int64_t *ord, const Real *w, Real *out,
@@ -70,7 +100,7 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
 int conv_output_size(const ht_conv_shape &s, int64_t *out_size);
 int ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, hipStream_t stream);
 
-// Fills n elements with zero through a kernel (safe to record into a HIP graph, unlike a memset node).
+// Fills `bytes` bytes with zero through a kernel (safe to record into a HIP graph, unlike a memset node).
 int zero_fill(void *p, size_t bytes, hipStream_t stream);
 
 }  // namespace ht

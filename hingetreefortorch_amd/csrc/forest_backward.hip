@@ -1,32 +1,289 @@
 // Forest / fern backward: dX, dThresholds, dWeights.
 //
-// Atomic mode: one fused kernel. Same sample tile as the forward; per pass every (sample, tree) pair is walked once,
-// the upstream gradient is read once with the thread index along its contiguous axis, dW is accumulated with one
-// atomic per element, and the per-pair scalar c = sum_m w[t,leaf,m] * g[b,t,k,m] is reduced in LDS before the two
-// scatter atomics (dX, dThr) are issued.
+// Global floating-point atomics are far too slow for the 10^8..10^9 updates of a large batch, so every gradient is
+// accumulated on chip and written once. The pass is a short pipeline over "walk records":
 //
-// Deterministic mode: the walk is done once by a tile kernel that writes (leaf, vertex, margin) records, then
-//   * dX is owner-computes: one thread per sample adds its trees in index order (the reference CPU order);
-//   * dThr / dW are owner-computes per tree: one wavefront per tree consumes its records in sample order and orders
-//     colliding updates inside each group of 64 samples by lane, so no result depends on scheduling.
+//   records   tile kernel (the forward's walk): per (tree, sample) the leaf key, the selected vertex, its ordinal and
+//             the signed margin, stored tree major.
+//   trees     tree-stationary: a workgroup owns a group of adjacent trees whose dW accumulators fill its LDS, streams
+//             all samples once (one thread per sample; the group's slice of the upstream gradient row is contiguous),
+//             adds |margin| * g into the LDS accumulators, and forms c = sign(margin) * sum_m w[t,leaf,m] * g[m],
+//             which it stores tree major. dW is written from LDS at the end (plain stores; atomics only if the
+//             samples had to be split over several workgroups).
+//   dthr      tree-stationary: per tree, -c is accumulated by selected vertex in LDS.
+//   dx        sample-stationary: a workgroup owns a tile of samples and a [features x tile] accumulator in LDS, adds
+//             each tree's c at the selected ordinal, and writes the tile of dX once.
+//
+// Deterministic mode reuses the records and replaces the three accumulating kernels by owner-computes kernels whose
+// order of additions is fixed (see below). Small problems, very deep trees and very wide inputs use a single fused
+// kernel with global atomics instead.
 #include "forest_tile.hpp"
 
 namespace ht {
 namespace {
 
+constexpr int kIlp = 2;
+
+// ---------------------------------------------------------------------------------------------------------------
+// walk records
+// ---------------------------------------------------------------------------------------------------------------
+// COMPACT (depth <= 16 and F <= 65536): key | vertex << 16 in one word, ordinal in 16 bits.
+template <typename Real, bool COMPACT>
+struct Records {
+  uint32_t *a;    // COMPACT: key | vertex << 16      else: key
+  uint32_t *b;    // COMPACT: unused                  else: vertex
+  void *ordinal;  // COMPACT: uint16_t[]              else: uint32_t[]
+  Real *margin;
+  Real *c;        // sign(margin) * sum_m w * g, filled by the tree kernel
+
+  __device__ __forceinline__ void put(long long at, uint32_t key, uint32_t vertex, uint32_t ord, Real m) const {
+    if (COMPACT) {
+      a[at] = key | (vertex << 16);
+      static_cast<uint16_t *>(ordinal)[at] = uint16_t(ord);
+    } else {
+      a[at] = key;
+      b[at] = vertex;
+      static_cast<uint32_t *>(ordinal)[at] = ord;
+    }
+    margin[at] = m;
+  }
+  __device__ __forceinline__ uint32_t key(long long at) const { return COMPACT ? (a[at] & 0xffffu) : a[at]; }
+  __device__ __forceinline__ uint32_t vertex(long long at) const { return COMPACT ? (a[at] >> 16) : b[at]; }
+  __device__ __forceinline__ uint32_t ord(long long at) const {
+    return COMPACT ? uint32_t(static_cast<const uint16_t *>(ordinal)[at]) : static_cast<const uint32_t *>(ordinal)[at];
+  }
+};
+
+static bool compact_ok(const ForestDims &d) { return d.depth <= 16 && d.F <= 65536; }
+
 template <typename Real>
-__device__ __forceinline__ void atomic_add(Real *p, Real v) {
-  atomicAdd(p, v);
+size_t records_bytes(const ForestDims &d) {
+  const size_t n = size_t(d.T) * size_t(d.S);
+  if (compact_ok(d)) return align_up(n * 4, 256) + align_up(n * 2, 256) + 2 * align_up(n * sizeof(Real), 256);
+  return 3 * align_up(n * 4, 256) + 2 * align_up(n * sizeof(Real), 256);
+}
+
+template <typename Real, bool COMPACT>
+Records<Real, COMPACT> carve_records(const ForestDims &d, void *ws) {
+  const size_t n = size_t(d.T) * size_t(d.S);
+  unsigned char *p = static_cast<unsigned char *>(ws);
+  Records<Real, COMPACT> r;
+  r.a = reinterpret_cast<uint32_t *>(p);
+  p += align_up(n * 4, 256);
+  r.b = nullptr;
+  if (!COMPACT) {
+    r.b = reinterpret_cast<uint32_t *>(p);
+    p += align_up(n * 4, 256);
+  }
+  r.ordinal = p;
+  p += align_up(n * (COMPACT ? 2 : 4), 256);
+  r.margin = reinterpret_cast<Real *>(p);
+  p += align_up(n * sizeof(Real), 256);
+  r.c = reinterpret_cast<Real *>(p);
+  return r;
+}
+
+template <typename Real, bool FERN, int BT, bool XLDS, bool COMPACT>
+__global__ __launch_bounds__(kForestThreads) void records_kernel(ForestDims d, const Real *__restrict__ x,
+                                                                 const Node<Real> *__restrict__ nodes,
+                                                                 Records<Real, COMPACT> rec, int trees_per_block) {
+  constexpr int NT = kForestThreads;
+  constexpr int TC = NT / BT;
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *xs = reinterpret_cast<Real *>(smem);
+  const long long s0 = (long long)blockIdx.x * BT;
+  if (XLDS) {
+    load_tile<Real, BT, NT>(xs, x, d, s0);
+    __syncthreads();
+  }
+  const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
+  const long long s = s0 + j;
+  if (s >= d.S) return;
+  const long long xbase = (s / d.K) * d.FK + (s % d.K);
+  const int t_begin = blockIdx.y * trees_per_block;
+  const int t_end = min(d.T, t_begin + trees_per_block);
+  for (int tb = t_begin + tt; tb < t_end; tb += TC * kIlp) {
+    const Node<Real> *nd[kIlp];
+    int t[kIlp];
+#pragma unroll
+    for (int i = 0; i < kIlp; ++i) {
+      t[i] = tb + i * TC;
+      nd[i] = nodes + (long long)min(t[i], t_end - 1) * d.V;
+    }
+    WalkResult<Real> r[kIlp];
+    if (XLDS)
+      walk_many<Real, FERN, kIlp>(d.depth, nd, [&](int, int f) { return xs[f * BT + j]; }, r);
+    else
+      walk_many<Real, FERN, kIlp>(d.depth, nd, [&](int, int f) { return x[xbase + (long long)f * d.K]; }, r);
+#pragma unroll
+    for (int i = 0; i < kIlp; ++i)
+      if (t[i] < t_end)
+        rec.put((long long)t[i] * d.S + s, r[i].key, r[i].vertex, uint32_t(nd[i][r[i].vertex].ord), r[i].margin);
+  }
+}
+
+template <typename Real, bool FERN, int BT, bool XLDS, bool COMPACT>
+int launch_records(const ForestDims &d, const Real *x, const Node<Real> *nodes, Records<Real, COMPACT> rec,
+                   hipStream_t stream) {
+  constexpr int TP = kForestThreads / BT * kIlp;
+  const size_t lds = XLDS ? size_t(d.F) * BT * sizeof(Real) : 0;
+  const long long tiles = (d.S + BT - 1) / BT;
+  int trees_per_block, gy;
+  split_trees(tiles, d.T, TP, &trees_per_block, &gy);
+  if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
+  auto kernel = records_kernel<Real, FERN, BT, XLDS, COMPACT>;
+  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   int(lds)));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, nodes, rec,
+                     trees_per_block);
+  HT_LAUNCH_CHECK("forest walk records");
+  return HT_OK;
+}
+
+template <typename Real, bool FERN, bool COMPACT>
+int dispatch_records(const ForestDims &d, const Real *x, const Node<Real> *nodes, Records<Real, COMPACT> rec,
+                     hipStream_t stream) {
+  switch (pick_tile<Real>(d.F, 1024)) {
+    case 64: return launch_records<Real, FERN, 64, true, COMPACT>(d, x, nodes, rec, stream);
+    case 32: return launch_records<Real, FERN, 32, true, COMPACT>(d, x, nodes, rec, stream);
+    case 16: return launch_records<Real, FERN, 16, true, COMPACT>(d, x, nodes, rec, stream);
+    case 8: return launch_records<Real, FERN, 8, true, COMPACT>(d, x, nodes, rec, stream);
+    default: return launch_records<Real, FERN, 64, false, COMPACT>(d, x, nodes, rec, stream);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// atomic mode
+// tree-stationary dW + c
+// ---------------------------------------------------------------------------------------------------------------
+// grid = (tree groups, sample parts). Workgroup (g, p) owns trees [g*TB, g*TB + TB) and samples of part p.
+// LDS: dW accumulators [TB][L][M] (if dw). VW = width of the vector loads of g and w (divides M).
+template <typename Real, int VW, bool COMPACT>
+__global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, const Real *__restrict__ w,
+                                                              const Real *__restrict__ gout,
+                                                              Records<Real, COMPACT> rec, Real *dw, int TB,
+                                                              long long part_size, bool need_c, bool dw_atomic) {
+  typedef Real Vec __attribute__((ext_vector_type(VW)));
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *acc = reinterpret_cast<Real *>(smem);
+  const int t0 = blockIdx.x * TB;
+  const int nt = min(TB, d.T - t0);
+  const long long LM = (long long)d.L * d.M;
+  if (dw) {
+    for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) acc[i] = Real(0);
+    __syncthreads();
+  }
+  const long long s_begin = (long long)blockIdx.y * part_size;
+  const long long s_end = min(d.S, s_begin + part_size);
+  for (long long s = s_begin + threadIdx.x; s < s_end; s += kForestThreads) {
+    const long long b = s / d.K, k = s % d.K;
+    for (int tl = 0; tl < nt; ++tl) {
+      const int t = t0 + tl;
+      const long long at = (long long)t * d.S + s;
+      const uint32_t key = rec.key(at);
+      const Real mg = rec.margin[at];
+      const Real a = ht_abs(mg);
+      const Real *gp = gout + ((b * d.T + t) * d.K + k) * d.M;
+      const Real *wl = w + ((long long)t * d.L + key) * d.M;
+      Real *cell = acc + (long long)tl * LM + (long long)key * d.M;
+      Real cs = Real(0);
+      for (int m = 0; m < d.M; m += VW) {
+        const Vec gv = *reinterpret_cast<const Vec *>(gp + m);
+        if (need_c) {
+          const Vec wv = *reinterpret_cast<const Vec *>(wl + m);
+#pragma unroll
+          for (int i = 0; i < VW; ++i) cs += wv[i] * gv[i];
+        }
+        if (dw) {
+#pragma unroll
+          for (int i = 0; i < VW; ++i) atomicAdd(cell + m + i, a * gv[i]);
+        }
+      }
+      if (need_c) rec.c[at] = ht_sign(mg) * cs;
+    }
+  }
+  if (dw) {
+    __syncthreads();
+    Real *dst = dw + (long long)t0 * LM;
+    if (dw_atomic) {
+      for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads)
+        if (acc[i] != Real(0)) atomicAdd(dst + i, acc[i]);
+    } else {
+      for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) dst[i] = acc[i];
+    }
+  }
+}
+
+// dThr[t, v] = sum over samples with selected vertex v of -c. One workgroup per tree (x sample parts).
+template <typename Real, bool COMPACT>
+__global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dthr,
+                                                   long long part_size, bool use_atomic) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *acc = reinterpret_cast<Real *>(smem);
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < d.V; i += 256) acc[i] = Real(0);
+  __syncthreads();
+  const long long s_begin = (long long)blockIdx.y * part_size;
+  const long long s_end = min(d.S, s_begin + part_size);
+  for (long long s = s_begin + threadIdx.x; s < s_end; s += 256) {
+    const long long at = (long long)t * d.S + s;
+    atomicAdd(acc + rec.vertex(at), -rec.c[at]);
+  }
+  __syncthreads();
+  Real *dst = dthr + (long long)t * d.V;
+  for (int i = threadIdx.x; i < d.V; i += 256) {
+    if (use_atomic) {
+      if (acc[i] != Real(0)) atomicAdd(dst + i, acc[i]);
+    } else {
+      dst[i] = acc[i];
+    }
+  }
+}
+
+// dX: sample tile x all trees. LDS accumulator [F][BT+1] (the pad keeps the transposing write-out conflict free).
+template <typename Real, int BT, bool COMPACT>
+__global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dx) {
+  constexpr int NT = kForestThreads;
+  constexpr int TC = NT / BT;
+  constexpr int LD = BT + 1;
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *acc = reinterpret_cast<Real *>(smem);
+  for (int i = threadIdx.x; i < d.F * LD; i += NT) acc[i] = Real(0);
+  __syncthreads();
+  const long long s0 = (long long)blockIdx.x * BT;
+  const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
+  const long long s = s0 + j;
+  if (s < d.S) {
+    for (int t = tt; t < d.T; t += TC) {
+      const long long at = (long long)t * d.S + s;
+      atomicAdd(acc + rec.ord(at) * LD + j, rec.c[at]);
+    }
+  }
+  __syncthreads();
+  if (d.K == 1) {
+    // dx[s, 0..F) is a contiguous row: a wavefront per sample, lanes along the features
+    const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+    for (int jj = wv; jj < BT && s0 + jj < d.S; jj += NT / kWave) {
+      Real *row = dx + (s0 + jj) * d.F;
+      for (int f = lane; f < d.F; f += kWave) row[f] = acc[f * LD + jj];
+    }
+  } else {
+    // dx[b, f, k]: consecutive samples of a tile are consecutive k (within one b)
+    for (int i = threadIdx.x; i < d.F * BT; i += NT) {
+      const int f = i / BT, jj = i - f * BT;
+      const long long ss = s0 + jj;
+      if (ss < d.S) dx[(ss / d.K) * d.FK + (long long)f * d.K + (ss % d.K)] = acc[f * LD + jj];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// fused kernel with global atomics (small problems, depth > 16, F > 65536, huge leaf tables)
 // ---------------------------------------------------------------------------------------------------------------
 template <typename Real, bool FERN, int BT, bool XLDS>
-__global__ __launch_bounds__(kForestThreads) void backward_atomic_kernel(
-    ForestDims d, const Real *__restrict__ x, const Real *__restrict__ thr, const int64_t *__restrict__ ord,
-    const Real *__restrict__ w, const Real *__restrict__ gout, Real *__restrict__ dx, Real *__restrict__ dthr,
-    Real *__restrict__ dw, int trees_per_block) {
+__global__ __launch_bounds__(kForestThreads) void backward_fused_kernel(
+    ForestDims d, const Real *__restrict__ x, const Node<Real> *__restrict__ nodes, const Real *__restrict__ w,
+    const Real *__restrict__ gout, Real *__restrict__ dx, Real *__restrict__ dthr, Real *__restrict__ dw,
+    int trees_per_block, FastDiv div_m) {
   constexpr int NT = kForestThreads;
   constexpr int TC = NT / BT;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -53,17 +310,15 @@ __global__ __launch_bounds__(kForestThreads) void backward_atomic_kernel(
     const int t = tb + tt;
     const bool mine = t < t_end && live;
     if (mine) {
-      const Real *th = thr + (long long)t * d.V;
-      const int64_t *od = ord + (long long)t * d.V;
-      auto node = [&](uint32_t at, Real &tv, int &ov) { tv = th[at]; ov = clamp_ordinal(od[at], d.F); };
-      WalkResult<Real> r;
+      const Node<Real> *nd[1] = {nodes + (long long)t * d.V};
+      WalkResult<Real> r[1];
       if (XLDS)
-        r = walk<Real, FERN>(d.depth, node, [&](int f) { return xs[f * BT + j]; });
+        walk_many<Real, FERN, 1>(d.depth, nd, [&](int, int f) { return xs[f * BT + j]; }, r);
       else
-        r = walk<Real, FERN>(d.depth, node, [&](int f) { return x[xbase + (long long)f * d.K]; });
-      r_margin[tt * BT + j] = r.margin;
-      r_key[tt * BT + j] = r.key;
-      r_vertex[tt * BT + j] = r.vertex;
+        walk_many<Real, FERN, 1>(d.depth, nd, [&](int, int f) { return x[xbase + (long long)f * d.K]; }, r);
+      r_margin[tt * BT + j] = r[0].margin;
+      r_key[tt * BT + j] = r[0].key;
+      r_vertex[tt * BT + j] = r[0].vertex;
     }
     r_csum[tt * BT + j] = Real(0);
     __syncthreads();
@@ -75,15 +330,15 @@ __global__ __launch_bounds__(kForestThreads) void backward_atomic_kernel(
       const int total = k1 ? BT * row : nt * row;
       for (int idx = threadIdx.x; idx < total; idx += NT) {
         const int hi = idx / row, r = idx - hi * row;
-        const int lo = r / d.M, m = r - lo * d.M;
+        const int lo = div_m.div(r), m = r - lo * d.M;
         const int jj = k1 ? hi : lo, t2 = k1 ? lo : hi;
         const long long ss = s0 + jj;
         if (ss < d.S) {
           const Real g = gout[out_offset(d, ss, tb + t2, m)];
           const uint32_t key = r_key[t2 * BT + jj];
           const long long wi = ((long long)(tb + t2) * d.L + key) * d.M + m;
-          if (dw) atomic_add(dw + wi, ht_abs(r_margin[t2 * BT + jj]) * g);
-          if (need_c) atomic_add(r_csum + t2 * BT + jj, w[wi] * g);
+          if (dw) atomicAdd(dw + wi, ht_abs(r_margin[t2 * BT + jj]) * g);
+          if (need_c) atomicAdd(r_csum + t2 * BT + jj, w[wi] * g);
         }
       }
     }
@@ -92,163 +347,64 @@ __global__ __launch_bounds__(kForestThreads) void backward_atomic_kernel(
     if (mine && need_c) {
       const Real c = ht_sign(r_margin[tt * BT + j]) * r_csum[tt * BT + j];
       const uint32_t v = r_vertex[tt * BT + j];
-      const long long o = clamp_ordinal(ord[(long long)t * d.V + v], d.F);
-      if (dx) atomic_add(dx + xbase + o * d.K, c);
-      if (dthr) atomic_add(dthr + (long long)t * d.V + v, -c);
+      const long long o = nodes[(long long)t * d.V + v].ord;
+      if (dx) atomicAdd(dx + xbase + o * d.K, c);
+      if (dthr) atomicAdd(dthr + (long long)t * d.V + v, -c);
     }
     __syncthreads();
   }
 }
 
 template <typename Real, bool FERN, int BT, bool XLDS>
-int launch_backward_atomic(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                           const Real *gout, Real *dx, Real *dthr, Real *dw, hipStream_t stream) {
+int launch_backward_fused(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, const Real *gout,
+                          Real *dx, Real *dthr, Real *dw, hipStream_t stream) {
   constexpr int TC = kForestThreads / BT;
   const size_t lds =
       (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TC) * BT * (2 * sizeof(Real) + 2 * sizeof(uint32_t));
   const long long tiles = (d.S + BT - 1) / BT;
-  const int passes = (d.T + TC - 1) / TC;
-  long long want = tiles >= 512 ? 1 : (512 + tiles - 1) / tiles;
-  const int split = int(want < passes ? want : passes);
-  const int trees_per_block = ((passes + split - 1) / split) * TC;
-  const int gy = (d.T + trees_per_block - 1) / trees_per_block;
+  int trees_per_block, gy;
+  split_trees(tiles, d.T, TC, &trees_per_block, &gy);
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
-  auto kernel = backward_atomic_kernel<Real, FERN, BT, XLDS>;
+  auto kernel = backward_fused_kernel<Real, FERN, BT, XLDS>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, thr, ord, w,
-                     gout, dx, dthr, dw, trees_per_block);
-  HT_LAUNCH_CHECK("forest backward (atomic)");
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, nodes, w, gout,
+                     dx, dthr, dw, trees_per_block, FastDiv(d.M));
+  HT_LAUNCH_CHECK("forest backward (fused, atomics)");
   return HT_OK;
 }
 
 template <typename Real, bool FERN>
-int dispatch_backward_atomic(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                             const Real *gout, Real *dx, Real *dthr, Real *dw, hipStream_t stream) {
+int dispatch_backward_fused(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w,
+                            const Real *gout, Real *dx, Real *dthr, Real *dw, hipStream_t stream) {
   const size_t reserve = 32 * 1024;
   switch (pick_tile<Real>(d.F, reserve)) {
-    case 64: return launch_backward_atomic<Real, FERN, 64, true>(d, x, thr, ord, w, gout, dx, dthr, dw, stream);
-    case 32: return launch_backward_atomic<Real, FERN, 32, true>(d, x, thr, ord, w, gout, dx, dthr, dw, stream);
-    case 16: return launch_backward_atomic<Real, FERN, 16, true>(d, x, thr, ord, w, gout, dx, dthr, dw, stream);
-    case 8: return launch_backward_atomic<Real, FERN, 8, true>(d, x, thr, ord, w, gout, dx, dthr, dw, stream);
-    default: return launch_backward_atomic<Real, FERN, 64, false>(d, x, thr, ord, w, gout, dx, dthr, dw, stream);
+    case 64: return launch_backward_fused<Real, FERN, 64, true>(d, x, nodes, w, gout, dx, dthr, dw, stream);
+    case 32: return launch_backward_fused<Real, FERN, 32, true>(d, x, nodes, w, gout, dx, dthr, dw, stream);
+    case 16: return launch_backward_fused<Real, FERN, 16, true>(d, x, nodes, w, gout, dx, dthr, dw, stream);
+    case 8: return launch_backward_fused<Real, FERN, 8, true>(d, x, nodes, w, gout, dx, dthr, dw, stream);
+    default: return launch_backward_fused<Real, FERN, 64, false>(d, x, nodes, w, gout, dx, dthr, dw, stream);
   }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// deterministic mode
+// deterministic owner-computes kernels (consume the records)
 // ---------------------------------------------------------------------------------------------------------------
-// Walk records, tree major: rec[t * S + s].
-template <typename Real>
-struct Records {
-  uint32_t *key;
-  uint32_t *vertex;
-  Real *margin;
-};
-
-template <typename Real>
-size_t records_bytes(const ForestDims &d) {
-  const size_t n = size_t(d.T) * size_t(d.S);
-  return align_up(n * sizeof(uint32_t), 256) * 2 + align_up(n * sizeof(Real), 256);
-}
-
-template <typename Real>
-Records<Real> carve_records(const ForestDims &d, void *ws) {
-  const size_t n = size_t(d.T) * size_t(d.S);
-  unsigned char *p = static_cast<unsigned char *>(ws);
-  Records<Real> r;
-  r.key = reinterpret_cast<uint32_t *>(p);
-  p += align_up(n * sizeof(uint32_t), 256);
-  r.vertex = reinterpret_cast<uint32_t *>(p);
-  p += align_up(n * sizeof(uint32_t), 256);
-  r.margin = reinterpret_cast<Real *>(p);
-  return r;
-}
-
-template <typename Real, bool FERN, int BT, bool XLDS>
-__global__ __launch_bounds__(kForestThreads) void records_kernel(ForestDims d, const Real *__restrict__ x,
-                                                                 const Real *__restrict__ thr,
-                                                                 const int64_t *__restrict__ ord, Records<Real> rec,
-                                                                 int trees_per_block) {
-  constexpr int NT = kForestThreads;
-  constexpr int TC = NT / BT;
-  extern __shared__ __align__(16) unsigned char smem[];
-  Real *xs = reinterpret_cast<Real *>(smem);
-  const long long s0 = (long long)blockIdx.x * BT;
-  if (XLDS) {
-    load_tile<Real, BT, NT>(xs, x, d, s0);
-    __syncthreads();
-  }
-  const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
-  const long long s = s0 + j;
-  if (s >= d.S) return;
-  const long long xbase = (s / d.K) * d.FK + (s % d.K);
-  const int t_begin = blockIdx.y * trees_per_block;
-  const int t_end = min(d.T, t_begin + trees_per_block);
-  for (int t = t_begin + tt; t < t_end; t += TC) {
-    const Real *th = thr + (long long)t * d.V;
-    const int64_t *od = ord + (long long)t * d.V;
-    auto node = [&](uint32_t at, Real &tv, int &ov) { tv = th[at]; ov = clamp_ordinal(od[at], d.F); };
-    WalkResult<Real> r;
-    if (XLDS)
-      r = walk<Real, FERN>(d.depth, node, [&](int f) { return xs[f * BT + j]; });
-    else
-      r = walk<Real, FERN>(d.depth, node, [&](int f) { return x[xbase + (long long)f * d.K]; });
-    const long long at = (long long)t * d.S + s;
-    rec.key[at] = r.key;
-    rec.vertex[at] = r.vertex;
-    rec.margin[at] = r.margin;
-  }
-}
-
-template <typename Real, bool FERN, int BT, bool XLDS>
-int launch_records(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, Records<Real> rec,
-                   hipStream_t stream) {
-  constexpr int TC = kForestThreads / BT;
-  const size_t lds = XLDS ? size_t(d.F) * BT * sizeof(Real) : 0;
-  const long long tiles = (d.S + BT - 1) / BT;
-  const int passes = (d.T + TC - 1) / TC;
-  long long want = tiles >= 512 ? 1 : (512 + tiles - 1) / tiles;
-  const int split = int(want < passes ? want : passes);
-  const int trees_per_block = ((passes + split - 1) / split) * TC;
-  const int gy = (d.T + trees_per_block - 1) / trees_per_block;
-  if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
-  auto kernel = records_kernel<Real, FERN, BT, XLDS>;
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   int(lds)));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, thr, ord,
-                     rec, trees_per_block);
-  HT_LAUNCH_CHECK("forest walk records");
-  return HT_OK;
-}
-
-template <typename Real, bool FERN>
-int dispatch_records(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, Records<Real> rec,
-                     hipStream_t stream) {
-  switch (pick_tile<Real>(d.F, 1024)) {
-    case 64: return launch_records<Real, FERN, 64, true>(d, x, thr, ord, rec, stream);
-    case 32: return launch_records<Real, FERN, 32, true>(d, x, thr, ord, rec, stream);
-    case 16: return launch_records<Real, FERN, 16, true>(d, x, thr, ord, rec, stream);
-    case 8: return launch_records<Real, FERN, 8, true>(d, x, thr, ord, rec, stream);
-    default: return launch_records<Real, FERN, 64, false>(d, x, thr, ord, rec, stream);
-  }
-}
-
 // dX: thread per sample, trees in index order, one add per (tree, m) term straight into the owned cell: the same
 // sequence of roundings as the reference CPU loop (hingetree.cpp:236-254).
-template <typename Real>
-__global__ __launch_bounds__(256) void det_dx_kernel(ForestDims d, const int64_t *__restrict__ ord,
-                                                     const Real *__restrict__ w, const Real *__restrict__ gout,
-                                                     Records<Real> rec, Real *dx) {
+template <typename Real, bool COMPACT>
+__global__ __launch_bounds__(256) void det_dx_kernel(ForestDims d, const Real *__restrict__ w,
+                                                     const Real *__restrict__ gout, Records<Real, COMPACT> rec,
+                                                     Real *dx) {
   const long long s = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (s >= d.S) return;
   const long long b = s / d.K, k = s % d.K;
   const long long xbase = b * d.FK + k;
   for (int t = 0; t < d.T; ++t) {
     const long long at = (long long)t * d.S + s;
-    const uint32_t key = rec.key[at];
+    const uint32_t key = rec.key(at);
     const Real sg = ht_sign(rec.margin[at]);
-    const long long o = clamp_ordinal(ord[(long long)t * d.V + rec.vertex[at]], d.F);
+    const long long o = rec.ord(at);
     const Real *wl = w + ((long long)t * d.L + key) * d.M;
     const Real *g = gout + ((b * d.T + t) * d.K + k) * d.M;
     Real *cell = dx + xbase + o * d.K;
@@ -282,10 +438,10 @@ __device__ __forceinline__ void ordered_add(Real *p, Real v) {
 //         its terms in ascending sample order (the reference CPU order, hingetree.cpp:290-305).
 //   dThr: for each distinct vertex in the group the member lanes' terms are summed by a fixed butterfly and the
 //         leader lane adds the group sum to the vertex' accumulator.
-template <typename Real, bool LDS_ACC>
+template <typename Real, bool LDS_ACC, bool COMPACT>
 __global__ __launch_bounds__(kWave) void det_tree_kernel(ForestDims d, const Real *__restrict__ w,
-                                                         const Real *__restrict__ gout, Records<Real> rec, Real *dthr,
-                                                         Real *dw) {
+                                                         const Real *__restrict__ gout, Records<Real, COMPACT> rec,
+                                                         Real *dthr, Real *dw) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int t = blockIdx.x;
   const int lane = threadIdx.x;
@@ -311,8 +467,8 @@ __global__ __launch_bounds__(kWave) void det_tree_kernel(ForestDims d, const Rea
     Real mg = Real(0);
     if (live) {
       const long long at = (long long)t * d.S + s;
-      key = rec.key[at];
-      v = rec.vertex[at];
+      key = rec.key(at);
+      v = rec.vertex(at);
       mg = rec.margin[at];
     }
     const long long goff = live ? out_offset(d, s, t, 0) : 0;
@@ -366,30 +522,152 @@ __global__ __launch_bounds__(kWave) void det_tree_kernel(ForestDims d, const Rea
   }
 }
 
-template <typename Real, bool FERN>
-int backward_deterministic(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                           const Real *gout, Real *dx, Real *dthr, Real *dw, void *ws, size_t ws_bytes,
-                           hipStream_t stream) {
-  if (ws_bytes < records_bytes<Real>(d) || ws == nullptr)
-    return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the deterministic backward pass.");
-  Records<Real> rec = carve_records<Real>(d, ws);
-  int rc = dispatch_records<Real, FERN>(d, x, thr, ord, rec, stream);
+// ---------------------------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------------------------
+struct TreePlan {
+  int TB;               // trees per workgroup
+  int groups, parts;    // grid
+  long long part_size;  // samples per part
+  size_t lds;
+  int vw;               // vector width of the g / w loads
+};
+
+template <typename Real>
+bool plan_trees(const ForestDims &d, bool need_dw, const Real *w, const Real *gout, TreePlan *p) {
+  const size_t per_tree = size_t(d.L) * d.M * sizeof(Real);
+  int tb = 4;
+  if (need_dw) {
+    if (per_tree > size_t(kLdsBytes)) return false;
+    tb = int(size_t(kLdsBytes) / per_tree);
+  }
+  if (tb > d.T) tb = d.T;
+  // keep at least ~one workgroup per CU by shrinking the groups before splitting the samples
+  while (tb > 4 && (d.T + tb - 1) / tb < kNumCUs) tb = (tb + 1) / 2;
+  p->TB = tb;
+  p->groups = (d.T + tb - 1) / tb;
+  long long parts = 1;
+  if (p->groups < kNumCUs) parts = (kNumCUs + p->groups - 1) / p->groups;
+  const long long max_parts = (d.S + 4 * kForestThreads - 1) / (4 * kForestThreads);  // >= 4 samples per thread
+  if (parts > max_parts) parts = max_parts;
+  if (parts < 1) parts = 1;
+  if (parts > 65535) parts = 65535;
+  p->part_size = (d.S + parts - 1) / parts;
+  p->parts = int((d.S + p->part_size - 1) / p->part_size);
+  p->lds = need_dw ? size_t(tb) * per_tree : 0;
+  const size_t vbytes2 = 2 * sizeof(Real), vbytes4 = 4 * sizeof(Real);
+  const uintptr_t pw = reinterpret_cast<uintptr_t>(w), pg = reinterpret_cast<uintptr_t>(gout);
+  p->vw = 1;
+  if (d.M % 2 == 0 && pw % vbytes2 == 0 && pg % vbytes2 == 0) p->vw = 2;
+  if (d.M % 4 == 0 && pw % vbytes4 == 0 && pg % vbytes4 == 0) p->vw = 4;
+  return true;
+}
+
+template <typename Real, int VW, bool COMPACT>
+int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, const Real *gout,
+                       Records<Real, COMPACT> rec, Real *dw, bool need_c, hipStream_t stream) {
+  auto kernel = tree_kernel<Real, VW, COMPACT>;
+  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   int(p.lds)));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)p.groups, (unsigned)p.parts), dim3(kForestThreads), p.lds, stream, d, w,
+                     gout, rec, dw, p.TB, p.part_size, need_c, p.parts > 1);
+  HT_LAUNCH_CHECK("forest backward (trees)");
+  return HT_OK;
+}
+
+template <typename Real, int BT, bool COMPACT>
+int launch_dx(const ForestDims &d, Records<Real, COMPACT> rec, Real *dx, hipStream_t stream) {
+  const size_t lds = size_t(d.F) * (BT + 1) * sizeof(Real);
+  const long long tiles = (d.S + BT - 1) / BT;
+  if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
+  auto kernel = dx_kernel<Real, BT, COMPACT>;
+  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   int(lds)));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kForestThreads), lds, stream, d, rec, dx);
+  HT_LAUNCH_CHECK("forest backward (dX)");
+  return HT_OK;
+}
+
+// Largest dX tile whose padded [F][BT+1] accumulator fits LDS; 0 if none.
+template <typename Real>
+int pick_dx_tile(int F) {
+  const int candidates[4] = {64, 32, 16, 8};
+  for (int bt : candidates)
+    if (size_t(F) * (bt + 1) * sizeof(Real) <= size_t(kLdsBytes)) return bt;
+  return 0;
+}
+
+template <typename Real>
+bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw) {
+  if (d.M < 1) return false;
+  if (need_dw && size_t(d.L) * d.M * sizeof(Real) > size_t(kLdsBytes)) return false;
+  if (size_t(d.V) * sizeof(Real) > size_t(kLdsBytes)) return false;
+  if (need_dx && pick_dx_tile<Real>(d.F) == 0) return false;
+  return true;
+}
+
+// Problems this small finish sooner in the single fused kernel than in four launches.
+static bool prefer_fused(const ForestDims &d) { return double(d.S) * double(d.T) < double(1 << 18); }
+
+template <typename Real, bool FERN, bool COMPACT>
+int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, const Real *gout,
+                    Real *dx, Real *dthr, Real *dw, void *rec_ws, hipStream_t stream) {
+  Records<Real, COMPACT> rec = carve_records<Real, COMPACT>(d, rec_ws);
+  int rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream);
+  if (rc != HT_OK) return rc;
+  const bool need_c = dx || dthr;
+  TreePlan plan;
+  if (!plan_trees<Real>(d, dw != nullptr, w, gout, &plan)) return fail(HT_ERR_RUNTIME, "Error: leaf table too large.");
+  switch (plan.vw) {
+    case 4: rc = launch_tree_kernel<Real, 4, COMPACT>(d, plan, w, gout, rec, dw, need_c, stream); break;
+    case 2: rc = launch_tree_kernel<Real, 2, COMPACT>(d, plan, w, gout, rec, dw, need_c, stream); break;
+    default: rc = launch_tree_kernel<Real, 1, COMPACT>(d, plan, w, gout, rec, dw, need_c, stream); break;
+  }
+  if (rc != HT_OK) return rc;
+  if (dthr) {
+    long long parts = d.T >= 2 * kNumCUs ? 1 : (2 * kNumCUs + d.T - 1) / d.T;
+    const long long max_parts = (d.S + 1023) / 1024;
+    if (parts > max_parts) parts = max_parts;
+    if (parts < 1) parts = 1;
+    if (parts > 65535) parts = 65535;
+    const long long part_size = (d.S + parts - 1) / parts;
+    const int gy = int((d.S + part_size - 1) / part_size);
+    hipLaunchKernelGGL((dthr_kernel<Real, COMPACT>), dim3((unsigned)d.T, (unsigned)gy), dim3(256),
+                       size_t(d.V) * sizeof(Real), stream, d, rec, dthr, part_size, gy > 1);
+    HT_LAUNCH_CHECK("forest backward (dThr)");
+  }
+  if (dx) {
+    switch (pick_dx_tile<Real>(d.F)) {
+      case 64: rc = launch_dx<Real, 64, COMPACT>(d, rec, dx, stream); break;
+      case 32: rc = launch_dx<Real, 32, COMPACT>(d, rec, dx, stream); break;
+      case 16: rc = launch_dx<Real, 16, COMPACT>(d, rec, dx, stream); break;
+      default: rc = launch_dx<Real, 8, COMPACT>(d, rec, dx, stream); break;
+    }
+  }
+  return rc;
+}
+
+template <typename Real, bool FERN, bool COMPACT>
+int backward_deterministic(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w,
+                           const Real *gout, Real *dx, Real *dthr, Real *dw, void *rec_ws, hipStream_t stream) {
+  Records<Real, COMPACT> rec = carve_records<Real, COMPACT>(d, rec_ws);
+  int rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream);
   if (rc != HT_OK) return rc;
   if (dx) {
     const long long blocks = (d.S + 255) / 256;
-    hipLaunchKernelGGL(det_dx_kernel<Real>, dim3((unsigned)blocks), dim3(256), 0, stream, d, ord, w, gout, rec, dx);
+    hipLaunchKernelGGL((det_dx_kernel<Real, COMPACT>), dim3((unsigned)blocks), dim3(256), 0, stream, d, w, gout, rec, dx);
     HT_LAUNCH_CHECK("deterministic dX");
   }
   if (dthr || dw) {
     const size_t need = (dw ? size_t(d.L) * d.M : 0) * sizeof(Real) + (dthr ? size_t(d.V) : 0) * sizeof(Real);
     if (need <= size_t(kLdsBytes) / 3) {
-      auto kernel = det_tree_kernel<Real, true>;
+      auto kernel = det_tree_kernel<Real, true, COMPACT>;
       HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, int(need)));
       hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, dthr, dw);
     } else {
-      hipLaunchKernelGGL((det_tree_kernel<Real, false>), dim3((unsigned)d.T), dim3(kWave), 0, stream, d, w, gout, rec,
-                         dthr, dw);
+      hipLaunchKernelGGL((det_tree_kernel<Real, false, COMPACT>), dim3((unsigned)d.T), dim3(kWave), 0, stream, d, w,
+                         gout, rec, dthr, dw);
     }
     HT_LAUNCH_CHECK("deterministic dThr/dW");
   }
@@ -399,8 +677,13 @@ int backward_deterministic(const ForestDims &d, const Real *x, const Real *thr, 
 }  // namespace
 
 template <typename Real>
-size_t forest_backward_workspace(const ForestDims &d, int mode) {
-  return mode == HT_BACKWARD_DETERMINISTIC ? records_bytes<Real>(d) : 0;
+size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw) {
+  size_t bytes = packed_nodes_bytes<Real>(d);
+  const bool staged = mode == HT_BACKWARD_DETERMINISTIC ||
+                      (staged_ok<Real>(d, need_dx, need_dw) && !prefer_fused(d));
+  (void)need_dthr;
+  if (staged) bytes += records_bytes<Real>(d);
+  return bytes;
 }
 
 template <typename Real>
@@ -408,19 +691,40 @@ int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *t
                     const Real *gout, Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes,
                     hipStream_t stream) {
   int rc;
-  if (dx && (rc = zero_fill(dx, size_t(d.S) * d.F * sizeof(Real), stream)) != HT_OK) return rc;
+  const bool det = mode == HT_BACKWARD_DETERMINISTIC;
+  const bool staged = det || (staged_ok<Real>(d, dx != nullptr, dw != nullptr) && !prefer_fused(d));
+  // The staged dX kernel overwrites every element of dX; everything else accumulates into zeros.
+  const bool empty = d.S == 0 || d.T == 0;
+  const bool clear_dx = !staged || det || empty;
+  if (dx && clear_dx && (rc = zero_fill(dx, size_t(d.S) * d.F * sizeof(Real), stream)) != HT_OK) return rc;
   if (dthr && (rc = zero_fill(dthr, size_t(d.T) * d.V * sizeof(Real), stream)) != HT_OK) return rc;
   if (dw && (rc = zero_fill(dw, size_t(d.T) * d.L * d.M * sizeof(Real), stream)) != HT_OK) return rc;
-  if (d.S == 0 || d.T == 0 || (!dx && !dthr && !dw)) return HT_OK;
-  if (mode == HT_BACKWARD_DETERMINISTIC)
-    return fern ? backward_deterministic<Real, true>(d, x, thr, ord, w, gout, dx, dthr, dw, ws, ws_bytes, stream)
-                : backward_deterministic<Real, false>(d, x, thr, ord, w, gout, dx, dthr, dw, ws, ws_bytes, stream);
-  return fern ? dispatch_backward_atomic<Real, true>(d, x, thr, ord, w, gout, dx, dthr, dw, stream)
-              : dispatch_backward_atomic<Real, false>(d, x, thr, ord, w, gout, dx, dthr, dw, stream);
+  if (empty || (!dx && !dthr && !dw)) return HT_OK;
+  const size_t node_bytes = packed_nodes_bytes<Real>(d);
+  const size_t need = node_bytes + (staged ? records_bytes<Real>(d) : 0);
+  if (ws == nullptr || ws_bytes < need)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the backward pass.");
+  if ((rc = pack_nodes<Real>(d, thr, ord, ws, stream)) != HT_OK) return rc;
+  const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
+  void *rec_ws = static_cast<unsigned char *>(ws) + node_bytes;
+  const bool compact = compact_ok(d);
+
+#define HT_CALL(fn, FERN_, COMPACT_) fn<Real, FERN_, COMPACT_>(d, x, nodes, w, gout, dx, dthr, dw, rec_ws, stream)
+  if (det) {
+    if (fern) return compact ? HT_CALL(backward_deterministic, true, true) : HT_CALL(backward_deterministic, true, false);
+    return compact ? HT_CALL(backward_deterministic, false, true) : HT_CALL(backward_deterministic, false, false);
+  }
+  if (staged) {
+    if (fern) return compact ? HT_CALL(backward_staged, true, true) : HT_CALL(backward_staged, true, false);
+    return compact ? HT_CALL(backward_staged, false, true) : HT_CALL(backward_staged, false, false);
+  }
+#undef HT_CALL
+  return fern ? dispatch_backward_fused<Real, true>(d, x, nodes, w, gout, dx, dthr, dw, stream)
+              : dispatch_backward_fused<Real, false>(d, x, nodes, w, gout, dx, dthr, dw, stream);
 }
 
-template size_t forest_backward_workspace<float>(const ForestDims &, int);
-template size_t forest_backward_workspace<double>(const ForestDims &, int);
+template size_t forest_backward_workspace<float>(const ForestDims &, int, bool, bool, bool);
+template size_t forest_backward_workspace<double>(const ForestDims &, int, bool, bool, bool);
 template int forest_backward<float>(const ForestDims &, bool, const float *, const float *, const int64_t *,
                                     const float *, const float *, float *, float *, float *, int, void *, size_t,
                                     hipStream_t);

@@ -1,26 +1,44 @@
 // Forest / fern forward: out[b,t,k,m] = |margin| * w[t,leaf,m].
 //
-// One workgroup = one tile of BT samples (all features in LDS, feature major) x a range of trees. Per pass the
-// NT/BT tree slots walk one tree each (lane = sample), park (|margin|, leaf) in LDS, and then the whole workgroup
-// writes the pass' outputs with the thread index running along the contiguous (tree, m) -- or for K > 1 the
-// contiguous (inner position, m) -- axis of `out`, so the dominant store traffic is emitted as full-width rows.
+// A tiny pre-pass packs (threshold, ordinal) of every vertex into one aligned word pair (ordinals narrowed from the
+// API's int64 and clamped into range), so a walk step costs one vertex load plus one LDS gather.
+//
+// One workgroup = one tile of BT samples (all features in LDS, feature major) x a range of trees. Per pass every
+// thread walks TWO trees for its sample (interleaved, so the two dependent load chains overlap), parks
+// (|margin|, leaf) in LDS, and then the workgroup writes the pass' outputs with the lane index running along the
+// contiguous (tree, m) -- or for K > 1 the contiguous (inner position, m) -- axis of `out`, so the dominant store
+// traffic is emitted as full-width rows.
 #include "forest_tile.hpp"
 
 namespace ht {
 namespace {
 
+template <typename Real>
+__global__ __launch_bounds__(256) void pack_nodes_kernel(const Real *__restrict__ thr, const int64_t *__restrict__ ord,
+                                                         Node<Real> *__restrict__ nodes, long long n, int F) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) {
+    Node<Real> v;
+    v.thr = thr[i];
+    v.ord = clamp_ordinal(ord[i], F);
+    nodes[i] = v;
+  }
+}
+
+constexpr int kIlp = 2;  // trees walked concurrently per thread
+
 template <typename Real, bool FERN, int BT, bool XLDS>
 __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, const Real *__restrict__ x,
-                                                                 const Real *__restrict__ thr,
-                                                                 const int64_t *__restrict__ ord,
+                                                                 const Node<Real> *__restrict__ nodes,
                                                                  const Real *__restrict__ w, Real *__restrict__ out,
-                                                                 int trees_per_block) {
+                                                                 int trees_per_block, FastDiv div_m) {
   constexpr int NT = kForestThreads;
-  constexpr int TC = NT / BT;  // trees walked per pass
+  constexpr int TC = NT / BT;        // tree slots per walk round
+  constexpr int TP = TC * kIlp;      // trees per pass
   extern __shared__ __align__(16) unsigned char smem[];
   Real *xs = reinterpret_cast<Real *>(smem);
   Real *r_abs = xs + (XLDS ? size_t(d.F) * BT : 0);
-  uint32_t *r_key = reinterpret_cast<uint32_t *>(r_abs + TC * BT);
+  uint32_t *r_key = reinterpret_cast<uint32_t *>(r_abs + TP * BT);
 
   const long long s0 = (long long)blockIdx.x * BT;
   if (XLDS) {
@@ -34,32 +52,39 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
 
   const int t_begin = blockIdx.y * trees_per_block;
   const int t_end = min(d.T, t_begin + trees_per_block);
-  for (int tb = t_begin; tb < t_end; tb += TC) {
-    const int t = tb + tt;
-    if (t < t_end && live) {
-      const Real *th = thr + (long long)t * d.V;
-      const int64_t *od = ord + (long long)t * d.V;
-      auto node = [&](uint32_t at, Real &tv, int &ov) { tv = th[at]; ov = clamp_ordinal(od[at], d.F); };
-      WalkResult<Real> r;
+  for (int tb = t_begin; tb < t_end; tb += TP) {
+    if (live && tb + tt < t_end) {
+      const Node<Real> *nd[kIlp];
+#pragma unroll
+      for (int i = 0; i < kIlp; ++i) {
+        const int t = min(tb + tt + i * TC, t_end - 1);  // an out-of-range slot re-walks the last tree, unused
+        nd[i] = nodes + (long long)t * d.V;
+      }
+      WalkResult<Real> r[kIlp];
       if (XLDS)
-        r = walk<Real, FERN>(d.depth, node, [&](int f) { return xs[f * BT + j]; });
+        walk_many<Real, FERN, kIlp>(d.depth, nd, [&](int, int f) { return xs[f * BT + j]; }, r);
       else
-        r = walk<Real, FERN>(d.depth, node, [&](int f) { return x[xbase + (long long)f * d.K]; });
-      r_abs[tt * BT + j] = ht_abs(r.margin);
-      r_key[tt * BT + j] = r.key;
+        walk_many<Real, FERN, kIlp>(d.depth, nd, [&](int, int f) { return x[xbase + (long long)f * d.K]; }, r);
+#pragma unroll
+      for (int i = 0; i < kIlp; ++i) {
+        r_abs[(tt + i * TC) * BT + j] = ht_abs(r[i].margin);
+        r_key[(tt + i * TC) * BT + j] = r[i].key;
+      }
     }
     __syncthreads();
-    const int nt = min(TC, t_end - tb);
+    const int nt = min(TP, t_end - tb);
     if (d.K == 1) {
-      // out[s, tb .. tb+nt, 0 .. M) is contiguous for a fixed sample
-      const int row = nt * d.M, total = BT * row;
-      for (int idx = threadIdx.x; idx < total; idx += NT) {
-        const int jj = idx / row, r = idx - jj * row;
-        const int t2 = r / d.M, m = r - t2 * d.M;
+      // out[s, tb .. tb+nt, 0 .. M) is one contiguous row per sample: a wavefront per row, lanes along the row
+      const int row = nt * d.M;
+      const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+      for (int jj = wv; jj < BT; jj += NT / kWave) {
         const long long ss = s0 + jj;
-        if (ss < d.S) {
+        if (ss >= d.S) break;
+        Real *orow = out + (ss * d.T + tb) * d.M;
+        for (int r = lane; r < row; r += kWave) {
+          const int t2 = div_m.div(r), m = r - t2 * d.M;
           const uint32_t key = r_key[t2 * BT + jj];
-          out[(ss * d.T + tb) * d.M + r] = r_abs[t2 * BT + jj] * w[((long long)(tb + t2) * d.L + key) * d.M + m];
+          orow[r] = r_abs[t2 * BT + jj] * w[((long long)(tb + t2) * d.L + key) * d.M + m];
         }
       }
     } else {
@@ -67,7 +92,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
       const int row = BT * d.M, total = nt * row;
       for (int idx = threadIdx.x; idx < total; idx += NT) {
         const int t2 = idx / row, r = idx - t2 * row;
-        const int jj = r / d.M, m = r - jj * d.M;
+        const int jj = div_m.div(r), m = r - jj * d.M;
         const long long ss = s0 + jj;
         if (ss < d.S) {
           const uint32_t key = r_key[t2 * BT + jj];
@@ -80,53 +105,79 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
 }
 
 template <typename Real, bool FERN, int BT, bool XLDS>
-int launch_forward(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, const Real *w, Real *out,
+int launch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
                    hipStream_t stream) {
-  constexpr int TC = kForestThreads / BT;
-  const size_t lds = (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TC) * BT * (sizeof(Real) + sizeof(uint32_t));
+  constexpr int TP = kForestThreads / BT * kIlp;
+  const size_t lds = (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TP) * BT * (sizeof(Real) + sizeof(uint32_t));
   const long long tiles = (d.S + BT - 1) / BT;
-  // Split the trees over blockIdx.y when there are too few sample tiles to fill 256 CUs.
-  const int passes = (d.T + TC - 1) / TC;
-  long long want = tiles >= 512 ? 1 : (512 + tiles - 1) / tiles;
-  const int split = int(want < passes ? want : passes);
-  const int trees_per_block = ((passes + split - 1) / split) * TC;
-  const int gy = (d.T + trees_per_block - 1) / trees_per_block;
+  int trees_per_block, gy;
+  split_trees(tiles, d.T, TP, &trees_per_block, &gy);
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
   auto kernel = forward_kernel<Real, FERN, BT, XLDS>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, thr, ord, w,
-                     out, trees_per_block);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, nodes, w, out,
+                     trees_per_block, FastDiv(d.M));
   HT_LAUNCH_CHECK("forest forward");
   return HT_OK;
 }
 
 template <typename Real, bool FERN>
-int dispatch_forward(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, const Real *w, Real *out,
+int dispatch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
                      hipStream_t stream) {
-  const size_t reserve = 16 * 1024;
+  const size_t reserve = 24 * 1024;
   switch (pick_tile<Real>(d.F, reserve)) {
-    case 64: return launch_forward<Real, FERN, 64, true>(d, x, thr, ord, w, out, stream);
-    case 32: return launch_forward<Real, FERN, 32, true>(d, x, thr, ord, w, out, stream);
-    case 16: return launch_forward<Real, FERN, 16, true>(d, x, thr, ord, w, out, stream);
-    case 8: return launch_forward<Real, FERN, 8, true>(d, x, thr, ord, w, out, stream);
-    default: return launch_forward<Real, FERN, 64, false>(d, x, thr, ord, w, out, stream);
+    case 64: return launch_forward<Real, FERN, 64, true>(d, x, nodes, w, out, stream);
+    case 32: return launch_forward<Real, FERN, 32, true>(d, x, nodes, w, out, stream);
+    case 16: return launch_forward<Real, FERN, 16, true>(d, x, nodes, w, out, stream);
+    case 8: return launch_forward<Real, FERN, 8, true>(d, x, nodes, w, out, stream);
+    default: return launch_forward<Real, FERN, 64, false>(d, x, nodes, w, out, stream);
   }
 }
 
 }  // namespace
 
 template <typename Real>
-int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                   Real *out, hipStream_t stream) {
-  if (d.S == 0 || d.T == 0) return HT_OK;
-  return fern ? dispatch_forward<Real, true>(d, x, thr, ord, w, out, stream)
-              : dispatch_forward<Real, false>(d, x, thr, ord, w, out, stream);
+size_t packed_nodes_bytes(const ForestDims &d) {
+  return align_up(size_t(d.T) * d.V * sizeof(Node<Real>), 256);
 }
 
-template int forest_forward<float>(const ForestDims &, bool, const float *, const float *, const int64_t *, const float *,
-                                   float *, hipStream_t);
-template int forest_forward<double>(const ForestDims &, bool, const double *, const double *, const int64_t *,
-                                    const double *, double *, hipStream_t);
+template <typename Real>
+int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *dst, hipStream_t stream) {
+  const long long n = (long long)d.T * d.V;
+  if (n == 0) return HT_OK;
+  hipLaunchKernelGGL(pack_nodes_kernel<Real>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, thr, ord,
+                     static_cast<Node<Real> *>(dst), n, d.F);
+  HT_LAUNCH_CHECK("pack vertices");
+  return HT_OK;
+}
+
+template <typename Real>
+size_t forest_forward_workspace(const ForestDims &d) {
+  return packed_nodes_bytes<Real>(d);
+}
+
+template <typename Real>
+int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
+                   Real *out, void *ws, size_t ws_bytes, hipStream_t stream) {
+  if (d.S == 0 || d.T == 0) return HT_OK;
+  if (ws == nullptr || ws_bytes < packed_nodes_bytes<Real>(d))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the forward pass.");
+  int rc = pack_nodes<Real>(d, thr, ord, ws, stream);
+  if (rc != HT_OK) return rc;
+  const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
+  return fern ? dispatch_forward<Real, true>(d, x, nodes, w, out, stream)
+              : dispatch_forward<Real, false>(d, x, nodes, w, out, stream);
+}
+
+#define HT_INSTANTIATE(Real)                                                                                          \
+  template size_t packed_nodes_bytes<Real>(const ForestDims &);                                                       \
+  template int pack_nodes<Real>(const ForestDims &, const Real *, const int64_t *, void *, hipStream_t);              \
+  template size_t forest_forward_workspace<Real>(const ForestDims &);                                                 \
+  template int forest_forward<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,            \
+                                    const Real *, Real *, void *, size_t, hipStream_t);
+HT_INSTANTIATE(float)
+HT_INSTANTIATE(double)
+#undef HT_INSTANTIATE
 
 }  // namespace ht

@@ -141,8 +141,13 @@ int ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, hipStream_t st
 }
 
 template <typename Real>
+size_t forest_maps_workspace(const ForestDims &) {
+  return 0;
+}
+
+template <typename Real>
 int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap,
-                Real *margins, int64_t *ordinals, int64_t *reach, hipStream_t stream) {
+                Real *margins, int64_t *ordinals, int64_t *reach, void *, size_t, hipStream_t stream) {
   int rc;
   if (reach && (rc = zero_fill(reach, size_t(d.T) * d.L * sizeof(int64_t), stream)) != HT_OK) return rc;
   if (d.S == 0 || d.T == 0) return HT_OK;
@@ -150,9 +155,11 @@ int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, 
               : dispatch_maps<Real, false>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
 }
 
+template size_t forest_maps_workspace<float>(const ForestDims &);
+template size_t forest_maps_workspace<double>(const ForestDims &);
 template int forest_maps<float>(const ForestDims &, bool, const float *, const float *, const int64_t *, int64_t *,
-                                float *, int64_t *, int64_t *, hipStream_t);
+                                float *, int64_t *, int64_t *, void *, size_t, hipStream_t);
 template int forest_maps<double>(const ForestDims &, bool, const double *, const double *, const int64_t *, int64_t *,
-                                 double *, int64_t *, int64_t *, hipStream_t);
+                                 double *, int64_t *, int64_t *, void *, size_t, hipStream_t);
 
 }  // namespace ht

@@ -35,6 +35,60 @@ __device__ __forceinline__ Real ht_sign(Real m) {
   return Real((Real(0) < m) - (m < Real(0)));
 }
 
+// A decision vertex as the kernels read it: threshold and (range-clamped) ordinal in one naturally aligned load.
+template <typename Real>
+struct Node;
+template <>
+struct __align__(8) Node<float> {
+  float thr;
+  int ord;
+};
+template <>
+struct __align__(16) Node<double> {
+  double thr;
+  long long ord;
+};
+
+// N independent walks advanced level by level in one loop, so that their dependent load chains overlap.
+// `nodes[i]` is the packed vertex array of walk i, `feature(i, f)` returns walk i's sample value of feature f.
+template <typename Real, bool FERN, int N, typename FeatureFn>
+__device__ __forceinline__ void walk_many(int depth, const Node<Real> *const (&nodes)[N], FeatureFn feature,
+                                          WalkResult<Real> (&r)[N]) {
+  uint32_t v[N];
+  Real best_abs[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    v[i] = 0;
+    r[i].key = 0;
+    r[i].vertex = 0;
+    r[i].margin = Real(0);
+    best_abs[i] = Real(0);
+  }
+  for (int lvl = 0; lvl < depth; ++lvl) {
+    Node<Real> n[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) n[i] = nodes[i][FERN ? uint32_t(lvl) : v[i]];
+    Real m[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) m[i] = feature(i, int(n[i].ord)) - n[i].thr;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const uint32_t at = FERN ? uint32_t(lvl) : v[i];
+      const uint32_t bit = (m[i] > Real(0)) ? 1u : 0u;
+      const Real a = ht_abs(m[i]);
+      // level 0 seeds the minimum unconditionally (also when the root margin is NaN, which then sticks)
+      if (lvl == 0 || a < best_abs[i]) {
+        best_abs[i] = a;
+        r[i].margin = m[i];
+        r[i].vertex = at;
+      }
+      r[i].key |= bit << lvl;
+      v[i] = 2u * v[i] + 1u + bit;
+    }
+  }
+}
+
+// Single walk over separate threshold / ordinal arrays (used where the vertices are not packed).
 // `node(i)` returns (threshold, ordinal) of decision i; `feature(f)` returns this sample's value of feature f.
 template <typename Real, bool FERN, typename NodeFn, typename FeatureFn>
 __device__ __forceinline__ WalkResult<Real> walk(int depth, NodeFn node, FeatureFn feature) {
@@ -42,13 +96,8 @@ __device__ __forceinline__ WalkResult<Real> walk(int depth, NodeFn node, Feature
   uint32_t v = 0;
   r.key = 0;
   r.vertex = 0;
-  {
-    Real th;
-    int o;
-    node(0u, th, o);
-    r.margin = feature(o) - th;
-  }
-  Real best_abs = ht_abs(r.margin);
+  r.margin = Real(0);
+  Real best_abs = Real(0);
   for (int lvl = 0; lvl < depth; ++lvl) {
     const uint32_t at = FERN ? uint32_t(lvl) : v;
     Real th;
@@ -57,7 +106,7 @@ __device__ __forceinline__ WalkResult<Real> walk(int depth, NodeFn node, Feature
     const Real m = feature(o) - th;
     const uint32_t bit = (m > Real(0)) ? 1u : 0u;
     const Real a = ht_abs(m);
-    if (a < best_abs) {
+    if (lvl == 0 || a < best_abs) {
       best_abs = a;
       r.margin = m;
       r.vertex = at;

@@ -43,6 +43,12 @@ def _stream(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
+def _workspace(nbytes, device):
+    """Scratch for one call from torch's caching allocator. It is allocated and released on the stream the kernels run
+    on, so the allocator cannot hand it to other work before they have finished."""
+    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
+
+
 def _compute_depth(leaves):
     # HingeTreeCommon.h:55-65,141-151: -1 unless the leaf count is a positive power of two
     if leaves <= 0 or (leaves & (leaves - 1)) != 0:
@@ -139,8 +145,10 @@ def _forward(kind, inData, inThresholds, inOrdinals, inWeights):
     with torch.cuda.device(inData.device):
         out = torch.empty(out_sizes, dtype=inData.dtype, device=inData.device)
         lib = L.load()
+        nbytes = lib.ht_forest_forward_workspace(ctypes.byref(shape))
+        ws = _workspace(nbytes, inData.device)
         L.check(lib.ht_forest_forward(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals),
-                                      _ptr(inWeights), _ptr(out), None, 0, _stream(inData.device)))
+                                      _ptr(inWeights), _ptr(out), _ptr(ws), nbytes, _stream(inData.device)))
     return out
 
 
@@ -157,12 +165,10 @@ def _backward(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, 
         lib = L.load()
         nbytes = lib.ht_forest_backward_workspace(ctypes.byref(shape), mode, int(bool(bInDataGrad)),
                                                   int(bool(bInThresholdsGrad)), int(bool(bInWeightsGrad)))
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=inData.device) if nbytes else None
+        ws = _workspace(nbytes, inData.device)
         L.check(lib.ht_forest_backward(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals),
                                        _ptr(inWeights), _ptr(outDataGrad), _ptr(dx), _ptr(dthr), _ptr(dw), mode, _ptr(ws),
                                        nbytes, _stream(inData.device)))
-        if ws is not None:
-            ws.record_stream(torch.cuda.current_stream(inData.device))
     return [dx, dthr, None, dw]
 
 

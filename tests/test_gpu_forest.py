@@ -25,6 +25,11 @@ CASES = [
     (5, 7, [70], 3, 5, [4]),
     (130, 300, [], 35, 10, [3]),
     (4, 5000, [], 3, 4, [2]),              # feature count too large for an LDS tile of 8 float64 rows
+    # large enough (>= 2^18 sample x tree pairs) for the staged backward: records -> trees -> dThr -> dX
+    (2048, 40, [], 130, 6, [10]),
+    (300, 17, [10], 90, 5, [3]),           # inner data dims, odd extra outputs
+    (9000, 20, [], 30, 5, [2]),            # few tree groups: samples split over workgroups, partial dW merged
+    (2100, 33, [], 126, 4, []),
 ]
 
 
