@@ -18,11 +18,13 @@
 // order of additions is fixed (see below). Small problems, very deep trees and very wide inputs use a single fused
 // kernel with global atomics instead.
 #include "forest_tile.hpp"
+#include "lds_accumulate.hpp"
 
 namespace ht {
 namespace {
 
-constexpr int kIlp = 2;
+constexpr int kIlp = 4;         // trees walked concurrently per thread by the records kernel
+constexpr int kTreeSteps = 4;   // steps of the tree-stationary kernel whose loads are in flight together
 
 // ---------------------------------------------------------------------------------------------------------------
 // walk records
@@ -155,50 +157,116 @@ int dispatch_records(const ForestDims &d, const Real *x, const Node<Real> *nodes
 // ---------------------------------------------------------------------------------------------------------------
 // tree-stationary dW + c
 // ---------------------------------------------------------------------------------------------------------------
-// grid = (tree groups, sample parts). Workgroup (g, p) owns trees [g*TB, g*TB + TB) and samples of part p.
-// LDS: dW accumulators [TB][L][M] (if dw). VW = width of the vector loads of g and w (divides M).
+// grid = (tree groups, sample parts). Workgroup (g, p) owns trees [g*TB, g*TB + TB) and the samples of part p.
+// LDS: dW accumulators [TB][L][M] in fp64 (if dw): the fp64 LDS atomic add is a fast hardware instruction on gfx950,
+// the fp32 one is not (see lds_accumulate.hpp); each product |margin| * g is still rounded to Real first, only the
+// running sum is wider.
+//
+// A (sample, tree) pair is served by P = M / VW adjacent lanes, lane p holding elements [p*VW, p*VW + VW) of the
+// pair's M upstream-gradient values and of its leaf-weight row; a wavefront serves G = 64 / P pairs per step, pairs
+// enumerated with the tree index fastest so that consecutive pairs read consecutive memory. This way every cache line
+// of g and w is requested by exactly one load instruction (a thread-per-sample layout re-requests each line once per
+// vector it takes out of it, and the L2 -> L1 traffic of those repeats dominated the kernel). c is reduced over the
+// P lanes with shuffles.
 template <typename Real, int VW, bool COMPACT>
 __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, const Real *__restrict__ w,
                                                               const Real *__restrict__ gout,
                                                               Records<Real, COMPACT> rec, Real *dw, int TB,
-                                                              long long part_size, bool need_c, bool dw_atomic) {
+                                                              long long part_size, bool need_c, bool dw_atomic, int P,
+                                                              FastDiv div_p) {
   typedef Real Vec __attribute__((ext_vector_type(VW)));
   extern __shared__ __align__(16) unsigned char smem[];
-  Real *acc = reinterpret_cast<Real *>(smem);
+  double *acc = reinterpret_cast<double *>(smem);
   const int t0 = blockIdx.x * TB;
   const int nt = min(TB, d.T - t0);
   const long long LM = (long long)d.L * d.M;
   if (dw) {
-    for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) acc[i] = Real(0);
+    for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) acc[i] = 0.0;
     __syncthreads();
   }
   const long long s_begin = (long long)blockIdx.y * part_size;
   const long long s_end = min(d.S, s_begin + part_size);
-  for (long long s = s_begin + threadIdx.x; s < s_end; s += kForestThreads) {
-    const long long b = s / d.K, k = s % d.K;
-    for (int tl = 0; tl < nt; ++tl) {
-      const int t = t0 + tl;
-      const long long at = (long long)t * d.S + s;
-      const uint32_t key = rec.key(at);
-      const Real mg = rec.margin[at];
-      const Real a = ht_abs(mg);
-      const Real *gp = gout + ((b * d.T + t) * d.K + k) * d.M;
-      const Real *wl = w + ((long long)t * d.L + key) * d.M;
-      Real *cell = acc + (long long)tl * LM + (long long)key * d.M;
-      Real cs = Real(0);
-      for (int m = 0; m < d.M; m += VW) {
-        const Vec gv = *reinterpret_cast<const Vec *>(gp + m);
-        if (need_c) {
-          const Vec wv = *reinterpret_cast<const Vec *>(wl + m);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  constexpr int kWaves = kForestThreads / kWave;
+  const int G = kWave / P;                         // pairs per wavefront step (P <= 64)
+  const int grp = div_p.div(lane), pl = lane - grp * P;
+  const bool lane_on = grp < G;
+  // pair q of this workgroup = (sample s_begin + q / nt, tree t0 + q % nt); a lane's q advances by kWaves * G per step
+  const long long npairs = (s_end - s_begin) * nt;
+  const int step = kWaves * G;
+  // kTreeSteps steps are in flight together: all their record loads are issued first, then all gradient and weight
+  // loads, so that a wavefront always has several independent memory round trips outstanding.
+  int sub_s[kTreeSteps], sub_t[kTreeSteps];
 #pragma unroll
-          for (int i = 0; i < VW; ++i) cs += wv[i] * gv[i];
-        }
-        if (dw) {
+  for (int u = 0; u < kTreeSteps; ++u) {
+    sub_s[u] = (u * step) / nt;
+    sub_t[u] = (u * step) - sub_s[u] * nt;
+  }
+  const int big = kTreeSteps * step;
+  const int big_s = big / nt, big_t = big - big_s * nt;
+  long long q = (long long)wave * G + grp;
+  long long sl = q / nt;
+  int tl = int(q - sl * nt);
+  const long long row_stride = (long long)d.T * d.M;  // K == 1: distance between the gradient rows of two samples
+  for (long long q0 = (long long)wave * G; q0 < npairs; q0 += big) {
+    bool on[kTreeSteps];
+    int tq[kTreeSteps];
+    long long at[kTreeSteps], goff[kTreeSteps];
+    uint32_t key[kTreeSteps];
+    Real mg[kTreeSteps];
 #pragma unroll
-          for (int i = 0; i < VW; ++i) atomicAdd(cell + m + i, a * gv[i]);
-        }
+    for (int u = 0; u < kTreeSteps; ++u) {
+      int tu = tl + sub_t[u];
+      long long su = sl + sub_s[u];
+      if (tu >= nt) {
+        tu -= nt;
+        ++su;
       }
-      if (need_c) rec.c[at] = ht_sign(mg) * cs;
+      on[u] = lane_on && q + (long long)u * step < npairs;
+      const long long s = s_begin + (on[u] ? su : 0);
+      tq[u] = on[u] ? tu : 0;
+      const int t = t0 + tq[u];
+      at[u] = (long long)t * d.S + s;
+      if (d.K == 1) {
+        goff[u] = s * row_stride + (long long)t * d.M;
+      } else {
+        const long long b = s / d.K, k = s - b * d.K;
+        goff[u] = ((b * d.T + t) * d.K + k) * d.M;
+      }
+      key[u] = rec.key(at[u]);
+      mg[u] = rec.margin[at[u]];
+    }
+    Vec gv[kTreeSteps], wv[kTreeSteps];
+#pragma unroll
+    for (int u = 0; u < kTreeSteps; ++u) {
+      gv[u] = *reinterpret_cast<const Vec *>(gout + goff[u] + pl * VW);
+      if (need_c) wv[u] = *reinterpret_cast<const Vec *>(w + ((long long)(t0 + tq[u]) * d.L + key[u]) * d.M + pl * VW);
+    }
+#pragma unroll
+    for (int u = 0; u < kTreeSteps; ++u) {
+      if (dw && on[u]) {
+        const Real a = ht_abs(mg[u]);
+        double *cell = acc + (long long)tq[u] * LM + (long long)key[u] * d.M + pl * VW;
+#pragma unroll
+        for (int i = 0; i < VW; ++i) atomicAdd(cell + i, double(a * gv[u][i]));
+      }
+      if (need_c) {
+        Real partial = Real(0);
+#pragma unroll
+        for (int i = 0; i < VW; ++i) partial += wv[u][i] * gv[u][i];
+        for (int off = 1; off < P; off <<= 1) {
+          const Real other = __shfl_down(partial, off, kWave);
+          if (pl + off < P) partial += other;
+        }
+        if (on[u] && pl == 0) rec.c[at[u]] = ht_sign(mg[u]) * partial;
+      }
+    }
+    q += big;
+    sl += big_s;
+    tl += big_t;
+    if (tl >= nt) {
+      tl -= nt;
+      ++sl;
     }
   }
   if (dw) {
@@ -206,9 +274,9 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
     Real *dst = dw + (long long)t0 * LM;
     if (dw_atomic) {
       for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads)
-        if (acc[i] != Real(0)) atomicAdd(dst + i, acc[i]);
+        if (acc[i] != 0.0) atomicAdd(dst + i, Real(acc[i]));
     } else {
-      for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) dst[i] = acc[i];
+      for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) dst[i] = Real(acc[i]);
     }
   }
 }
@@ -218,23 +286,23 @@ template <typename Real, bool COMPACT>
 __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dthr,
                                                    long long part_size, bool use_atomic) {
   extern __shared__ __align__(16) unsigned char smem[];
-  Real *acc = reinterpret_cast<Real *>(smem);
+  double *acc = reinterpret_cast<double *>(smem);  // fp64: fast LDS atomic, and the root vertex is a hot spot
   const int t = blockIdx.x;
-  for (int i = threadIdx.x; i < d.V; i += 256) acc[i] = Real(0);
+  for (int i = threadIdx.x; i < d.V; i += 256) acc[i] = 0.0;
   __syncthreads();
   const long long s_begin = (long long)blockIdx.y * part_size;
   const long long s_end = min(d.S, s_begin + part_size);
   for (long long s = s_begin + threadIdx.x; s < s_end; s += 256) {
     const long long at = (long long)t * d.S + s;
-    atomicAdd(acc + rec.vertex(at), -rec.c[at]);
+    atomicAdd(acc + rec.vertex(at), -double(rec.c[at]));
   }
   __syncthreads();
   Real *dst = dthr + (long long)t * d.V;
   for (int i = threadIdx.x; i < d.V; i += 256) {
     if (use_atomic) {
-      if (acc[i] != Real(0)) atomicAdd(dst + i, acc[i]);
+      if (acc[i] != 0.0) atomicAdd(dst + i, Real(acc[i]));
     } else {
-      dst[i] = acc[i];
+      dst[i] = Real(acc[i]);
     }
   }
 }
@@ -255,7 +323,7 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
   if (s < d.S) {
     for (int t = tt; t < d.T; t += TC) {
       const long long at = (long long)t * d.S + s;
-      atomicAdd(acc + rec.ord(at) * LD + j, rec.c[at]);
+      lds_add(acc + rec.ord(at) * LD + j, rec.c[at]);
     }
   }
   __syncthreads();
@@ -338,7 +406,7 @@ __global__ __launch_bounds__(kForestThreads) void backward_fused_kernel(
           const uint32_t key = r_key[t2 * BT + jj];
           const long long wi = ((long long)(tb + t2) * d.L + key) * d.M + m;
           if (dw) atomicAdd(dw + wi, ht_abs(r_margin[t2 * BT + jj]) * g);
-          if (need_c) atomicAdd(r_csum + t2 * BT + jj, w[wi] * g);
+          if (need_c) lds_add(r_csum + t2 * BT + jj, w[wi] * g);
         }
       }
     }
@@ -535,7 +603,7 @@ struct TreePlan {
 
 template <typename Real>
 bool plan_trees(const ForestDims &d, bool need_dw, const Real *w, const Real *gout, TreePlan *p) {
-  const size_t per_tree = size_t(d.L) * d.M * sizeof(Real);
+  const size_t per_tree = size_t(d.L) * d.M * sizeof(double);
   int tb = 4;
   if (need_dw) {
     if (per_tree > size_t(kLdsBytes)) return false;
@@ -570,7 +638,7 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(p.lds)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)p.groups, (unsigned)p.parts), dim3(kForestThreads), p.lds, stream, d, w,
-                     gout, rec, dw, p.TB, p.part_size, need_c, p.parts > 1);
+                     gout, rec, dw, p.TB, p.part_size, need_c, p.parts > 1, d.M / VW, FastDiv(d.M / VW));
   HT_LAUNCH_CHECK("forest backward (trees)");
   return HT_OK;
 }
@@ -600,8 +668,9 @@ int pick_dx_tile(int F) {
 template <typename Real>
 bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw) {
   if (d.M < 1) return false;
-  if (need_dw && size_t(d.L) * d.M * sizeof(Real) > size_t(kLdsBytes)) return false;
-  if (size_t(d.V) * sizeof(Real) > size_t(kLdsBytes)) return false;
+  if (d.M > kWave) return false;  // the lanes serving one (sample, tree) pair must fit a wavefront
+  if (need_dw && size_t(d.L) * d.M * sizeof(double) > size_t(kLdsBytes)) return false;
+  if (size_t(d.V) * sizeof(double) > size_t(kLdsBytes)) return false;
   if (need_dx && pick_dx_tile<Real>(d.F) == 0) return false;
   return true;
 }
@@ -633,7 +702,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
     const long long part_size = (d.S + parts - 1) / parts;
     const int gy = int((d.S + part_size - 1) / part_size);
     hipLaunchKernelGGL((dthr_kernel<Real, COMPACT>), dim3((unsigned)d.T, (unsigned)gy), dim3(256),
-                       size_t(d.V) * sizeof(Real), stream, d, rec, dthr, part_size, gy > 1);
+                       size_t(d.V) * sizeof(double), stream, d, rec, dthr, part_size, gy > 1);
     HT_LAUNCH_CHECK("forest backward (dThr)");
   }
   if (dx) {

@@ -25,20 +25,25 @@ __global__ __launch_bounds__(256) void pack_nodes_kernel(const Real *__restrict_
   }
 }
 
-constexpr int kIlp = 2;  // trees walked concurrently per thread
+constexpr int kOutUnroll = 10;  // outputs per lane whose weight gathers are in flight together
 
-template <typename Real, bool FERN, int BT, bool XLDS>
+// ILP = trees walked concurrently per thread; KeyT = storage type of the parked leaf keys (uint16_t up to depth 16).
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT>
 __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, const Real *__restrict__ x,
                                                                  const Node<Real> *__restrict__ nodes,
                                                                  const Real *__restrict__ w, Real *__restrict__ out,
                                                                  int trees_per_block, FastDiv div_m) {
   constexpr int NT = kForestThreads;
   constexpr int TC = NT / BT;        // tree slots per walk round
+  constexpr int kIlp = ILP;
   constexpr int TP = TC * kIlp;      // trees per pass
+  constexpr int LDR = TP + 1;        // row pitch of the per-pass results, [sample][tree]: odd, so that both the
+                                     // walk's writes (lane = sample) and the output's reads (lane = tree) spread
+                                     // over the LDS banks
   extern __shared__ __align__(16) unsigned char smem[];
   Real *xs = reinterpret_cast<Real *>(smem);
   Real *r_abs = xs + (XLDS ? size_t(d.F) * BT : 0);
-  uint32_t *r_key = reinterpret_cast<uint32_t *>(r_abs + TP * BT);
+  KeyT *r_key = reinterpret_cast<KeyT *>(r_abs + LDR * BT);
 
   const long long s0 = (long long)blockIdx.x * BT;
   if (XLDS) {
@@ -67,8 +72,8 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
         walk_many<Real, FERN, kIlp>(d.depth, nd, [&](int, int f) { return x[xbase + (long long)f * d.K]; }, r);
 #pragma unroll
       for (int i = 0; i < kIlp; ++i) {
-        r_abs[(tt + i * TC) * BT + j] = ht_abs(r[i].margin);
-        r_key[(tt + i * TC) * BT + j] = r[i].key;
+        r_abs[j * LDR + tt + i * TC] = ht_abs(r[i].margin);
+        r_key[j * LDR + tt + i * TC] = KeyT(r[i].key);
       }
     }
     __syncthreads();
@@ -76,15 +81,25 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
     if (d.K == 1) {
       // out[s, tb .. tb+nt, 0 .. M) is one contiguous row per sample: a wavefront per row, lanes along the row
       const int row = nt * d.M;
-      const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
-      for (int jj = wv; jj < BT; jj += NT / kWave) {
+      const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+      for (int jj = wave; jj < BT; jj += NT / kWave) {
         const long long ss = s0 + jj;
         if (ss >= d.S) break;
         Real *orow = out + (ss * d.T + tb) * d.M;
-        for (int r = lane; r < row; r += kWave) {
-          const int t2 = div_m.div(r), m = r - t2 * d.M;
-          const uint32_t key = r_key[t2 * BT + jj];
-          orow[r] = r_abs[t2 * BT + jj] * w[((long long)(tb + t2) * d.L + key) * d.M + m];
+        // kOutUnroll independent leaf-weight gathers are issued before the first store
+        for (int r0 = lane; r0 < row; r0 += kWave * kOutUnroll) {
+          Real a[kOutUnroll], wv[kOutUnroll];
+#pragma unroll
+          for (int u = 0; u < kOutUnroll; ++u) {
+            const int r = min(r0 + u * kWave, row - 1);
+            const int t2 = div_m.div(r), m = r - t2 * d.M;
+            const uint32_t key = r_key[jj * LDR + t2];
+            a[u] = r_abs[jj * LDR + t2];
+            wv[u] = w[((long long)(tb + t2) * d.L + key) * d.M + m];
+          }
+#pragma unroll
+          for (int u = 0; u < kOutUnroll; ++u)
+            if (r0 + u * kWave < row) orow[r0 + u * kWave] = a[u] * wv[u];
         }
       }
     } else {
@@ -95,8 +110,8 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
         const int jj = div_m.div(r), m = r - jj * d.M;
         const long long ss = s0 + jj;
         if (ss < d.S) {
-          const uint32_t key = r_key[t2 * BT + jj];
-          out[out_offset(d, ss, tb + t2, m)] = r_abs[t2 * BT + jj] * w[((long long)(tb + t2) * d.L + key) * d.M + m];
+          const uint32_t key = r_key[jj * LDR + t2];
+          out[out_offset(d, ss, tb + t2, m)] = r_abs[jj * LDR + t2] * w[((long long)(tb + t2) * d.L + key) * d.M + m];
         }
       }
     }
@@ -104,16 +119,16 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
   }
 }
 
-template <typename Real, bool FERN, int BT, bool XLDS>
-int launch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                   hipStream_t stream) {
-  constexpr int TP = kForestThreads / BT * kIlp;
-  const size_t lds = (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TP) * BT * (sizeof(Real) + sizeof(uint32_t));
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT>
+int launch_forward_as(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
+                      hipStream_t stream) {
+  constexpr int TP = kForestThreads / BT * ILP;
+  const size_t lds = (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TP + 1) * BT * (sizeof(Real) + sizeof(KeyT));
   const long long tiles = (d.S + BT - 1) / BT;
   int trees_per_block, gy;
   split_trees(tiles, d.T, TP, &trees_per_block, &gy);
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
-  auto kernel = forward_kernel<Real, FERN, BT, XLDS>;
+  auto kernel = forward_kernel<Real, FERN, BT, XLDS, ILP, KeyT>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, nodes, w, out,
@@ -122,10 +137,20 @@ int launch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, 
   return HT_OK;
 }
 
+// Four trees per thread with 16-bit parked keys where the depth allows it, else two trees with 32-bit keys: both keep
+// the per-pass results of a 1024-thread workgroup under the LDS left beside a 128 KB sample tile.
+template <typename Real, bool FERN, int BT, bool XLDS>
+int launch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
+                   hipStream_t stream) {
+  if (d.depth <= 16) return launch_forward_as<Real, FERN, BT, XLDS, 4, uint16_t>(d, x, nodes, w, out, stream);
+  return launch_forward_as<Real, FERN, BT, XLDS, 2, uint32_t>(d, x, nodes, w, out, stream);
+}
+
 template <typename Real, bool FERN>
 int dispatch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
                      hipStream_t stream) {
-  const size_t reserve = 24 * 1024;
+  // room for the per-pass results: (4 trees x 1024 threads + one pad column) x (|margin| + key)
+  const size_t reserve = size_t(4) * kForestThreads * (sizeof(Real) + sizeof(uint32_t));
   switch (pick_tile<Real>(d.F, reserve)) {
     case 64: return launch_forward<Real, FERN, 64, true>(d, x, nodes, w, out, stream);
     case 32: return launch_forward<Real, FERN, 32, true>(d, x, nodes, w, out, stream);

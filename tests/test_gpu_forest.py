@@ -30,6 +30,8 @@ CASES = [
     (300, 17, [10], 90, 5, [3]),           # inner data dims, odd extra outputs
     (9000, 20, [], 30, 5, [2]),            # few tree groups: samples split over workgroups, partial dW merged
     (2100, 33, [], 126, 4, []),
+    (600, 16, [], 450, 3, [8, 8]),         # 64 outputs per leaf: 16 lanes per pair with 4-wide loads
+    (520, 12, [], 520, 3, [70]),           # more outputs per leaf than a wavefront has lanes: fused kernel
 ]
 
 
