@@ -10,9 +10,11 @@ extra_outputs = 10 (out [65536, 1000, 10]); thresholds ~ U(-3,3) made consistent
 ordinals ~ U{0..1023}, leaf weights ~ N(0,1), upstream gradient ~ N(0,1).
 
 Prints ONE JSON line. `value` is samples/s over the timed steps (wall clock between device synchronisations);
-`roofline` prices the dominant pass (backward) against the 8 TB/s HBM peak using the algorithmic bytes of that pass
-(every input read once, every output written once) and its duration measured with events on the launch stream;
-`cpu_baseline` is the single-threaded CPU oracle timed on a bounded slice of the same workload on this host.
+`roofline` prices the dominant kernel (the forward kernel: tree_forward launches it plus a ~7 us vertex-packing
+pre-pass) against the 8 TB/s HBM peak using its algorithmic bytes (every input read once, every output written once)
+and its duration measured with events on the launch stream; `backward` and `step_hbm_frac` give the same fraction for
+the backward pass (five kernels) and for the whole step; `cpu_baseline` is the single-threaded CPU oracle timed on a
+bounded slice of the same workload on this host.
 """
 import argparse
 import json
@@ -24,6 +26,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per launch of the forward kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (KiB per dispatch,
+# scaled by what the same counters read for a plain 1 GiB copy: x2.0 for FETCH_SIZE, x1.0 for WRITE_SIZE); the
+# summaries are under profiles/.
+MEASURED_TRAFFIC = {"c3": None}
 
 WORKLOADS = {
     # name: (B, F, T, depth, M, kind, x distribution, description)
@@ -139,7 +146,7 @@ def main():
     bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
 
     fwd_bytes, bwd_bytes = algorithmic_bytes(B, F, T, depth, M, kind)
-    achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    achieved = fwd_bytes / (fwd_ms * 1e-3) / 1e9
     result = {
         "metric": "fwd+bwd samples/s (forest B=65536,F=1024,T=1000,D=10) + % of HBM peak BW",
         "value": B / (ms_per_step * 1e-3),
@@ -155,11 +162,11 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{name}: {desc}", "backward_mode": args.mode, "B": B, "F": F, "T": T, "depth": depth,
                    "extra_outputs": M},
-        "roofline": {"bound": "hbm", "kernel": f"{kind} backward ({args.mode})", "achieved": achieved,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
-                     "algorithmic_bytes": bwd_bytes, "ms": bwd_ms},
-        "forward": {"ms": fwd_ms, "samples_per_s": B / (fwd_ms * 1e-3), "algorithmic_bytes": fwd_bytes,
-                    "hbm_frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "roofline": {"bound": "hbm", "kernel": "forward_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get(name),
+                     "algorithmic_bytes": fwd_bytes, "ms": fwd_ms, "samples_per_s": B / (fwd_ms * 1e-3)},
+        "backward": {"mode": args.mode, "ms": bwd_ms, "samples_per_s": B / (bwd_ms * 1e-3),
+                     "algorithmic_bytes": bwd_bytes, "hbm_frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
         "step_hbm_frac": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
     }
     if args.cpu_rows > 0:

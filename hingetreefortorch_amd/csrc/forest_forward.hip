@@ -25,14 +25,17 @@ __global__ __launch_bounds__(256) void pack_nodes_kernel(const Real *__restrict_
   }
 }
 
-constexpr int kOutUnroll = 10;  // outputs per lane whose weight gathers are in flight together
+constexpr int kOutUnroll = 5;  // output vectors per lane whose weight gathers are in flight together
 
-// ILP = trees walked concurrently per thread; KeyT = storage type of the parked leaf keys (uint16_t up to depth 16).
-template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT>
+// ILP = trees walked concurrently per thread; KeyT = storage type of the parked leaf keys (uint16_t up to depth 16);
+// VW = outputs per lane in the output phase (divides M): the memory pipeline charges a gather instruction by its
+// lanes, not by the lines it touches, so wider lanes mean proportionally fewer cycles per output.
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
 __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, const Real *__restrict__ x,
                                                                  const Node<Real> *__restrict__ nodes,
                                                                  const Real *__restrict__ w, Real *__restrict__ out,
                                                                  int trees_per_block, FastDiv div_m) {
+  typedef Real Vec __attribute__((ext_vector_type(VW)));
   constexpr int NT = kForestThreads;
   constexpr int TC = NT / BT;        // tree slots per walk round
   constexpr int kIlp = ILP;
@@ -87,19 +90,26 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
         if (ss >= d.S) break;
         Real *orow = out + (ss * d.T + tb) * d.M;
         // kOutUnroll independent leaf-weight gathers are issued before the first store
-        for (int r0 = lane; r0 < row; r0 += kWave * kOutUnroll) {
-          Real a[kOutUnroll], wv[kOutUnroll];
+        for (int r0 = lane * VW; r0 < row; r0 += kWave * VW * kOutUnroll) {
+          Real a[kOutUnroll];
+          Vec wv[kOutUnroll];
 #pragma unroll
           for (int u = 0; u < kOutUnroll; ++u) {
-            const int r = min(r0 + u * kWave, row - 1);
+            const int r = min(r0 + u * kWave * VW, row - VW);
             const int t2 = div_m.div(r), m = r - t2 * d.M;
             const uint32_t key = r_key[jj * LDR + t2];
             a[u] = r_abs[jj * LDR + t2];
-            wv[u] = w[((long long)(tb + t2) * d.L + key) * d.M + m];
+            wv[u] = *reinterpret_cast<const Vec *>(w + ((long long)(tb + t2) * d.L + key) * d.M + m);
           }
 #pragma unroll
-          for (int u = 0; u < kOutUnroll; ++u)
-            if (r0 + u * kWave < row) orow[r0 + u * kWave] = a[u] * wv[u];
+          for (int u = 0; u < kOutUnroll; ++u) {
+            if (r0 + u * kWave * VW < row) {
+              Vec o;
+#pragma unroll
+              for (int i = 0; i < VW; ++i) o[i] = a[u] * wv[u][i];
+              *reinterpret_cast<Vec *>(orow + r0 + u * kWave * VW) = o;
+            }
+          }
         }
       }
     } else {
@@ -119,8 +129,8 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
   }
 }
 
-template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT>
-int launch_forward_as(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
+int launch_forward_vw(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
                       hipStream_t stream) {
   constexpr int TP = kForestThreads / BT * ILP;
   const size_t lds = (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TP + 1) * BT * (sizeof(Real) + sizeof(KeyT));
@@ -128,13 +138,25 @@ int launch_forward_as(const ForestDims &d, const Real *x, const Node<Real> *node
   int trees_per_block, gy;
   split_trees(tiles, d.T, TP, &trees_per_block, &gy);
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
-  auto kernel = forward_kernel<Real, FERN, BT, XLDS, ILP, KeyT>;
+  auto kernel = forward_kernel<Real, FERN, BT, XLDS, ILP, KeyT, VW>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, nodes, w, out,
                      trees_per_block, FastDiv(d.M));
   HT_LAUNCH_CHECK("forest forward");
   return HT_OK;
+}
+
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT>
+int launch_forward_as(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
+                      hipStream_t stream) {
+  // widest output vector that M and the pointers allow (K > 1 keeps scalar outputs)
+  const uintptr_t pw = reinterpret_cast<uintptr_t>(w), po = reinterpret_cast<uintptr_t>(out);
+  if (d.K == 1 && d.M % 4 == 0 && pw % (4 * sizeof(Real)) == 0 && po % (4 * sizeof(Real)) == 0)
+    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, 4>(d, x, nodes, w, out, stream);
+  if (d.K == 1 && d.M % 2 == 0 && pw % (2 * sizeof(Real)) == 0 && po % (2 * sizeof(Real)) == 0)
+    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, 2>(d, x, nodes, w, out, stream);
+  return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, 1>(d, x, nodes, w, out, stream);
 }
 
 // Four trees per thread with 16-bit parked keys where the depth allows it, else two trees with 32-bit keys: both keep
