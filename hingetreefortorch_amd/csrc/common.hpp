@@ -41,6 +41,7 @@ constexpr int kWave = 64;
 constexpr int kLdsBytes = 160 * 1024;       // LDS per CU / per workgroup limit on gfx950
 constexpr int kForestThreads = 1024;        // workgroup size of the tile kernels
 constexpr int kNumCUs = 256;                // MI355X
+constexpr int kNumXCDs = 8;                 // accelerator dies, each with its own L2; workgroup i runs on XCD i mod 8
 
 // n / d for n * d < 2^32 by multiply-high with ceil(2^32 / d) (d >= 1).
 struct FastDiv {

@@ -173,11 +173,17 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
                                                               const Real *__restrict__ gout,
                                                               Records<Real, COMPACT> rec, Real *dw, int TB,
                                                               long long part_size, bool need_c, bool dw_atomic, int P,
-                                                              FastDiv div_p) {
+                                                              FastDiv div_p, int num_groups) {
   typedef Real Vec __attribute__((ext_vector_type(VW)));
   extern __shared__ __align__(16) unsigned char smem[];
   double *acc = reinterpret_cast<double *>(smem);
-  const int t0 = blockIdx.x * TB;
+  // Workgroups are dealt to the 8 XCDs round robin by index, and each XCD has its own L2. Adjacent tree groups read
+  // adjacent pieces of the same 128-byte lines of the upstream gradient, so they are placed on the same XCD (group =
+  // (index mod 8) * groups_per_xcd + index / 8): the line is then fetched from memory once instead of once per XCD.
+  const int per_xcd = (num_groups + kNumXCDs - 1) / kNumXCDs;
+  const int group = int(blockIdx.x % kNumXCDs) * per_xcd + int(blockIdx.x / kNumXCDs);
+  if (group >= num_groups) return;
+  const int t0 = group * TB;
   const int nt = min(TB, d.T - t0);
   const long long LM = (long long)d.L * d.M;
   if (dw) {
@@ -637,8 +643,10 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
   auto kernel = tree_kernel<Real, VW, COMPACT>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(p.lds)));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)p.groups, (unsigned)p.parts), dim3(kForestThreads), p.lds, stream, d, w,
-                     gout, rec, dw, p.TB, p.part_size, need_c, p.parts > 1, d.M / VW, FastDiv(d.M / VW));
+  const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts), dim3(kForestThreads), p.lds,
+                     stream, d, w, gout, rec, dw, p.TB, p.part_size, need_c, p.parts > 1, d.M / VW,
+                     FastDiv(d.M / VW), p.groups);
   HT_LAUNCH_CHECK("forest backward (trees)");
   return HT_OK;
 }
