@@ -17,6 +17,8 @@
 // Deterministic mode reuses the records and replaces the three accumulating kernels by owner-computes kernels whose
 // order of additions is fixed (see below). Small problems, very deep trees and very wide inputs use a single fused
 // kernel with global atomics instead.
+#include <type_traits>
+
 #include "forest_tile.hpp"
 #include "lds_accumulate.hpp"
 
@@ -155,6 +157,113 @@ int dispatch_records(const ForestDims &d, const Real *x, const Node<Real> *nodes
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// fixed-point accumulation (deterministic mode)
+// ---------------------------------------------------------------------------------------------------------------
+// Integer addition is associative, so sums kept as 64-bit integers do not depend on the order in which the hardware
+// applies the atomics: the accumulating kernels below run unchanged, massively parallel, and are still bit
+// reproducible. Each term is scaled by a power of two 2^k and rounded to an integer once; k is chosen on the device from
+// a bound on the largest term and the largest number of terms a cell can receive so that no sum can overflow:
+//   dW terms   |margin| * g   bound max|margin| * max|g|, at most S terms per cell
+//   dThr / dX  c              bound max|c| (measured),    at most max(S, T) terms per cell
+// which leaves >= 61 - ceil(log2(count)) bits below the largest term (an fp32 running sum keeps 24). Non-finite
+// bounds (inf / NaN in the inputs) cannot be represented: the header then routes the affected gradients to the
+// sequential owner-computes kernels further down, on the device, without a host round trip.
+struct DetHeader {
+  unsigned long long max_g, max_a, max_c;  // bit patterns of non-negative doubles (ordered like the values)
+  double scale_w, inv_scale_w, scale_c, inv_scale_c;
+  int fallback_w, fallback_c;
+};
+constexpr size_t kDetHeaderBytes = 256;
+
+__global__ void det_init_kernel(DetHeader *h) {
+  if (threadIdx.x == 0) {
+    h->max_g = h->max_a = h->max_c = 0ull;
+    h->scale_w = h->inv_scale_w = h->scale_c = h->inv_scale_c = 1.0;
+    h->fallback_w = h->fallback_c = 0;
+  }
+}
+
+// max |p[i]| (NaN counts as +inf) folded into *slot.
+template <typename Real>
+__global__ __launch_bounds__(256) void absmax_kernel(const Real *__restrict__ p, long long n,
+                                                     unsigned long long *slot) {
+  constexpr int VEC = 16 / sizeof(Real);
+  typedef Real Vec __attribute__((ext_vector_type(VEC)));
+  double m = 0.0;
+  auto take = [&](Real r) {
+    const double v = fabs(double(r));
+    if (!(v <= m)) m = (v != v) ? double(INFINITY) : v;
+  };
+  const long long tid = (long long)blockIdx.x * 256 + threadIdx.x, nthreads = (long long)gridDim.x * 256;
+  long long body = 0;
+  if (reinterpret_cast<uintptr_t>(p) % 16 == 0) {
+    body = n / VEC;
+    const Vec *pv = reinterpret_cast<const Vec *>(p);
+    for (long long i = tid; i < body; i += nthreads) {
+      const Vec v = __builtin_nontemporal_load(pv + i);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) take(v[e]);
+    }
+    body *= VEC;
+  }
+  for (long long i = body + tid; i < n; i += nthreads) take(p[i]);
+  for (int off = 32; off > 0; off >>= 1) {
+    const double o = __shfl_xor(m, off, kWave);
+    if (!(o <= m)) m = o;
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0 && m > 0.0) atomicMax(slot, (unsigned long long)__double_as_longlong(m));
+}
+
+__device__ inline void det_pick_scale(double bound, double count, double *scale, double *inv, int *fallback) {
+  if (!(bound < double(INFINITY))) {
+    *fallback = 1;
+    *scale = *inv = 0.0;
+    return;
+  }
+  *fallback = 0;
+  if (bound == 0.0) {
+    *scale = *inv = 1.0;
+    return;
+  }
+  int e;
+  frexp(bound, &e);  // bound < 2^e
+  int bits = 0;
+  while (ldexp(1.0, bits) < count) ++bits;
+  // a product rounded to Real can exceed the bound by an ulp: 61, not 62, keeps every sum inside int64
+  int k = 61 - e - bits;
+  k = k > 1000 ? 1000 : (k < -1000 ? -1000 : k);
+  *scale = ldexp(1.0, k);
+  *inv = ldexp(1.0, -k);
+}
+
+__global__ void det_scale_kernel(DetHeader *h, int which, double count) {
+  if (threadIdx.x != 0) return;
+  if (which == 0)
+    det_pick_scale(__longlong_as_double((long long)h->max_g) * __longlong_as_double((long long)h->max_a), count,
+                   &h->scale_w, &h->inv_scale_w, &h->fallback_w);
+  else
+    det_pick_scale(__longlong_as_double((long long)h->max_c), count, &h->scale_c, &h->inv_scale_c, &h->fallback_c);
+}
+
+__device__ __forceinline__ unsigned long long to_fixed(double v, double scale) {
+  return (unsigned long long)__double2ll_rn(v * scale);
+}
+template <typename Real>
+__device__ __forceinline__ Real from_fixed(unsigned long long q, double inv) {
+  return Real(double((long long)q) * inv);
+}
+
+// out[i] = fixed[i] / scale (skipped when the header routed this gradient to the sequential kernels).
+template <typename Real>
+__global__ __launch_bounds__(256) void fixed_to_real_kernel(const unsigned long long *__restrict__ src, Real *dst,
+                                                            long long n, const DetHeader *h, int which) {
+  if (which == 0 ? h->fallback_w : h->fallback_c) return;
+  const double inv = which == 0 ? h->inv_scale_w : h->inv_scale_c;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    dst[i] = from_fixed<Real>(src[i], inv);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // tree-stationary dW + c
 // ---------------------------------------------------------------------------------------------------------------
 // grid = (tree groups, sample parts). Workgroup (g, p) owns trees [g*TB, g*TB + TB) and the samples of part p.
@@ -168,15 +277,27 @@ int dispatch_records(const ForestDims &d, const Real *x, const Node<Real> *nodes
 // of g and w is requested by exactly one load instruction (a thread-per-sample layout re-requests each line once per
 // vector it takes out of it, and the L2 -> L1 traffic of those repeats dominated the kernel). c is reduced over the
 // P lanes with shuffles.
-template <typename Real, int VW, bool COMPACT>
+//
+// FIXED (deterministic mode): the accumulators are 64-bit fixed point (see above); partial sums of sample parts are
+// merged with integer atomics into dw_fixed and converted by fixed_to_real_kernel.
+template <typename Real, int VW, bool COMPACT, bool FIXED>
 __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, const Real *__restrict__ w,
                                                               const Real *__restrict__ gout,
-                                                              Records<Real, COMPACT> rec, Real *dw, int TB,
-                                                              long long part_size, bool need_c, bool dw_atomic, int P,
-                                                              FastDiv div_p, int num_groups) {
+                                                              Records<Real, COMPACT> rec, Real *dw,
+                                                              unsigned long long *dw_fixed, const DetHeader *hdr,
+                                                              int TB, long long part_size, bool need_c,
+                                                              bool dw_atomic, int P, FastDiv div_p, int num_groups) {
   typedef Real Vec __attribute__((ext_vector_type(VW)));
+  typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
   extern __shared__ __align__(16) unsigned char smem[];
-  double *acc = reinterpret_cast<double *>(smem);
+  Acc *acc = reinterpret_cast<Acc *>(smem);
+  double scale = 1.0, inv_scale = 1.0;
+  if (FIXED) {
+    if (hdr->fallback_w) dw = nullptr;
+    scale = hdr->scale_w;
+    inv_scale = hdr->inv_scale_w;
+    if (!dw && !need_c) return;
+  }
   // Workgroups are dealt to the 8 XCDs round robin by index, and each XCD has its own L2. Adjacent tree groups read
   // adjacent pieces of the same 128-byte lines of the upstream gradient, so they are placed on the same XCD (group =
   // (index mod 8) * groups_per_xcd + index / 8): the line is then fetched from memory once instead of once per XCD.
@@ -187,7 +308,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
   const int nt = min(TB, d.T - t0);
   const long long LM = (long long)d.L * d.M;
   if (dw) {
-    for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) acc[i] = 0.0;
+    for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) acc[i] = Acc(0);
     __syncthreads();
   }
   const long long s_begin = (long long)blockIdx.y * part_size;
@@ -252,9 +373,14 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
     for (int u = 0; u < kTreeSteps; ++u) {
       if (dw && on[u]) {
         const Real a = ht_abs(mg[u]);
-        double *cell = acc + (long long)tq[u] * LM + (long long)key[u] * d.M + pl * VW;
+        Acc *cell = acc + (long long)tq[u] * LM + (long long)key[u] * d.M + pl * VW;
 #pragma unroll
-        for (int i = 0; i < VW; ++i) atomicAdd(cell + i, double(a * gv[u][i]));
+        for (int i = 0; i < VW; ++i) {
+          if (FIXED)
+            atomicAdd(reinterpret_cast<unsigned long long *>(cell) + i, to_fixed(double(a * gv[u][i]), scale));
+          else
+            atomicAdd(reinterpret_cast<double *>(cell) + i, double(a * gv[u][i]));
+        }
       }
       if (need_c) {
         Real partial = Real(0);
@@ -278,50 +404,91 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
   if (dw) {
     __syncthreads();
     Real *dst = dw + (long long)t0 * LM;
-    if (dw_atomic) {
-      for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads)
-        if (acc[i] != 0.0) atomicAdd(dst + i, Real(acc[i]));
+    if (FIXED) {
+      const unsigned long long *q = reinterpret_cast<const unsigned long long *>(acc);
+      if (dw_atomic) {
+        for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads)
+          if (q[i] != 0ull) atomicAdd(dw_fixed + (long long)t0 * LM + i, q[i]);
+      } else {
+        for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) dst[i] = from_fixed<Real>(q[i], inv_scale);
+      }
     } else {
-      for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) dst[i] = Real(acc[i]);
+      const double *q = reinterpret_cast<const double *>(acc);
+      if (dw_atomic) {
+        for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads)
+          if (q[i] != 0.0) atomicAdd(dst + i, Real(q[i]));
+      } else {
+        for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) dst[i] = Real(q[i]);
+      }
     }
   }
 }
 
 // dThr[t, v] = sum over samples with selected vertex v of -c. One workgroup per tree (x sample parts).
-template <typename Real, bool COMPACT>
+template <typename Real, bool COMPACT, bool FIXED>
 __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dthr,
+                                                   unsigned long long *dthr_fixed, const DetHeader *hdr,
                                                    long long part_size, bool use_atomic) {
+  typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
   extern __shared__ __align__(16) unsigned char smem[];
-  double *acc = reinterpret_cast<double *>(smem);  // fp64: fast LDS atomic, and the root vertex is a hot spot
+  Acc *acc = reinterpret_cast<Acc *>(smem);  // fp64 / int64: fast LDS atomics, and the root vertex is a hot spot
+  double scale = 1.0, inv_scale = 1.0;
+  if (FIXED) {
+    if (hdr->fallback_c) return;
+    scale = hdr->scale_c;
+    inv_scale = hdr->inv_scale_c;
+  }
   const int t = blockIdx.x;
-  for (int i = threadIdx.x; i < d.V; i += 256) acc[i] = 0.0;
+  for (int i = threadIdx.x; i < d.V; i += 256) acc[i] = Acc(0);
   __syncthreads();
   const long long s_begin = (long long)blockIdx.y * part_size;
   const long long s_end = min(d.S, s_begin + part_size);
   for (long long s = s_begin + threadIdx.x; s < s_end; s += 256) {
     const long long at = (long long)t * d.S + s;
-    atomicAdd(acc + rec.vertex(at), -double(rec.c[at]));
+    if (FIXED)
+      atomicAdd(reinterpret_cast<unsigned long long *>(acc) + rec.vertex(at), to_fixed(-double(rec.c[at]), scale));
+    else
+      atomicAdd(reinterpret_cast<double *>(acc) + rec.vertex(at), -double(rec.c[at]));
   }
   __syncthreads();
   Real *dst = dthr + (long long)t * d.V;
   for (int i = threadIdx.x; i < d.V; i += 256) {
-    if (use_atomic) {
-      if (acc[i] != 0.0) atomicAdd(dst + i, Real(acc[i]));
+    if (FIXED) {
+      const unsigned long long q = reinterpret_cast<const unsigned long long *>(acc)[i];
+      if (use_atomic) {
+        if (q != 0ull) atomicAdd(dthr_fixed + (long long)t * d.V + i, q);
+      } else {
+        dst[i] = from_fixed<Real>(q, inv_scale);
+      }
     } else {
-      dst[i] = Real(acc[i]);
+      const double q = reinterpret_cast<const double *>(acc)[i];
+      if (use_atomic) {
+        if (q != 0.0) atomicAdd(dst + i, Real(q));
+      } else {
+        dst[i] = Real(q);
+      }
     }
   }
 }
 
 // dX: sample tile x all trees. LDS accumulator [F][BT+1] (the pad keeps the transposing write-out conflict free).
-template <typename Real, int BT, bool COMPACT>
-__global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dx) {
+// FIXED: 64-bit fixed-point cells; dX is cleared beforehand and left alone when the header asks for the fallback.
+template <typename Real, int BT, bool COMPACT, bool FIXED>
+__global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dx,
+                                                            const DetHeader *hdr) {
+  typedef typename std::conditional<FIXED, unsigned long long, Real>::type Acc;
   constexpr int NT = kForestThreads;
   constexpr int TC = NT / BT;
   constexpr int LD = BT + 1;
   extern __shared__ __align__(16) unsigned char smem[];
-  Real *acc = reinterpret_cast<Real *>(smem);
-  for (int i = threadIdx.x; i < d.F * LD; i += NT) acc[i] = Real(0);
+  Acc *acc = reinterpret_cast<Acc *>(smem);
+  double scale = 1.0, inv_scale = 1.0;
+  if (FIXED) {
+    if (hdr->fallback_c) return;
+    scale = hdr->scale_c;
+    inv_scale = hdr->inv_scale_c;
+  }
+  for (int i = threadIdx.x; i < d.F * LD; i += NT) acc[i] = Acc(0);
   __syncthreads();
   const long long s0 = (long long)blockIdx.x * BT;
   const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
@@ -329,23 +496,31 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
   if (s < d.S) {
     for (int t = tt; t < d.T; t += TC) {
       const long long at = (long long)t * d.S + s;
-      lds_add(acc + rec.ord(at) * LD + j, rec.c[at]);
+      if (FIXED)
+        atomicAdd(reinterpret_cast<unsigned long long *>(acc) + rec.ord(at) * LD + j,
+                  to_fixed(double(rec.c[at]), scale));
+      else
+        lds_add(reinterpret_cast<Real *>(acc) + rec.ord(at) * LD + j, rec.c[at]);
     }
   }
   __syncthreads();
+  auto cell = [&](int f, int jj) -> Real {
+    if (FIXED) return from_fixed<Real>(reinterpret_cast<const unsigned long long *>(acc)[f * LD + jj], inv_scale);
+    return reinterpret_cast<const Real *>(acc)[f * LD + jj];
+  };
   if (d.K == 1) {
     // dx[s, 0..F) is a contiguous row: a wavefront per sample, lanes along the features
     const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
     for (int jj = wv; jj < BT && s0 + jj < d.S; jj += NT / kWave) {
       Real *row = dx + (s0 + jj) * d.F;
-      for (int f = lane; f < d.F; f += kWave) row[f] = acc[f * LD + jj];
+      for (int f = lane; f < d.F; f += kWave) row[f] = cell(f, jj);
     }
   } else {
     // dx[b, f, k]: consecutive samples of a tile are consecutive k (within one b)
     for (int i = threadIdx.x; i < d.F * BT; i += NT) {
       const int f = i / BT, jj = i - f * BT;
       const long long ss = s0 + jj;
-      if (ss < d.S) dx[(ss / d.K) * d.FK + (long long)f * d.K + (ss % d.K)] = acc[f * LD + jj];
+      if (ss < d.S) dx[(ss / d.K) * d.FK + (long long)f * d.K + (ss % d.K)] = cell(f, jj);
     }
   }
 }
@@ -469,7 +644,8 @@ int dispatch_backward_fused(const ForestDims &d, const Real *x, const Node<Real>
 template <typename Real, bool COMPACT>
 __global__ __launch_bounds__(256) void det_dx_kernel(ForestDims d, const Real *__restrict__ w,
                                                      const Real *__restrict__ gout, Records<Real, COMPACT> rec,
-                                                     Real *dx) {
+                                                     Real *dx, const int *run_if) {
+  if (run_if && *run_if == 0) return;
   const long long s = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (s >= d.S) return;
   const long long b = s / d.K, k = s % d.K;
@@ -515,8 +691,9 @@ __device__ __forceinline__ void ordered_add(Real *p, Real v) {
 template <typename Real, bool LDS_ACC, bool COMPACT>
 __global__ __launch_bounds__(kWave) void det_tree_kernel(ForestDims d, const Real *__restrict__ w,
                                                          const Real *__restrict__ gout, Records<Real, COMPACT> rec,
-                                                         Real *dthr, Real *dw) {
+                                                         Real *dthr, Real *dw, const int *run_if) {
   extern __shared__ __align__(16) unsigned char smem[];
+  if (run_if && *run_if == 0) return;
   const int t = blockIdx.x;
   const int lane = threadIdx.x;
   const long long nW = (long long)d.L * d.M;
@@ -604,11 +781,9 @@ struct TreePlan {
   int groups, parts;    // grid
   long long part_size;  // samples per part
   size_t lds;
-  int vw;               // vector width of the g / w loads
 };
 
-template <typename Real>
-bool plan_trees(const ForestDims &d, bool need_dw, const Real *w, const Real *gout, TreePlan *p) {
+static bool plan_trees(const ForestDims &d, bool need_dw, TreePlan *p) {
   const size_t per_tree = size_t(d.L) * d.M * sizeof(double);
   int tb = 4;
   if (need_dw) {
@@ -629,110 +804,239 @@ bool plan_trees(const ForestDims &d, bool need_dw, const Real *w, const Real *go
   p->part_size = (d.S + parts - 1) / parts;
   p->parts = int((d.S + p->part_size - 1) / p->part_size);
   p->lds = need_dw ? size_t(tb) * per_tree : 0;
-  const size_t vbytes2 = 2 * sizeof(Real), vbytes4 = 4 * sizeof(Real);
-  const uintptr_t pw = reinterpret_cast<uintptr_t>(w), pg = reinterpret_cast<uintptr_t>(gout);
-  p->vw = 1;
-  if (d.M % 2 == 0 && pw % vbytes2 == 0 && pg % vbytes2 == 0) p->vw = 2;
-  if (d.M % 4 == 0 && pw % vbytes4 == 0 && pg % vbytes4 == 0) p->vw = 4;
   return true;
 }
 
-template <typename Real, int VW, bool COMPACT>
+// Vector width of the g / w loads of the tree kernel.
+template <typename Real>
+int pick_vw(const ForestDims &d, const Real *w, const Real *gout) {
+  const size_t vbytes2 = 2 * sizeof(Real), vbytes4 = 4 * sizeof(Real);
+  const uintptr_t pw = reinterpret_cast<uintptr_t>(w), pg = reinterpret_cast<uintptr_t>(gout);
+  if (d.M % 4 == 0 && pw % vbytes4 == 0 && pg % vbytes4 == 0) return 4;
+  if (d.M % 2 == 0 && pw % vbytes2 == 0 && pg % vbytes2 == 0) return 2;
+  return 1;
+}
+
+// Sample parts of the dThr kernel: one workgroup per tree unless the trees alone cannot fill the device.
+static void plan_dthr(const ForestDims &d, long long *part_size, int *gy) {
+  long long parts = d.T >= 2 * kNumCUs ? 1 : (2 * kNumCUs + d.T - 1) / d.T;
+  const long long max_parts = (d.S + 1023) / 1024;
+  if (parts > max_parts) parts = max_parts;
+  if (parts < 1) parts = 1;
+  if (parts > 65535) parts = 65535;
+  *part_size = (d.S + parts - 1) / parts;
+  *gy = int((d.S + *part_size - 1) / *part_size);
+}
+
+template <typename Real, int VW, bool COMPACT, bool FIXED>
 int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, const Real *gout,
-                       Records<Real, COMPACT> rec, Real *dw, bool need_c, hipStream_t stream) {
-  auto kernel = tree_kernel<Real, VW, COMPACT>;
+                       Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
+                       bool need_c, hipStream_t stream) {
+  auto kernel = tree_kernel<Real, VW, COMPACT, FIXED>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(p.lds)));
   const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
   hipLaunchKernelGGL(kernel, dim3((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts), dim3(kForestThreads), p.lds,
-                     stream, d, w, gout, rec, dw, p.TB, p.part_size, need_c, p.parts > 1, d.M / VW,
+                     stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB, p.part_size, need_c, p.parts > 1, d.M / VW,
                      FastDiv(d.M / VW), p.groups);
   HT_LAUNCH_CHECK("forest backward (trees)");
   return HT_OK;
 }
 
-template <typename Real, int BT, bool COMPACT>
-int launch_dx(const ForestDims &d, Records<Real, COMPACT> rec, Real *dx, hipStream_t stream) {
-  const size_t lds = size_t(d.F) * (BT + 1) * sizeof(Real);
+template <typename Real, int BT, bool COMPACT, bool FIXED>
+int launch_dx(const ForestDims &d, Records<Real, COMPACT> rec, Real *dx, const DetHeader *hdr, hipStream_t stream) {
+  const size_t lds = size_t(d.F) * (BT + 1) * (FIXED ? sizeof(unsigned long long) : sizeof(Real));
   const long long tiles = (d.S + BT - 1) / BT;
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
-  auto kernel = dx_kernel<Real, BT, COMPACT>;
+  auto kernel = dx_kernel<Real, BT, COMPACT, FIXED>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kForestThreads), lds, stream, d, rec, dx);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kForestThreads), lds, stream, d, rec, dx, hdr);
   HT_LAUNCH_CHECK("forest backward (dX)");
   return HT_OK;
 }
 
-// Largest dX tile whose padded [F][BT+1] accumulator fits LDS; 0 if none.
-template <typename Real>
-int pick_dx_tile(int F) {
+// Largest dX tile whose padded [F][BT+1] accumulator of `cell`-byte cells fits LDS; 0 if none.
+static int pick_dx_tile(int F, size_t cell) {
   const int candidates[4] = {64, 32, 16, 8};
   for (int bt : candidates)
-    if (size_t(F) * (bt + 1) * sizeof(Real) <= size_t(kLdsBytes)) return bt;
+    if (size_t(F) * (bt + 1) * cell <= size_t(kLdsBytes)) return bt;
   return 0;
 }
 
 template <typename Real>
-bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw) {
+bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw, bool fixed) {
   if (d.M < 1) return false;
   if (d.M > kWave) return false;  // the lanes serving one (sample, tree) pair must fit a wavefront
   if (need_dw && size_t(d.L) * d.M * sizeof(double) > size_t(kLdsBytes)) return false;
   if (size_t(d.V) * sizeof(double) > size_t(kLdsBytes)) return false;
-  if (need_dx && pick_dx_tile<Real>(d.F) == 0) return false;
+  if (need_dx && pick_dx_tile(d.F, fixed ? sizeof(unsigned long long) : sizeof(Real)) == 0) return false;
   return true;
 }
 
 // Problems this small finish sooner in the single fused kernel than in four launches.
 static bool prefer_fused(const ForestDims &d) { return double(d.S) * double(d.T) < double(1 << 18); }
 
-template <typename Real, bool FERN, bool COMPACT>
+// Extra workspace of the fixed-point deterministic pass behind the records: header, then the integer dW and dThr
+// buffers that merge sample parts (present only when the respective kernel splits the samples).
+struct FixedLayout {
+  size_t header, dw, dthr, total;
+};
+static FixedLayout fixed_layout(const ForestDims &d, bool need_dthr, bool need_dw) {
+  FixedLayout l{};
+  TreePlan plan;
+  l.header = 0;
+  size_t at = kDetHeaderBytes;
+  l.dw = at;
+  if (need_dw && plan_trees(d, true, &plan) && plan.parts > 1) at += align_up(size_t(d.T) * d.L * d.M * 8, 256);
+  l.dthr = at;
+  long long part_size;
+  int gy;
+  plan_dthr(d, &part_size, &gy);
+  if (need_dthr && gy > 1) at += align_up(size_t(d.T) * d.V * 8, 256);
+  l.total = at;
+  return l;
+}
+
+template <typename Real>
+int launch_absmax(const Real *p, long long n, unsigned long long *slot, hipStream_t stream) {
+  if (n <= 0) return HT_OK;
+  long long blocks = (n / (16 / (long long)sizeof(Real)) + 255) / 256;
+  if (blocks > 8 * kNumCUs) blocks = 8 * kNumCUs;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL((absmax_kernel<Real>), dim3((unsigned)blocks), dim3(256), 0, stream, p, n, slot);
+  HT_LAUNCH_CHECK("forest backward (magnitude bound)");
+  return HT_OK;
+}
+
+// Staged pipeline. FIXED selects the bit-reproducible fixed-point accumulators; fixed_ws then points at the
+// FixedLayout area and dX must have been cleared by the caller.
+template <typename Real, bool FERN, bool COMPACT, bool FIXED>
 int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, const Real *gout,
-                    Real *dx, Real *dthr, Real *dw, void *rec_ws, hipStream_t stream) {
+                    Real *dx, Real *dthr, Real *dw, void *rec_ws, void *fixed_ws, hipStream_t stream) {
   Records<Real, COMPACT> rec = carve_records<Real, COMPACT>(d, rec_ws);
   int rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream);
   if (rc != HT_OK) return rc;
   const bool need_c = dx || dthr;
+  const long long pairs = (long long)d.T * d.S;
   TreePlan plan;
-  if (!plan_trees<Real>(d, dw != nullptr, w, gout, &plan)) return fail(HT_ERR_RUNTIME, "Error: leaf table too large.");
-  switch (plan.vw) {
-    case 4: rc = launch_tree_kernel<Real, 4, COMPACT>(d, plan, w, gout, rec, dw, need_c, stream); break;
-    case 2: rc = launch_tree_kernel<Real, 2, COMPACT>(d, plan, w, gout, rec, dw, need_c, stream); break;
-    default: rc = launch_tree_kernel<Real, 1, COMPACT>(d, plan, w, gout, rec, dw, need_c, stream); break;
+  if (!plan_trees(d, dw != nullptr, &plan)) return fail(HT_ERR_RUNTIME, "Error: leaf table too large.");
+  long long dthr_part;
+  int dthr_gy;
+  plan_dthr(d, &dthr_part, &dthr_gy);
+
+  DetHeader *hdr = nullptr;
+  unsigned long long *dw_fixed = nullptr, *dthr_fixed = nullptr;
+  if (FIXED) {
+    const FixedLayout lay = fixed_layout(d, dthr != nullptr, dw != nullptr);
+    unsigned char *base = static_cast<unsigned char *>(fixed_ws);
+    hdr = reinterpret_cast<DetHeader *>(base + lay.header);
+    dw_fixed = reinterpret_cast<unsigned long long *>(base + lay.dw);
+    dthr_fixed = reinterpret_cast<unsigned long long *>(base + lay.dthr);
+    hipLaunchKernelGGL(det_init_kernel, dim3(1), dim3(kWave), 0, stream, hdr);
+    HT_LAUNCH_CHECK("forest backward (deterministic header)");
+    if (dw) {
+      if ((rc = launch_absmax<Real>(gout, pairs * d.M, &hdr->max_g, stream)) != HT_OK) return rc;
+      if ((rc = launch_absmax<Real>(rec.margin, pairs, &hdr->max_a, stream)) != HT_OK) return rc;
+      hipLaunchKernelGGL(det_scale_kernel, dim3(1), dim3(kWave), 0, stream, hdr, 0, double(d.S));
+      HT_LAUNCH_CHECK("forest backward (dW scale)");
+      if (plan.parts > 1 && (rc = zero_fill(dw_fixed, size_t(d.T) * d.L * d.M * 8, stream)) != HT_OK) return rc;
+    }
+    if (dthr && dthr_gy > 1 && (rc = zero_fill(dthr_fixed, size_t(d.T) * d.V * 8, stream)) != HT_OK) return rc;
+  }
+
+  switch (pick_vw<Real>(d, w, gout)) {
+    case 4:
+      rc = launch_tree_kernel<Real, 4, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
+      break;
+    case 2:
+      rc = launch_tree_kernel<Real, 2, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
+      break;
+    default:
+      rc = launch_tree_kernel<Real, 1, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
+      break;
   }
   if (rc != HT_OK) return rc;
+
+  if (FIXED) {
+    if (dw) {
+      if (plan.parts > 1) {
+        const long long n = (long long)d.T * d.L * d.M;
+        hipLaunchKernelGGL((fixed_to_real_kernel<Real>), dim3((unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096)),
+                           dim3(256), 0, stream, dw_fixed, dw, n, hdr, 0);
+        HT_LAUNCH_CHECK("forest backward (dW conversion)");
+      }
+      // non-finite magnitudes: dW by the sequential kernel instead (it does nothing unless the header says so)
+      const size_t need = size_t(d.L) * d.M * sizeof(Real);
+      if (need <= size_t(kLdsBytes) / 3) {
+        auto kernel = det_tree_kernel<Real, true, COMPACT>;
+        HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(need)));
+        hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, (Real *)nullptr,
+                           dw, &hdr->fallback_w);
+      } else {
+        hipLaunchKernelGGL((det_tree_kernel<Real, false, COMPACT>), dim3((unsigned)d.T), dim3(kWave), 0, stream, d,
+                           w, gout, rec, (Real *)nullptr, dw, &hdr->fallback_w);
+      }
+      HT_LAUNCH_CHECK("forest backward (dW fallback)");
+    }
+    if (need_c) {
+      if ((rc = launch_absmax<Real>(rec.c, pairs, &hdr->max_c, stream)) != HT_OK) return rc;
+      hipLaunchKernelGGL(det_scale_kernel, dim3(1), dim3(kWave), 0, stream, hdr, 1,
+                         double(d.S > d.T ? d.S : (long long)d.T));
+      HT_LAUNCH_CHECK("forest backward (c scale)");
+    }
+  }
+
   if (dthr) {
-    long long parts = d.T >= 2 * kNumCUs ? 1 : (2 * kNumCUs + d.T - 1) / d.T;
-    const long long max_parts = (d.S + 1023) / 1024;
-    if (parts > max_parts) parts = max_parts;
-    if (parts < 1) parts = 1;
-    if (parts > 65535) parts = 65535;
-    const long long part_size = (d.S + parts - 1) / parts;
-    const int gy = int((d.S + part_size - 1) / part_size);
-    hipLaunchKernelGGL((dthr_kernel<Real, COMPACT>), dim3((unsigned)d.T, (unsigned)gy), dim3(256),
-                       size_t(d.V) * sizeof(double), stream, d, rec, dthr, part_size, gy > 1);
+    hipLaunchKernelGGL((dthr_kernel<Real, COMPACT, FIXED>), dim3((unsigned)d.T, (unsigned)dthr_gy), dim3(256),
+                       size_t(d.V) * sizeof(double), stream, d, rec, dthr, dthr_fixed, hdr, dthr_part, dthr_gy > 1);
     HT_LAUNCH_CHECK("forest backward (dThr)");
+    if (FIXED) {
+      if (dthr_gy > 1) {
+        const long long n = (long long)d.T * d.V;
+        hipLaunchKernelGGL((fixed_to_real_kernel<Real>), dim3((unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096)),
+                           dim3(256), 0, stream, dthr_fixed, dthr, n, hdr, 1);
+        HT_LAUNCH_CHECK("forest backward (dThr conversion)");
+      }
+      const size_t need = size_t(d.V) * sizeof(Real);
+      auto kernel = det_tree_kernel<Real, true, COMPACT>;
+      HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(need)));
+      hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, dthr,
+                         (Real *)nullptr, &hdr->fallback_c);
+      HT_LAUNCH_CHECK("forest backward (dThr fallback)");
+    }
   }
   if (dx) {
-    switch (pick_dx_tile<Real>(d.F)) {
-      case 64: rc = launch_dx<Real, 64, COMPACT>(d, rec, dx, stream); break;
-      case 32: rc = launch_dx<Real, 32, COMPACT>(d, rec, dx, stream); break;
-      case 16: rc = launch_dx<Real, 16, COMPACT>(d, rec, dx, stream); break;
-      default: rc = launch_dx<Real, 8, COMPACT>(d, rec, dx, stream); break;
+    switch (pick_dx_tile(d.F, FIXED ? sizeof(unsigned long long) : sizeof(Real))) {
+      case 64: rc = launch_dx<Real, 64, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
+      case 32: rc = launch_dx<Real, 32, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
+      case 16: rc = launch_dx<Real, 16, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
+      default: rc = launch_dx<Real, 8, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
+    }
+    if (rc != HT_OK) return rc;
+    if (FIXED) {
+      const long long blocks = (d.S + 255) / 256;
+      hipLaunchKernelGGL((det_dx_kernel<Real, COMPACT>), dim3((unsigned)blocks), dim3(256), 0, stream, d, w, gout,
+                         rec, dx, &hdr->fallback_c);
+      HT_LAUNCH_CHECK("forest backward (dX fallback)");
     }
   }
   return rc;
 }
 
+// Sequential owner-computes pass for shapes whose accumulators do not fit LDS.
 template <typename Real, bool FERN, bool COMPACT>
-int backward_deterministic(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w,
-                           const Real *gout, Real *dx, Real *dthr, Real *dw, void *rec_ws, hipStream_t stream) {
+int backward_sequential(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w,
+                        const Real *gout, Real *dx, Real *dthr, Real *dw, void *rec_ws, hipStream_t stream) {
   Records<Real, COMPACT> rec = carve_records<Real, COMPACT>(d, rec_ws);
   int rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream);
   if (rc != HT_OK) return rc;
   if (dx) {
     const long long blocks = (d.S + 255) / 256;
-    hipLaunchKernelGGL((det_dx_kernel<Real, COMPACT>), dim3((unsigned)blocks), dim3(256), 0, stream, d, w, gout, rec, dx);
+    hipLaunchKernelGGL((det_dx_kernel<Real, COMPACT>), dim3((unsigned)blocks), dim3(256), 0, stream, d, w, gout, rec,
+                       dx, (const int *)nullptr);
     HT_LAUNCH_CHECK("deterministic dX");
   }
   if (dthr || dw) {
@@ -741,10 +1045,11 @@ int backward_deterministic(const ForestDims &d, const Real *x, const Node<Real> 
       auto kernel = det_tree_kernel<Real, true, COMPACT>;
       HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, int(need)));
-      hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, dthr, dw);
+      hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, dthr, dw,
+                         (const int *)nullptr);
     } else {
       hipLaunchKernelGGL((det_tree_kernel<Real, false, COMPACT>), dim3((unsigned)d.T), dim3(kWave), 0, stream, d, w,
-                         gout, rec, dthr, dw);
+                         gout, rec, dthr, dw, (const int *)nullptr);
     }
     HT_LAUNCH_CHECK("deterministic dThr/dW");
   }
@@ -756,10 +1061,12 @@ int backward_deterministic(const ForestDims &d, const Real *x, const Node<Real> 
 template <typename Real>
 size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw) {
   size_t bytes = packed_nodes_bytes<Real>(d);
-  const bool staged = mode == HT_BACKWARD_DETERMINISTIC ||
-                      (staged_ok<Real>(d, need_dx, need_dw) && !prefer_fused(d));
-  (void)need_dthr;
-  if (staged) bytes += records_bytes<Real>(d);
+  if (mode == HT_BACKWARD_DETERMINISTIC) {
+    bytes += align_up(records_bytes<Real>(d), 256);
+    if (staged_ok<Real>(d, need_dx, need_dw, true)) bytes += fixed_layout(d, need_dthr, need_dw).total;
+    return bytes;
+  }
+  if (staged_ok<Real>(d, need_dx, need_dw, false) && !prefer_fused(d)) bytes += records_bytes<Real>(d);
   return bytes;
 }
 
@@ -769,7 +1076,8 @@ int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *t
                     hipStream_t stream) {
   int rc;
   const bool det = mode == HT_BACKWARD_DETERMINISTIC;
-  const bool staged = det || (staged_ok<Real>(d, dx != nullptr, dw != nullptr) && !prefer_fused(d));
+  const bool fixed = det && staged_ok<Real>(d, dx != nullptr, dw != nullptr, true);
+  const bool staged = det || (staged_ok<Real>(d, dx != nullptr, dw != nullptr, false) && !prefer_fused(d));
   // The staged dX kernel overwrites every element of dX; everything else accumulates into zeros.
   const bool empty = d.S == 0 || d.T == 0;
   const bool clear_dx = !staged || det || empty;
@@ -778,24 +1086,36 @@ int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *t
   if (dw && (rc = zero_fill(dw, size_t(d.T) * d.L * d.M * sizeof(Real), stream)) != HT_OK) return rc;
   if (empty || (!dx && !dthr && !dw)) return HT_OK;
   const size_t node_bytes = packed_nodes_bytes<Real>(d);
-  const size_t need = node_bytes + (staged ? records_bytes<Real>(d) : 0);
+  const size_t rec_bytes = staged ? align_up(records_bytes<Real>(d), 256) : 0;
+  const size_t need =
+      node_bytes + (det ? rec_bytes : (staged ? records_bytes<Real>(d) : 0)) +
+      (fixed ? fixed_layout(d, dthr != nullptr, dw != nullptr).total : 0);
   if (ws == nullptr || ws_bytes < need)
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the backward pass.");
   if ((rc = pack_nodes<Real>(d, thr, ord, ws, stream)) != HT_OK) return rc;
   const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
   void *rec_ws = static_cast<unsigned char *>(ws) + node_bytes;
+  void *fixed_ws = static_cast<unsigned char *>(rec_ws) + rec_bytes;
   const bool compact = compact_ok(d);
 
-#define HT_CALL(fn, FERN_, COMPACT_) fn<Real, FERN_, COMPACT_>(d, x, nodes, w, gout, dx, dthr, dw, rec_ws, stream)
+#define HT_STAGED(FERN_, COMPACT_, FIXED_) \
+  backward_staged<Real, FERN_, COMPACT_, FIXED_>(d, x, nodes, w, gout, dx, dthr, dw, rec_ws, fixed_ws, stream)
+#define HT_SEQ(FERN_, COMPACT_) \
+  backward_sequential<Real, FERN_, COMPACT_>(d, x, nodes, w, gout, dx, dthr, dw, rec_ws, stream)
+  if (fixed) {
+    if (fern) return compact ? HT_STAGED(true, true, true) : HT_STAGED(true, false, true);
+    return compact ? HT_STAGED(false, true, true) : HT_STAGED(false, false, true);
+  }
   if (det) {
-    if (fern) return compact ? HT_CALL(backward_deterministic, true, true) : HT_CALL(backward_deterministic, true, false);
-    return compact ? HT_CALL(backward_deterministic, false, true) : HT_CALL(backward_deterministic, false, false);
+    if (fern) return compact ? HT_SEQ(true, true) : HT_SEQ(true, false);
+    return compact ? HT_SEQ(false, true) : HT_SEQ(false, false);
   }
   if (staged) {
-    if (fern) return compact ? HT_CALL(backward_staged, true, true) : HT_CALL(backward_staged, true, false);
-    return compact ? HT_CALL(backward_staged, false, true) : HT_CALL(backward_staged, false, false);
+    if (fern) return compact ? HT_STAGED(true, true, false) : HT_STAGED(true, false, false);
+    return compact ? HT_STAGED(false, true, false) : HT_STAGED(false, false, false);
   }
-#undef HT_CALL
+#undef HT_STAGED
+#undef HT_SEQ
   return fern ? dispatch_backward_fused<Real, true>(d, x, nodes, w, gout, dx, dthr, dw, stream)
               : dispatch_backward_fused<Real, false>(d, x, nodes, w, gout, dx, dthr, dw, stream);
 }
