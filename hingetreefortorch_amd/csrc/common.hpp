@@ -47,8 +47,8 @@ constexpr int kNumXCDs = 8;                 // accelerator dies, each with its o
 struct FastDiv {
   uint32_t inv;
   uint32_t d;
-  FastDiv() : inv(0), d(1) {}
-  explicit FastDiv(int divisor) : inv(divisor <= 1 ? 0u : uint32_t(((1ull << 32) + divisor - 1) / divisor)), d(divisor) {}
+  __host__ __device__ FastDiv() : inv(0), d(1) {}
+  __host__ __device__ explicit FastDiv(int divisor) : inv(divisor <= 1 ? 0u : uint32_t(((1ull << 32) + divisor - 1) / divisor)), d(divisor) {}
   __device__ __forceinline__ int div(int n) const { return d <= 1 ? n : int(__umulhi(uint32_t(n), inv)); }
 };
 

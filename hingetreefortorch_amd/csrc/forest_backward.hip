@@ -26,7 +26,6 @@ namespace ht {
 namespace {
 
 constexpr int kIlp = 4;         // trees walked concurrently per thread by the records kernel
-constexpr int kTreeSteps = 4;   // steps of the tree-stationary kernel whose loads are in flight together
 
 // ---------------------------------------------------------------------------------------------------------------
 // walk records
@@ -266,28 +265,52 @@ __global__ __launch_bounds__(256) void fixed_to_real_kernel(const unsigned long 
 // ---------------------------------------------------------------------------------------------------------------
 // tree-stationary dW + c
 // ---------------------------------------------------------------------------------------------------------------
-// grid = (tree groups, sample parts). Workgroup (g, p) owns trees [g*TB, g*TB + TB) and the samples of part p.
-// LDS: dW accumulators [TB][L][M] in fp64 (if dw): the fp64 LDS atomic add is a fast hardware instruction on gfx950,
+// grid = (tree groups, sample parts). Workgroup (g, p) owns trees [g*TB, g*TB + nt) and the samples of part p.
+// LDS: dW accumulators [nt][L][M] in fp64 (if dw): the fp64 LDS atomic add is a fast hardware instruction on gfx950,
 // the fp32 one is not (see lds_accumulate.hpp); each product |margin| * g is still rounded to Real first, only the
 // running sum is wider.
 //
-// A (sample, tree) pair is served by P = M / VW adjacent lanes, lane p holding elements [p*VW, p*VW + VW) of the
-// pair's M upstream-gradient values and of its leaf-weight row; a wavefront serves G = 64 / P pairs per step, pairs
-// enumerated with the tree index fastest so that consecutive pairs read consecutive memory. This way every cache line
-// of g and w is requested by exactly one load instruction (a thread-per-sample layout re-requests each line once per
-// vector it takes out of it, and the L2 -> L1 traffic of those repeats dominated the kernel). c is reduced over the
-// P lanes with shuffles.
+// The kernel is bound by the number of accesses its loads cost in the vector memory pipeline, which handles a load
+// four lanes at a time and charges every distinct line those four lanes touch. So:
+//   * records are loaded one pair per lane, trees in lane blocks (lanes [r*SPT, r*SPT + SPT) hold SPT consecutive
+//     samples of tree r): fully coalesced, one load per 64 pairs; c is stored the same way.
+//   * a pair's M upstream-gradient values and its M leaf weights are each one contiguous run of memory. It is read by
+//     P adjacent lanes (P a power of two, so groups never straddle a quad unless they fill several) with one 16-byte
+//     load per lane; the last lane's chunk is shifted back to end at M, and it owns only the elements past its
+//     neighbour's. Pairs are taken sample major, tree minor, so adjacent lane groups read adjacent memory.
+//   * the record fields travel from the lane that loaded them to the lanes that need them by ds_bpermute.
 //
 // FIXED (deterministic mode): the accumulators are 64-bit fixed point (see above); partial sums of sample parts are
 // merged with integer atomics into dw_fixed and converted by fixed_to_real_kernel.
-template <typename Real, int VW, bool COMPACT, bool FIXED>
+constexpr int kMaxGroupTrees = 16;  // trees per workgroup (so a 64-pair step covers >= 4 consecutive samples per tree)
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_swap(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_swap(double v) {
+  const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, 0xF, 0xF, true);
+  const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, 0xF, 0xF, true);
+  return __hiloint2double(hi, lo);
+}
+// Sum over aligned groups of P adjacent lanes (P a power of two); every lane of a group receives the total.
+template <typename Real>
+__device__ __forceinline__ Real group_sum(Real v, int P) {
+  if (P >= 2) v += dpp_swap<0xB1>(v);  // quad_perm [1,0,3,2]
+  if (P >= 4) v += dpp_swap<0x4E>(v);  // quad_perm [2,3,0,1]
+  for (int off = 4; off < P; off <<= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+template <typename Real, bool COMPACT, bool FIXED, int U>
 __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, const Real *__restrict__ w,
                                                               const Real *__restrict__ gout,
                                                               Records<Real, COMPACT> rec, Real *dw,
                                                               unsigned long long *dw_fixed, const DetHeader *hdr,
                                                               int TB, long long part_size, bool need_c,
-                                                              bool dw_atomic, int P, FastDiv div_p, int num_groups) {
-  typedef Real Vec __attribute__((ext_vector_type(VW)));
+                                                              bool dw_atomic, int P, int num_groups) {
+  constexpr int VE = 16 / sizeof(Real);  // elements per 16-byte chunk
   typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
   extern __shared__ __align__(16) unsigned char smem[];
   Acc *acc = reinterpret_cast<Acc *>(smem);
@@ -313,93 +336,134 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
   }
   const long long s_begin = (long long)blockIdx.y * part_size;
   const long long s_end = min(d.S, s_begin + part_size);
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   constexpr int kWaves = kForestThreads / kWave;
-  const int G = kWave / P;                         // pairs per wavefront step (P <= 64)
-  const int grp = div_p.div(lane), pl = lane - grp * P;
-  const bool lane_on = grp < G;
-  // pair q of this workgroup = (sample s_begin + q / nt, tree t0 + q % nt); a lane's q advances by kWaves * G per step
-  const long long npairs = (s_end - s_begin) * nt;
-  const int step = kWaves * G;
-  // kTreeSteps steps are in flight together: all their record loads are issued first, then all gradient and weight
-  // loads, so that a wavefront always has several independent memory round trips outstanding.
-  int sub_s[kTreeSteps], sub_t[kTreeSteps];
+  const int SPT = kWave / nt;  // samples per tree in one 64-pair block
+  const int NP = kWave / P;    // pairs per sub-step; a block has P sub-steps, taken U at a time (U divides P)
+  const FastDiv div_nt(nt), div_spt(SPT);
+
+  // this lane as a loader of records: tree rt, sample offset rj of the block
+  const int rt = div_spt.div(lane), rj = lane - rt * SPT;
+  const bool rec_lane = rt < nt;
+  // ... and where that pair is processed: sub-step my_sub, lane group my_src / P
+  const int my_pp = rj * nt + rt;
+  const int my_sub = my_pp / NP, my_src = (my_pp - my_sub * NP) * P;
+  // this lane as a member of a lane group.
+  // The M elements are dealt evenly to the P lanes (lane li owns [li*M/P, (li+1)*M/P): at least one, at most VE), so
+  // the LDS atomics -- whose cost is per instruction, not per active lane -- need only ceil(M/P) rounds. A lane loads
+  // the 16-byte chunk that starts at its first element (shifted back where it would pass the end of the row): lanes
+  // with overlapping chunks hit the same line, which costs nothing extra.
+  const int grp = lane / P, li = lane & (P - 1);
+  const int own_begin = li * d.M / P, own_end = (li + 1) * d.M / P;
+  const int e0 = d.M >= VE ? min(own_begin, d.M - VE) : 0;  // first element of this lane's chunk
+  const int own = own_begin - e0;                            // chunk elements [own, own + cnt) belong to this lane
+  const int cnt = own_end - own_begin;
+  const int rounds = (d.M + P - 1) / P;                      // wave uniform: max cnt over the lanes
+
+  auto load_chunk = [&](const Real *p, Real (&v)[VE]) {
+    if (d.M >= VE) {
+      __builtin_memcpy(v, p, sizeof(Real) * VE);  // 16 bytes, element aligned
+    } else {
 #pragma unroll
-  for (int u = 0; u < kTreeSteps; ++u) {
-    sub_s[u] = (u * step) / nt;
-    sub_t[u] = (u * step) - sub_s[u] * nt;
-  }
-  const int big = kTreeSteps * step;
-  const int big_s = big / nt, big_t = big - big_s * nt;
-  long long q = (long long)wave * G + grp;
-  long long sl = q / nt;
-  int tl = int(q - sl * nt);
-  const long long row_stride = (long long)d.T * d.M;  // K == 1: distance between the gradient rows of two samples
-  for (long long q0 = (long long)wave * G; q0 < npairs; q0 += big) {
-    bool on[kTreeSteps];
-    int tq[kTreeSteps];
-    long long at[kTreeSteps], goff[kTreeSteps];
-    uint32_t key[kTreeSteps];
-    Real mg[kTreeSteps];
-#pragma unroll
-    for (int u = 0; u < kTreeSteps; ++u) {
-      int tu = tl + sub_t[u];
-      long long su = sl + sub_s[u];
-      if (tu >= nt) {
-        tu -= nt;
-        ++su;
-      }
-      on[u] = lane_on && q + (long long)u * step < npairs;
-      const long long s = s_begin + (on[u] ? su : 0);
-      tq[u] = on[u] ? tu : 0;
-      const int t = t0 + tq[u];
-      at[u] = (long long)t * d.S + s;
-      if (d.K == 1) {
-        goff[u] = s * row_stride + (long long)t * d.M;
-      } else {
-        const long long b = s / d.K, k = s - b * d.K;
-        goff[u] = ((b * d.T + t) * d.K + k) * d.M;
-      }
-      key[u] = rec.key(at[u]);
-      mg[u] = rec.margin[at[u]];
+      for (int k = 0; k < VE; ++k) v[k] = k < d.M ? p[k] : Real(0);
     }
-    Vec gv[kTreeSteps], wv[kTreeSteps];
+  };
+
+  // The samples of a wavefront form blocks of SPT (x nt trees = up to 64 pairs); a block is worked off in P / U
+  // chunks of U sub-steps. Per chunk the record loads and the gradient loads (whose addresses depend on nothing
+  // loaded) go out together; the weight loads follow when the keys are there. Every load is unconditional, idle lanes
+  // aimed at the block's first pair, which keeps the number of loads in flight at each wait a compile-time constant,
+  // so a wait never covers more than it has to. (Prefetching the next chunk during the arithmetic was measured and
+  // did not pay: the kernel is not latency bound.)
+  struct Chunk {
+    long long at;   // record index of this lane as a loader
+    bool have;      // ... and whether it holds a pair
+    int npairs;
+    uint32_t key_r;
+    Real mg_r;
+    bool on[U];
+    int src[U], tq_of[U];
+    Real gv[U][VE];
+  };
+  const Real *wbase = w + (long long)t0 * LM;
+  const int CPB = P / U;  // chunks per block (a power of two)
+  const long long my_first = s_begin + (long long)wave * SPT;
+  const long long nblk = my_first < s_end ? (s_end - my_first + (long long)kWaves * SPT - 1) / ((long long)kWaves * SPT) : 0;
+  const long long nchunks = nblk * CPB;
+
+  auto prefetch = [&](long long c, Chunk &q) {
+    const long long blk = c / CPB;
+    const int sub0 = int(c - blk * CPB) * U;
+    const long long sblk = my_first + blk * kWaves * SPT;
+    const int ns = int(min<long long>(SPT, s_end - sblk));
+    q.npairs = ns * nt;
+    q.have = rec_lane && rj < ns;
+    q.at = (long long)(t0 + (q.have ? rt : 0)) * d.S + sblk + (q.have ? rj : 0);
+    q.key_r = rec.key(q.at);
+    q.mg_r = rec.margin[q.at];
+    const Real *gbase = gout + (d.K == 1 ? (sblk * d.T + t0) * d.M : 0);
 #pragma unroll
-    for (int u = 0; u < kTreeSteps; ++u) {
-      gv[u] = *reinterpret_cast<const Vec *>(gout + goff[u] + pl * VW);
-      if (need_c) wv[u] = *reinterpret_cast<const Vec *>(w + ((long long)(t0 + tq[u]) * d.L + key[u]) * d.M + pl * VW);
+    for (int u = 0; u < U; ++u) {
+      const int pp = (sub0 + u) * NP + grp;
+      q.on[u] = pp < q.npairs;
+      const int j = q.on[u] ? div_nt.div(pp) : 0;
+      const int tq = q.on[u] ? pp - j * nt : 0;
+      q.src[u] = tq * SPT + j;
+      q.tq_of[u] = tq;
+      if (d.K == 1)
+        load_chunk(gbase + (uint32_t(j) * d.T + tq) * d.M + e0, q.gv[u]);
+      else
+        load_chunk(gout + out_offset(d, sblk + j, t0 + tq, e0), q.gv[u]);
+    }
+  };
+
+  Real c_mine = Real(0);
+  for (long long c = 0; c < nchunks; ++c) {
+    const int sub0 = int(c & (CPB - 1)) * U;
+    Chunk cur;
+    prefetch(c, cur);
+    uint32_t rel[U];
+    Real mg[U];
+    Real wv[U][VE];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t key = __shfl(cur.key_r, cur.src[u], kWave);
+      mg[u] = __shfl(cur.mg_r, cur.src[u], kWave);
+      rel[u] = (uint32_t(cur.tq_of[u]) * d.L + key) * d.M + e0;
+      if (need_c) load_chunk(wbase + rel[u], wv[u]);
     }
 #pragma unroll
-    for (int u = 0; u < kTreeSteps; ++u) {
-      if (dw && on[u]) {
+    for (int u = 0; u < U; ++u) {
+      if (dw && cur.on[u]) {
         const Real a = ht_abs(mg[u]);
-        Acc *cell = acc + (long long)tq[u] * LM + (long long)key[u] * d.M + pl * VW;
+        Acc *cell = acc + rel[u];
 #pragma unroll
-        for (int i = 0; i < VW; ++i) {
-          if (FIXED)
-            atomicAdd(reinterpret_cast<unsigned long long *>(cell) + i, to_fixed(double(a * gv[u][i]), scale));
-          else
-            atomicAdd(reinterpret_cast<double *>(cell) + i, double(a * gv[u][i]));
+        for (int i = 0; i < VE; ++i) {
+          if (i >= rounds) break;  // wave uniform
+          if (i < cnt) {
+            // element own + i of the chunk (own is not a compile-time constant: select, do not index)
+            Real g = cur.gv[u][0];
+#pragma unroll
+            for (int k = 1; k < VE; ++k) g = (own + i == k) ? cur.gv[u][k] : g;
+            if (FIXED)
+              atomicAdd(reinterpret_cast<unsigned long long *>(cell) + own + i, to_fixed(double(a * g), scale));
+            else
+              atomicAdd(reinterpret_cast<double *>(cell) + own + i, double(a * g));
+          }
         }
       }
       if (need_c) {
         Real partial = Real(0);
 #pragma unroll
-        for (int i = 0; i < VW; ++i) partial += wv[u][i] * gv[u][i];
-        for (int off = 1; off < P; off <<= 1) {
-          const Real other = __shfl_down(partial, off, kWave);
-          if (pl + off < P) partial += other;
-        }
-        if (on[u] && pl == 0) rec.c[at[u]] = ht_sign(mg[u]) * partial;
+        for (int k = 0; k < VE; ++k)
+          if (k >= own && k < own + cnt) partial += wv[u][k] * cur.gv[u][k];
+        partial = group_sum<Real>(cur.on[u] ? partial : Real(0), P);
+        const Real got = __shfl(ht_sign(mg[u]) * partial, my_src, kWave);
+        if (my_sub == sub0 + u) c_mine = got;
       }
     }
-    q += big;
-    sl += big_s;
-    tl += big_t;
-    if (tl >= nt) {
-      tl -= nt;
-      ++sl;
-    }
+    if (need_c && sub0 + U == P && cur.have) rec.c[cur.at] = c_mine;
   }
   if (dw) {
     __syncthreads();
@@ -790,6 +854,7 @@ static bool plan_trees(const ForestDims &d, bool need_dw, TreePlan *p) {
     if (per_tree > size_t(kLdsBytes)) return false;
     tb = int(size_t(kLdsBytes) / per_tree);
   }
+  if (tb > kMaxGroupTrees) tb = kMaxGroupTrees;
   if (tb > d.T) tb = d.T;
   // keep at least ~one workgroup per CU by shrinking the groups before splitting the samples
   while (tb > 4 && (d.T + tb - 1) / tb < kNumCUs) tb = (tb + 1) / 2;
@@ -807,16 +872,6 @@ static bool plan_trees(const ForestDims &d, bool need_dw, TreePlan *p) {
   return true;
 }
 
-// Vector width of the g / w loads of the tree kernel.
-template <typename Real>
-int pick_vw(const ForestDims &d, const Real *w, const Real *gout) {
-  const size_t vbytes2 = 2 * sizeof(Real), vbytes4 = 4 * sizeof(Real);
-  const uintptr_t pw = reinterpret_cast<uintptr_t>(w), pg = reinterpret_cast<uintptr_t>(gout);
-  if (d.M % 4 == 0 && pw % vbytes4 == 0 && pg % vbytes4 == 0) return 4;
-  if (d.M % 2 == 0 && pw % vbytes2 == 0 && pg % vbytes2 == 0) return 2;
-  return 1;
-}
-
 // Sample parts of the dThr kernel: one workgroup per tree unless the trees alone cannot fill the device.
 static void plan_dthr(const ForestDims &d, long long *part_size, int *gy) {
   long long parts = d.T >= 2 * kNumCUs ? 1 : (2 * kNumCUs + d.T - 1) / d.T;
@@ -828,19 +883,31 @@ static void plan_dthr(const ForestDims &d, long long *part_size, int *gy) {
   *gy = int((d.S + *part_size - 1) / *part_size);
 }
 
-template <typename Real, int VW, bool COMPACT, bool FIXED>
-int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, const Real *gout,
-                       Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
-                       bool need_c, hipStream_t stream) {
-  auto kernel = tree_kernel<Real, VW, COMPACT, FIXED>;
+template <typename Real, bool COMPACT, bool FIXED, int U>
+int launch_tree_kernel_u(const ForestDims &d, const TreePlan &p, int P, const Real *w, const Real *gout,
+                         Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
+                         bool need_c, hipStream_t stream) {
+  auto kernel = tree_kernel<Real, COMPACT, FIXED, U>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(p.lds)));
   const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
   hipLaunchKernelGGL(kernel, dim3((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts), dim3(kForestThreads), p.lds,
-                     stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB, p.part_size, need_c, p.parts > 1, d.M / VW,
-                     FastDiv(d.M / VW), p.groups);
+                     stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB, p.part_size, need_c, p.parts > 1, P, p.groups);
   HT_LAUNCH_CHECK("forest backward (trees)");
   return HT_OK;
+}
+
+template <typename Real, bool COMPACT, bool FIXED>
+int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, const Real *gout,
+                       Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
+                       bool need_c, hipStream_t stream) {
+  constexpr int VE = 16 / sizeof(Real);
+  const int Q = d.M >= VE ? (d.M + VE - 1) / VE : 1;  // 16-byte chunks in one pair's values
+  int P = 1;                                          // lanes per pair
+  while (P < Q) P <<= 1;
+  if (P >= 4) return launch_tree_kernel_u<Real, COMPACT, FIXED, 4>(d, p, P, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
+  if (P == 2) return launch_tree_kernel_u<Real, COMPACT, FIXED, 2>(d, p, P, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
+  return launch_tree_kernel_u<Real, COMPACT, FIXED, 1>(d, p, P, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
 }
 
 template <typename Real, int BT, bool COMPACT, bool FIXED>
@@ -867,7 +934,10 @@ static int pick_dx_tile(int F, size_t cell) {
 template <typename Real>
 bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw, bool fixed) {
   if (d.M < 1) return false;
-  if (d.M > kWave) return false;  // the lanes serving one (sample, tree) pair must fit a wavefront
+  // the lanes serving one (sample, tree) pair (16 bytes each) must fit a wavefront, and the tree kernel addresses
+  // the gradient rows of one 64-sample step with 32-bit offsets
+  if ((d.M + 16 / int(sizeof(Real)) - 1) / (16 / int(sizeof(Real))) > kWave) return false;
+  if ((long long)d.T * d.M * kWave >= (1ll << 31)) return false;
   if (need_dw && size_t(d.L) * d.M * sizeof(double) > size_t(kLdsBytes)) return false;
   if (size_t(d.V) * sizeof(double) > size_t(kLdsBytes)) return false;
   if (need_dx && pick_dx_tile(d.F, fixed ? sizeof(unsigned long long) : sizeof(Real)) == 0) return false;
@@ -945,17 +1015,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
     if (dthr && dthr_gy > 1 && (rc = zero_fill(dthr_fixed, size_t(d.T) * d.V * 8, stream)) != HT_OK) return rc;
   }
 
-  switch (pick_vw<Real>(d, w, gout)) {
-    case 4:
-      rc = launch_tree_kernel<Real, 4, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
-      break;
-    case 2:
-      rc = launch_tree_kernel<Real, 2, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
-      break;
-    default:
-      rc = launch_tree_kernel<Real, 1, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
-      break;
-  }
+  rc = launch_tree_kernel<Real, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
   if (rc != HT_OK) return rc;
 
   if (FIXED) {

@@ -30,13 +30,12 @@ constexpr int kOutUnroll = 5;  // output vectors per lane whose weight gathers a
 // ILP = trees walked concurrently per thread; KeyT = storage type of the parked leaf keys (uint16_t up to depth 16);
 // VW = outputs per lane in the output phase (divides M): the memory pipeline charges a gather instruction by its
 // lanes, not by the lines it touches, so wider lanes mean proportionally fewer cycles per output.
-template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
-__global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, const Real *__restrict__ x,
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW, int NT>
+__global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *__restrict__ x,
                                                                  const Node<Real> *__restrict__ nodes,
                                                                  const Real *__restrict__ w, Real *__restrict__ out,
                                                                  int trees_per_block, FastDiv div_m) {
   typedef Real Vec __attribute__((ext_vector_type(VW)));
-  constexpr int NT = kForestThreads;
   constexpr int TC = NT / BT;        // tree slots per walk round
   constexpr int kIlp = ILP;
   constexpr int TP = TC * kIlp;      // trees per pass
@@ -85,17 +84,21 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
       // out[s, tb .. tb+nt, 0 .. M) is one contiguous row per sample: a wavefront per row, lanes along the row
       const int row = nt * d.M;
       const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-      for (int jj = wave; jj < BT; jj += NT / kWave) {
+      constexpr int kWaves = NT / kWave;
+      constexpr int WPR = kWaves > BT ? kWaves / BT : 1;  // wavefronts sharing one row
+      constexpr int kStride = WPR * kWave * VW;            // elements between a lane's consecutive vectors
+      const int sub = wave % WPR;
+      for (int jj = wave / WPR; jj < BT; jj += kWaves / WPR) {
         const long long ss = s0 + jj;
         if (ss >= d.S) break;
         Real *orow = out + (ss * d.T + tb) * d.M;
         // kOutUnroll independent leaf-weight gathers are issued before the first store
-        for (int r0 = lane * VW; r0 < row; r0 += kWave * VW * kOutUnroll) {
+        for (int r0 = (sub * kWave + lane) * VW; r0 < row; r0 += kStride * kOutUnroll) {
           Real a[kOutUnroll];
           Vec wv[kOutUnroll];
 #pragma unroll
           for (int u = 0; u < kOutUnroll; ++u) {
-            const int r = min(r0 + u * kWave * VW, row - VW);
+            const int r = min(r0 + u * kStride, row - VW);
             const int t2 = div_m.div(r), m = r - t2 * d.M;
             const uint32_t key = r_key[jj * LDR + t2];
             a[u] = r_abs[jj * LDR + t2];
@@ -103,11 +106,11 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
           }
 #pragma unroll
           for (int u = 0; u < kOutUnroll; ++u) {
-            if (r0 + u * kWave * VW < row) {
+            if (r0 + u * kStride < row) {
               Vec o;
 #pragma unroll
               for (int i = 0; i < VW; ++i) o[i] = a[u] * wv[u][i];
-              *reinterpret_cast<Vec *>(orow + r0 + u * kWave * VW) = o;
+              *reinterpret_cast<Vec *>(orow + r0 + u * kStride) = o;
             }
           }
         }
@@ -129,19 +132,19 @@ __global__ __launch_bounds__(kForestThreads) void forward_kernel(ForestDims d, c
   }
 }
 
-template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW, int NT = kForestThreads>
 int launch_forward_vw(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
                       hipStream_t stream) {
-  constexpr int TP = kForestThreads / BT * ILP;
+  constexpr int TP = NT / BT * ILP;
   const size_t lds = (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TP + 1) * BT * (sizeof(Real) + sizeof(KeyT));
   const long long tiles = (d.S + BT - 1) / BT;
   int trees_per_block, gy;
   split_trees(tiles, d.T, TP, &trees_per_block, &gy);
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
-  auto kernel = forward_kernel<Real, FERN, BT, XLDS, ILP, KeyT, VW>;
+  auto kernel = forward_kernel<Real, FERN, BT, XLDS, ILP, KeyT, VW, NT>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, nodes, w, out,
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(NT), lds, stream, d, x, nodes, w, out,
                      trees_per_block, FastDiv(d.M));
   HT_LAUNCH_CHECK("forest forward");
   return HT_OK;
@@ -173,7 +176,11 @@ int dispatch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes
                      hipStream_t stream) {
   // room for the per-pass results: (4 trees x 1024 threads + one pad column) x (|margin| + key)
   const size_t reserve = size_t(4) * kForestThreads * (sizeof(Real) + sizeof(uint32_t));
-  switch (pick_tile<Real>(d.F, reserve)) {
+  int bt = pick_tile<Real>(d.F, reserve);
+  // With many outputs per leaf the output phase dominates, and it runs better on a narrower tile: twice the trees per
+  // pass (longer contiguous row segments per store burst, half the barriers) and one row per wavefront.
+  if (d.M >= 8 && bt >= 32) bt /= 2;
+  switch (bt) {
     case 64: return launch_forward<Real, FERN, 64, true>(d, x, nodes, w, out, stream);
     case 32: return launch_forward<Real, FERN, 32, true>(d, x, nodes, w, out, stream);
     case 16: return launch_forward<Real, FERN, 16, true>(d, x, nodes, w, out, stream);
