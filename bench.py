@@ -2,9 +2,13 @@
 """Headline benchmark: RandomHingeForest fp32 forward+backward on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c1] [--mode atomic|deterministic]
+                    [--path train|stateless]
 
-One step = one forward (tree_forward) plus one backward (tree_backward, all three gradients requested, atomic mode)
-over one batch of synthetic input that is already resident in HBM, called through the C ABI on torch's current stream.
+One step = one forward plus one backward (all three gradients requested, atomic mode) over one batch of synthetic input
+that is already resident in HBM, called through the C ABI on torch's current stream. `--path train` (default) is what
+the autograd functions run in training: the forward keeps its walk records and the backward consumes them
+(tree_forward_records / tree_backward_records); `--path stateless` is the reference's operator pair (tree_forward /
+tree_backward), whose backward walks the trees again. The other path is timed too and reported under `other_path`.
 The default workload is the configuration the metric is quoted on: x ~ N(0,1) [65536, 1024], 1000 trees, depth 10,
 extra_outputs = 10 (out [65536, 1000, 10]); thresholds ~ U(-3,3) made consistent like the module constructor does,
 ordinals ~ U{0..1023}, leaf weights ~ N(0,1), upstream gradient ~ N(0,1).
@@ -99,6 +103,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--mode", default="atomic", choices=["atomic", "deterministic"])
+    ap.add_argument("--path", default="train", choices=["train", "stateless"])
     ap.add_argument("--cpu-rows", type=int, default=32768, help="rows of the batch timed on the CPU (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -115,35 +120,56 @@ def main():
     name = args.workload
     B, F, T, depth, M, kind, _, desc = WORKLOADS[name]
     x, thr, ordn, w, gout = make_inputs(torch, name, dev)
-    fwd = ops.fern_forward if kind == "fern" else ops.tree_forward
-    if args.mode == "deterministic":
-        bwd = ops.fern_backward_deterministic if kind == "fern" else ops.tree_backward_deterministic
-    else:
-        bwd = ops.fern_backward if kind == "fern" else ops.tree_backward
+    pre = "fern_" if kind == "fern" else "tree_"
+    det = args.mode == "deterministic"
 
-    def step():
-        out = fwd(x, thr, ordn, w)
-        grads = bwd(x, True, thr, True, ordn, False, w, True, gout)
-        return out, grads
+    def make_step(path):
+        if path == "train":
+            fwd_op, bwd_op = getattr(ops, pre + "forward_records"), getattr(ops, pre + "backward_records")
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+            def fwd():
+                return fwd_op(x, thr, ordn, w)
 
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        ev[i][0].record()
-        out = fwd(x, thr, ordn, w)
-        ev[i][1].record()
-        grads = bwd(x, True, thr, True, ordn, False, w, True, gout)
-        ev[i][2].record()
-        del out, grads
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+            stateless_bwd = getattr(ops, pre + ("backward_deterministic" if det else "backward"))
+
+            def bwd(state):
+                if state[1] is None:   # shape for which the library keeps no records: the autograd function re-walks
+                    return stateless_bwd(x, True, thr, True, ordn, False, w, True, gout)
+                return bwd_op(state[1], det, x, True, thr, True, ordn, False, w, True, gout)
+        else:
+            fwd_op = getattr(ops, pre + "forward")
+            bwd_op = getattr(ops, pre + ("backward_deterministic" if det else "backward"))
+
+            def fwd():
+                return fwd_op(x, thr, ordn, w)
+
+            def bwd(state):
+                return bwd_op(x, True, thr, True, ordn, False, w, True, gout)
+        return fwd, bwd
+
+    def run(path, steps, warmup):
+        fwd, bwd = make_step(path)
+        for _ in range(warmup):
+            bwd(fwd())
+        torch.cuda.synchronize()
+        # events on torch's current stream, which is the stream the library launches on
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+        t0 = time.perf_counter()
+        for i in range(steps):
+            ev[i][0].record()
+            state = fwd()
+            ev[i][1].record()
+            grads = bwd(state)
+            ev[i][2].record()
+            del state, grads
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return ((t1 - t0) * 1e3 / steps, sum(e[0].elapsed_time(e[1]) for e in ev) / steps,
+                sum(e[1].elapsed_time(e[2]) for e in ev) / steps)
+
+    other = "stateless" if args.path == "train" else "train"
+    o_ms, o_fwd, o_bwd = run(other, max(3, args.steps // 4), 2)
+    ms_per_step, fwd_ms, bwd_ms = run(args.path, args.steps, args.warmup)
 
     fwd_bytes, bwd_bytes = algorithmic_bytes(B, F, T, depth, M, kind)
     achieved = fwd_bytes / (fwd_ms * 1e-3) / 1e9
@@ -160,7 +186,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": f"{name}: {desc}", "backward_mode": args.mode, "B": B, "F": F, "T": T, "depth": depth,
+        "config": {"workload": f"{name}: {desc}", "backward_mode": args.mode, "path": args.path, "B": B, "F": F, "T": T, "depth": depth,
                    "extra_outputs": M},
         "roofline": {"bound": "hbm", "kernel": "forward_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get(name),
@@ -168,6 +194,8 @@ def main():
         "backward": {"mode": args.mode, "ms": bwd_ms, "samples_per_s": B / (bwd_ms * 1e-3),
                      "algorithmic_bytes": bwd_bytes, "hbm_frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
         "step_hbm_frac": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "other_path": {"path": other, "ms_per_step": o_ms, "forward_ms": o_fwd, "backward_ms": o_bwd,
+                       "samples_per_s": B / (o_ms * 1e-3)},
     }
     if args.cpu_rows > 0:
         result["cpu_baseline"] = cpu_baseline(torch, name, x, thr, ordn, w, gout, args.cpu_rows)

@@ -42,6 +42,10 @@ SIGNATURES = {
     "ht_forest_forward": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "ht_forest_backward_workspace": (_SZ, [ctypes.POINTER(ForestShape), _I, _I, _I, _I]),
     "ht_forest_backward": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _SZ, _P]),
+    "ht_forest_records_bytes": (_SZ, [ctypes.POINTER(ForestShape)]),
+    "ht_forest_forward_records": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _SZ, _P, _SZ, _P]),
+    "ht_forest_backward_records_workspace": (_SZ, [ctypes.POINTER(ForestShape), _I, _I, _I, _I]),
+    "ht_forest_backward_records": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _SZ, _P, _P, _P, _I, _P, _SZ, _P]),
     "ht_forest_maps_workspace": (_SZ, [ctypes.POINTER(ForestShape)]),
     "ht_forest_maps": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "ht_conv_output_size": (_I, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int64)]),

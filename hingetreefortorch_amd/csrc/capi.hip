@@ -124,9 +124,65 @@ int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, 
   const bool fern = s->kind == HT_FERN;
   if (s->dtype == HT_F32)
     return forest_forward<float>(d, fern, (const float *)x, (const float *)thr, ord, (const float *)w, (float *)out,
-                                 workspace, workspace_bytes, st);
+                                 nullptr, workspace, workspace_bytes, st);
   return forest_forward<double>(d, fern, (const double *)x, (const double *)thr, ord, (const double *)w, (double *)out,
-                                workspace, workspace_bytes, st);
+                                nullptr, workspace, workspace_bytes, st);
+}
+
+size_t ht_forest_records_bytes(const ht_forest_shape *s) {
+  ForestDims d;
+  if (make_dims(s, &d) != HT_OK) return 0;
+  return s->dtype == HT_F32 ? forest_records_bytes<float>(d) : forest_records_bytes<double>(d);
+}
+
+int ht_forest_forward_records(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord,
+                              const void *w, void *out, void *records, size_t records_bytes, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+  ForestDims d;
+  int rc = make_dims(s, &d);
+  if (rc != HT_OK) return rc;
+  const size_t need = ht_forest_records_bytes(s);
+  if (need == 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: walk records are not offered for this shape.");
+  if (d.S > 0 && d.T > 0 && (!x || !thr || !ord || !w || !out || !records))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (records_bytes < need) return fail(HT_ERR_INVALID_ARGUMENT, "Error: records buffer too small.");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool fern = s->kind == HT_FERN;
+  if (s->dtype == HT_F32)
+    return forest_forward<float>(d, fern, (const float *)x, (const float *)thr, ord, (const float *)w, (float *)out,
+                                 records, workspace, workspace_bytes, st);
+  return forest_forward<double>(d, fern, (const double *)x, (const double *)thr, ord, (const double *)w, (double *)out,
+                                records, workspace, workspace_bytes, st);
+}
+
+size_t ht_forest_backward_records_workspace(const ht_forest_shape *s, int mode, int need_dx, int need_dthr,
+                                            int need_dw) {
+  ForestDims d;
+  if (make_dims(s, &d) != HT_OK) return 0;
+  return s->dtype == HT_F32
+             ? forest_backward_records_workspace<float>(d, mode, need_dx != 0, need_dthr != 0, need_dw != 0)
+             : forest_backward_records_workspace<double>(d, mode, need_dx != 0, need_dthr != 0, need_dw != 0);
+}
+
+int ht_forest_backward_records(const ht_forest_shape *s, const void *w, const void *gout, const void *records,
+                               size_t records_bytes, void *dx, void *dthr, void *dw, int mode, void *workspace,
+                               size_t workspace_bytes, void *stream) {
+  ForestDims d;
+  int rc = make_dims(s, &d);
+  if (rc != HT_OK) return rc;
+  if (mode != HT_BACKWARD_ATOMIC && mode != HT_BACKWARD_DETERMINISTIC)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: unknown backward mode.");
+  const size_t need = ht_forest_records_bytes(s);
+  if (need == 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: walk records are not offered for this shape.");
+  if (d.S > 0 && d.T > 0 && (!w || !gout || !records)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (records_bytes < need) return fail(HT_ERR_INVALID_ARGUMENT, "Error: records buffer too small.");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool fern = s->kind == HT_FERN;
+  if (s->dtype == HT_F32)
+    return forest_backward_records<float>(d, fern, (const float *)w, (const float *)gout, records, (float *)dx,
+                                          (float *)dthr, (float *)dw, mode, workspace, workspace_bytes, st);
+  return forest_backward_records<double>(d, fern, (const double *)w, (const double *)gout, records, (double *)dx,
+                                         (double *)dthr, (double *)dw, mode, workspace, workspace_bytes, st);
 }
 
 size_t ht_forest_backward_workspace(const ht_forest_shape *s, int mode, int need_dx, int need_dthr, int need_dw) {

@@ -74,9 +74,10 @@ int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *d
 
 template <typename Real>
 size_t forest_forward_workspace(const ForestDims &d);
+// `records` (optional): forest_records_bytes() bytes that receive the walk records for forest_backward_records().
 template <typename Real>
 int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                   Real *out, void *ws, size_t ws_bytes, hipStream_t stream);
+                   Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream);
 
 template <typename Real>
 size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw);
@@ -84,6 +85,15 @@ template <typename Real>
 int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
                     const Real *gout, Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes,
                     hipStream_t stream);
+
+// Training path: backward from the records a forward pass wrote (0 bytes: not offered for this shape).
+template <typename Real>
+size_t forest_records_bytes(const ForestDims &d);
+template <typename Real>
+size_t forest_backward_records_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw);
+template <typename Real>
+int forest_backward_records(const ForestDims &d, bool fern, const Real *w, const Real *gout, const void *records,
+                            Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes, hipStream_t stream);
 
 template <typename Real>
 size_t forest_maps_workspace(const ForestDims &d);

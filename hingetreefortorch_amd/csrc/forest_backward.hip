@@ -21,6 +21,7 @@
 
 #include "forest_tile.hpp"
 #include "lds_accumulate.hpp"
+#include "records.hpp"
 
 namespace ht {
 namespace {
@@ -28,64 +29,8 @@ namespace {
 constexpr int kIlp = 4;         // trees walked concurrently per thread by the records kernel
 
 // ---------------------------------------------------------------------------------------------------------------
-// walk records
+// walk records (layout in records.hpp)
 // ---------------------------------------------------------------------------------------------------------------
-// COMPACT (depth <= 16 and F <= 65536): key | vertex << 16 in one word, ordinal in 16 bits.
-template <typename Real, bool COMPACT>
-struct Records {
-  uint32_t *a;    // COMPACT: key | vertex << 16      else: key
-  uint32_t *b;    // COMPACT: unused                  else: vertex
-  void *ordinal;  // COMPACT: uint16_t[]              else: uint32_t[]
-  Real *margin;
-  Real *c;        // sign(margin) * sum_m w * g, filled by the tree kernel
-
-  __device__ __forceinline__ void put(long long at, uint32_t key, uint32_t vertex, uint32_t ord, Real m) const {
-    if (COMPACT) {
-      a[at] = key | (vertex << 16);
-      static_cast<uint16_t *>(ordinal)[at] = uint16_t(ord);
-    } else {
-      a[at] = key;
-      b[at] = vertex;
-      static_cast<uint32_t *>(ordinal)[at] = ord;
-    }
-    margin[at] = m;
-  }
-  __device__ __forceinline__ uint32_t key(long long at) const { return COMPACT ? (a[at] & 0xffffu) : a[at]; }
-  __device__ __forceinline__ uint32_t vertex(long long at) const { return COMPACT ? (a[at] >> 16) : b[at]; }
-  __device__ __forceinline__ uint32_t ord(long long at) const {
-    return COMPACT ? uint32_t(static_cast<const uint16_t *>(ordinal)[at]) : static_cast<const uint32_t *>(ordinal)[at];
-  }
-};
-
-static bool compact_ok(const ForestDims &d) { return d.depth <= 16 && d.F <= 65536; }
-
-template <typename Real>
-size_t records_bytes(const ForestDims &d) {
-  const size_t n = size_t(d.T) * size_t(d.S);
-  if (compact_ok(d)) return align_up(n * 4, 256) + align_up(n * 2, 256) + 2 * align_up(n * sizeof(Real), 256);
-  return 3 * align_up(n * 4, 256) + 2 * align_up(n * sizeof(Real), 256);
-}
-
-template <typename Real, bool COMPACT>
-Records<Real, COMPACT> carve_records(const ForestDims &d, void *ws) {
-  const size_t n = size_t(d.T) * size_t(d.S);
-  unsigned char *p = static_cast<unsigned char *>(ws);
-  Records<Real, COMPACT> r;
-  r.a = reinterpret_cast<uint32_t *>(p);
-  p += align_up(n * 4, 256);
-  r.b = nullptr;
-  if (!COMPACT) {
-    r.b = reinterpret_cast<uint32_t *>(p);
-    p += align_up(n * 4, 256);
-  }
-  r.ordinal = p;
-  p += align_up(n * (COMPACT ? 2 : 4), 256);
-  r.margin = reinterpret_cast<Real *>(p);
-  p += align_up(n * sizeof(Real), 256);
-  r.c = reinterpret_cast<Real *>(p);
-  return r;
-}
-
 template <typename Real, bool FERN, int BT, bool XLDS, bool COMPACT>
 __global__ __launch_bounds__(kForestThreads) void records_kernel(ForestDims d, const Real *__restrict__ x,
                                                                  const Node<Real> *__restrict__ nodes,
@@ -121,7 +66,7 @@ __global__ __launch_bounds__(kForestThreads) void records_kernel(ForestDims d, c
 #pragma unroll
     for (int i = 0; i < kIlp; ++i)
       if (t[i] < t_end)
-        rec.put((long long)t[i] * d.S + s, r[i].key, r[i].vertex, uint32_t(nd[i][r[i].vertex].ord), r[i].margin);
+        rec.put((long long)t[i] * d.S + s, r[i].key, r[i].vertex, r[i].ord, r[i].margin);
   }
 }
 
@@ -979,14 +924,14 @@ int launch_absmax(const Real *p, long long n, unsigned long long *slot, hipStrea
   return HT_OK;
 }
 
-// Staged pipeline. FIXED selects the bit-reproducible fixed-point accumulators; fixed_ws then points at the
+// Staged pipeline over the records `rec`, which are produced here first (walk) or came from a forward pass. FIXED selects the bit-reproducible fixed-point accumulators; fixed_ws then points at the
 // FixedLayout area and dX must have been cleared by the caller.
 template <typename Real, bool FERN, bool COMPACT, bool FIXED>
 int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, const Real *gout,
-                    Real *dx, Real *dthr, Real *dw, void *rec_ws, void *fixed_ws, hipStream_t stream) {
-  Records<Real, COMPACT> rec = carve_records<Real, COMPACT>(d, rec_ws);
-  int rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream);
-  if (rc != HT_OK) return rc;
+                    Real *dx, Real *dthr, Real *dw, Records<Real, COMPACT> rec, bool walk, void *fixed_ws,
+                    hipStream_t stream) {
+  int rc = HT_OK;
+  if (walk && (rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream)) != HT_OK) return rc;
   const bool need_c = dx || dthr;
   const long long pairs = (long long)d.T * d.S;
   TreePlan plan;
@@ -1089,10 +1034,10 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
 // Sequential owner-computes pass for shapes whose accumulators do not fit LDS.
 template <typename Real, bool FERN, bool COMPACT>
 int backward_sequential(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w,
-                        const Real *gout, Real *dx, Real *dthr, Real *dw, void *rec_ws, hipStream_t stream) {
-  Records<Real, COMPACT> rec = carve_records<Real, COMPACT>(d, rec_ws);
-  int rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream);
-  if (rc != HT_OK) return rc;
+                        const Real *gout, Real *dx, Real *dthr, Real *dw, Records<Real, COMPACT> rec, bool walk,
+                        hipStream_t stream) {
+  int rc = HT_OK;
+  if (walk && (rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream)) != HT_OK) return rc;
   if (dx) {
     const long long blocks = (d.S + 255) / 256;
     hipLaunchKernelGGL((det_dx_kernel<Real, COMPACT>), dim3((unsigned)blocks), dim3(256), 0, stream, d, w, gout, rec,
@@ -1116,18 +1061,77 @@ int backward_sequential(const ForestDims &d, const Real *x, const Node<Real> *no
   return HT_OK;
 }
 
+// Which pipeline serves a backward call.
+enum class Route { kFused, kStaged, kFixed, kSequential };
+
+template <typename Real>
+Route pick_route(const ForestDims &d, int mode, bool need_dx, bool need_dw, bool have_records) {
+  if (mode == HT_BACKWARD_DETERMINISTIC)
+    return staged_ok<Real>(d, need_dx, need_dw, true) ? Route::kFixed : Route::kSequential;
+  if (staged_ok<Real>(d, need_dx, need_dw, false)) return (have_records || !prefer_fused(d)) ? Route::kStaged : Route::kFused;
+  return have_records ? Route::kSequential : Route::kFused;  // with records there is no need to walk again
+}
+
+// Workspace after the packed vertices (stateless call) / from the start (records call): [saved records] c scratch,
+// fixed-point area.
+template <typename Real>
+size_t route_bytes(const ForestDims &d, Route r, bool need_dthr, bool need_dw, bool have_records) {
+  if (r == Route::kFused) return 0;
+  size_t bytes = (have_records ? 0 : records_saved_bytes<Real>(d)) + records_scratch_bytes<Real>(d);
+  if (r == Route::kFixed) bytes += fixed_layout(d, need_dthr, need_dw).total;
+  return bytes;
+}
+
+template <typename Real>
+int run_route(const ForestDims &d, Route route, bool fern, const Real *x, const Node<Real> *nodes, const Real *w,
+              const Real *gout, Real *dx, Real *dthr, Real *dw, void *saved, void *scratch, bool walk,
+              hipStream_t stream) {
+  void *fixed_ws = static_cast<unsigned char *>(scratch) + records_scratch_bytes<Real>(d);
+  const bool compact = compact_ok(d);
+#define HT_STAGED(FERN_, COMPACT_, FIXED_)                                                            \
+  backward_staged<Real, FERN_, COMPACT_, FIXED_>(d, x, nodes, w, gout, dx, dthr, dw,                  \
+                                                 carve_records<Real, COMPACT_>(d, saved, scratch), walk, fixed_ws, stream)
+#define HT_SEQ(FERN_, COMPACT_)                                                                       \
+  backward_sequential<Real, FERN_, COMPACT_>(d, x, nodes, w, gout, dx, dthr, dw,                      \
+                                             carve_records<Real, COMPACT_>(d, saved, scratch), walk, stream)
+  switch (route) {
+    case Route::kFixed:
+      if (fern) return compact ? HT_STAGED(true, true, true) : HT_STAGED(true, false, true);
+      return compact ? HT_STAGED(false, true, true) : HT_STAGED(false, false, true);
+    case Route::kSequential:
+      if (fern) return compact ? HT_SEQ(true, true) : HT_SEQ(true, false);
+      return compact ? HT_SEQ(false, true) : HT_SEQ(false, false);
+    case Route::kStaged:
+      if (fern) return compact ? HT_STAGED(true, true, false) : HT_STAGED(true, false, false);
+      return compact ? HT_STAGED(false, true, false) : HT_STAGED(false, false, false);
+    default:
+      return fern ? dispatch_backward_fused<Real, true>(d, x, nodes, w, gout, dx, dthr, dw, stream)
+                  : dispatch_backward_fused<Real, false>(d, x, nodes, w, gout, dx, dthr, dw, stream);
+  }
+#undef HT_STAGED
+#undef HT_SEQ
+}
+
+// Clears the requested gradients as far as the route accumulates into them (the staged dX kernel overwrites all of
+// dX). Returns 1 if there is nothing else to do.
+template <typename Real>
+int clear_gradients(const ForestDims &d, Route route, Real *dx, Real *dthr, Real *dw, hipStream_t stream, bool *done) {
+  int rc;
+  const bool empty = d.S == 0 || d.T == 0;
+  const bool clear_dx = route != Route::kStaged || empty;
+  if (dx && clear_dx && (rc = zero_fill(dx, size_t(d.S) * d.F * sizeof(Real), stream)) != HT_OK) return rc;
+  if (dthr && (rc = zero_fill(dthr, size_t(d.T) * d.V * sizeof(Real), stream)) != HT_OK) return rc;
+  if (dw && (rc = zero_fill(dw, size_t(d.T) * d.L * d.M * sizeof(Real), stream)) != HT_OK) return rc;
+  *done = empty || (!dx && !dthr && !dw);
+  return HT_OK;
+}
+
 }  // namespace
 
 template <typename Real>
 size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw) {
-  size_t bytes = packed_nodes_bytes<Real>(d);
-  if (mode == HT_BACKWARD_DETERMINISTIC) {
-    bytes += align_up(records_bytes<Real>(d), 256);
-    if (staged_ok<Real>(d, need_dx, need_dw, true)) bytes += fixed_layout(d, need_dthr, need_dw).total;
-    return bytes;
-  }
-  if (staged_ok<Real>(d, need_dx, need_dw, false) && !prefer_fused(d)) bytes += records_bytes<Real>(d);
-  return bytes;
+  const Route r = pick_route<Real>(d, mode, need_dx, need_dw, false);
+  return packed_nodes_bytes<Real>(d) + route_bytes<Real>(d, r, need_dthr, need_dw, false);
 }
 
 template <typename Real>
@@ -1135,58 +1139,59 @@ int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *t
                     const Real *gout, Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes,
                     hipStream_t stream) {
   int rc;
-  const bool det = mode == HT_BACKWARD_DETERMINISTIC;
-  const bool fixed = det && staged_ok<Real>(d, dx != nullptr, dw != nullptr, true);
-  const bool staged = det || (staged_ok<Real>(d, dx != nullptr, dw != nullptr, false) && !prefer_fused(d));
-  // The staged dX kernel overwrites every element of dX; everything else accumulates into zeros.
-  const bool empty = d.S == 0 || d.T == 0;
-  const bool clear_dx = !staged || det || empty;
-  if (dx && clear_dx && (rc = zero_fill(dx, size_t(d.S) * d.F * sizeof(Real), stream)) != HT_OK) return rc;
-  if (dthr && (rc = zero_fill(dthr, size_t(d.T) * d.V * sizeof(Real), stream)) != HT_OK) return rc;
-  if (dw && (rc = zero_fill(dw, size_t(d.T) * d.L * d.M * sizeof(Real), stream)) != HT_OK) return rc;
-  if (empty || (!dx && !dthr && !dw)) return HT_OK;
+  const Route route = pick_route<Real>(d, mode, dx != nullptr, dw != nullptr, false);
+  bool done;
+  if ((rc = clear_gradients<Real>(d, route, dx, dthr, dw, stream, &done)) != HT_OK || done) return rc;
   const size_t node_bytes = packed_nodes_bytes<Real>(d);
-  const size_t rec_bytes = staged ? align_up(records_bytes<Real>(d), 256) : 0;
-  const size_t need =
-      node_bytes + (det ? rec_bytes : (staged ? records_bytes<Real>(d) : 0)) +
-      (fixed ? fixed_layout(d, dthr != nullptr, dw != nullptr).total : 0);
+  const size_t need = node_bytes + route_bytes<Real>(d, route, dthr != nullptr, dw != nullptr, false);
   if (ws == nullptr || ws_bytes < need)
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the backward pass.");
   if ((rc = pack_nodes<Real>(d, thr, ord, ws, stream)) != HT_OK) return rc;
   const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
-  void *rec_ws = static_cast<unsigned char *>(ws) + node_bytes;
-  void *fixed_ws = static_cast<unsigned char *>(rec_ws) + rec_bytes;
-  const bool compact = compact_ok(d);
-
-#define HT_STAGED(FERN_, COMPACT_, FIXED_) \
-  backward_staged<Real, FERN_, COMPACT_, FIXED_>(d, x, nodes, w, gout, dx, dthr, dw, rec_ws, fixed_ws, stream)
-#define HT_SEQ(FERN_, COMPACT_) \
-  backward_sequential<Real, FERN_, COMPACT_>(d, x, nodes, w, gout, dx, dthr, dw, rec_ws, stream)
-  if (fixed) {
-    if (fern) return compact ? HT_STAGED(true, true, true) : HT_STAGED(true, false, true);
-    return compact ? HT_STAGED(false, true, true) : HT_STAGED(false, false, true);
-  }
-  if (det) {
-    if (fern) return compact ? HT_SEQ(true, true) : HT_SEQ(true, false);
-    return compact ? HT_SEQ(false, true) : HT_SEQ(false, false);
-  }
-  if (staged) {
-    if (fern) return compact ? HT_STAGED(true, true, false) : HT_STAGED(true, false, false);
-    return compact ? HT_STAGED(false, true, false) : HT_STAGED(false, false, false);
-  }
-#undef HT_STAGED
-#undef HT_SEQ
-  return fern ? dispatch_backward_fused<Real, true>(d, x, nodes, w, gout, dx, dthr, dw, stream)
-              : dispatch_backward_fused<Real, false>(d, x, nodes, w, gout, dx, dthr, dw, stream);
+  unsigned char *saved = static_cast<unsigned char *>(ws) + node_bytes;
+  unsigned char *scratch = saved + records_saved_bytes<Real>(d);
+  return run_route<Real>(d, route, fern, x, nodes, w, gout, dx, dthr, dw, saved, scratch, true, stream);
 }
 
-template size_t forest_backward_workspace<float>(const ForestDims &, int, bool, bool, bool);
-template size_t forest_backward_workspace<double>(const ForestDims &, int, bool, bool, bool);
-template int forest_backward<float>(const ForestDims &, bool, const float *, const float *, const int64_t *,
-                                    const float *, const float *, float *, float *, float *, int, void *, size_t,
-                                    hipStream_t);
-template int forest_backward<double>(const ForestDims &, bool, const double *, const double *, const int64_t *,
-                                     const double *, const double *, double *, double *, double *, int, void *, size_t,
-                                     hipStream_t);
+template <typename Real>
+size_t forest_records_bytes(const ForestDims &d) {
+  // offered where the staged kernels can consume them for every combination of requested gradients
+  if (!staged_ok<Real>(d, true, true, false)) return 0;
+  return records_saved_bytes<Real>(d);
+}
+
+template <typename Real>
+size_t forest_backward_records_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw) {
+  const Route r = pick_route<Real>(d, mode, need_dx, need_dw, true);
+  return route_bytes<Real>(d, r, need_dthr, need_dw, true);
+}
+
+template <typename Real>
+int forest_backward_records(const ForestDims &d, bool fern, const Real *w, const Real *gout, const void *records,
+                            Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes,
+                            hipStream_t stream) {
+  int rc;
+  const Route route = pick_route<Real>(d, mode, dx != nullptr, dw != nullptr, true);
+  bool done;
+  if ((rc = clear_gradients<Real>(d, route, dx, dthr, dw, stream, &done)) != HT_OK || done) return rc;
+  const size_t need = route_bytes<Real>(d, route, dthr != nullptr, dw != nullptr, true);
+  if (ws == nullptr || ws_bytes < need)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the backward pass.");
+  return run_route<Real>(d, route, fern, (const Real *)nullptr, (const Node<Real> *)nullptr, w, gout, dx, dthr, dw,
+                         const_cast<void *>(records), ws, false, stream);
+}
+
+#define HT_INSTANTIATE(Real)                                                                                          \
+  template size_t forest_backward_workspace<Real>(const ForestDims &, int, bool, bool, bool);                         \
+  template int forest_backward<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,           \
+                                     const Real *, const Real *, Real *, Real *, Real *, int, void *, size_t,         \
+                                     hipStream_t);                                                                    \
+  template size_t forest_records_bytes<Real>(const ForestDims &);                                                     \
+  template size_t forest_backward_records_workspace<Real>(const ForestDims &, int, bool, bool, bool);                 \
+  template int forest_backward_records<Real>(const ForestDims &, bool, const Real *, const Real *, const void *,      \
+                                             Real *, Real *, Real *, int, void *, size_t, hipStream_t);
+HT_INSTANTIATE(float)
+HT_INSTANTIATE(double)
+#undef HT_INSTANTIATE
 
 }  // namespace ht

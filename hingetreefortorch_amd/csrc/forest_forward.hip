@@ -9,6 +9,7 @@
 // contiguous (tree, m) -- or for K > 1 the contiguous (inner position, m) -- axis of `out`, so the dominant store
 // traffic is emitted as full-width rows.
 #include "forest_tile.hpp"
+#include "records.hpp"
 
 namespace ht {
 namespace {
@@ -30,11 +31,16 @@ constexpr int kOutUnroll = 5;  // output vectors per lane whose weight gathers a
 // ILP = trees walked concurrently per thread; KeyT = storage type of the parked leaf keys (uint16_t up to depth 16);
 // VW = outputs per lane in the output phase (divides M): the memory pipeline charges a gather instruction by its
 // lanes, not by the lines it touches, so wider lanes mean proportionally fewer cycles per output.
-template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW, int NT>
+//
+// RECORD (training path): the walk results are also written out as walk records (records.hpp) for a later backward
+// pass, which then does not have to walk again.
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW, int NT, bool RECORD,
+          bool COMPACT>
 __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *__restrict__ x,
-                                                                 const Node<Real> *__restrict__ nodes,
-                                                                 const Real *__restrict__ w, Real *__restrict__ out,
-                                                                 int trees_per_block, FastDiv div_m) {
+                                                     const Node<Real> *__restrict__ nodes,
+                                                     const Real *__restrict__ w, Real *__restrict__ out,
+                                                     Records<Real, COMPACT> rec, int trees_per_block,
+                                                     FastDiv div_m) {
   typedef Real Vec __attribute__((ext_vector_type(VW)));
   constexpr int TC = NT / BT;        // tree slots per walk round
   constexpr int kIlp = ILP;
@@ -76,6 +82,8 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
       for (int i = 0; i < kIlp; ++i) {
         r_abs[j * LDR + tt + i * TC] = ht_abs(r[i].margin);
         r_key[j * LDR + tt + i * TC] = KeyT(r[i].key);
+        if (RECORD && tb + tt + i * TC < t_end)
+          rec.put((long long)(tb + tt + i * TC) * d.S + s, r[i].key, r[i].vertex, r[i].ord, r[i].margin);
       }
     }
     __syncthreads();
@@ -132,48 +140,65 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
   }
 }
 
-template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW, int NT = kForestThreads>
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
+int launch_forward_rec(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
+                       void *records, hipStream_t stream);
+
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW, bool RECORD, bool COMPACT>
 int launch_forward_vw(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                      hipStream_t stream) {
+                      void *records, hipStream_t stream) {
+  constexpr int NT = kForestThreads;
   constexpr int TP = NT / BT * ILP;
   const size_t lds = (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TP + 1) * BT * (sizeof(Real) + sizeof(KeyT));
   const long long tiles = (d.S + BT - 1) / BT;
   int trees_per_block, gy;
   split_trees(tiles, d.T, TP, &trees_per_block, &gy);
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
-  auto kernel = forward_kernel<Real, FERN, BT, XLDS, ILP, KeyT, VW, NT>;
+  auto kernel = forward_kernel<Real, FERN, BT, XLDS, ILP, KeyT, VW, NT, RECORD, COMPACT>;
+  Records<Real, COMPACT> rec{};
+  if (RECORD) rec = carve_records<Real, COMPACT>(d, records, nullptr);
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(NT), lds, stream, d, x, nodes, w, out,
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(NT), lds, stream, d, x, nodes, w, out, rec,
                      trees_per_block, FastDiv(d.M));
   HT_LAUNCH_CHECK("forest forward");
   return HT_OK;
 }
 
+template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
+int launch_forward_rec(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
+                       void *records, hipStream_t stream) {
+  if (!records)
+    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, false, true>(d, x, nodes, w, out, records, stream);
+  if (compact_ok(d))
+    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, true, true>(d, x, nodes, w, out, records, stream);
+  return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, true, false>(d, x, nodes, w, out, records, stream);
+}
+
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT>
 int launch_forward_as(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                      hipStream_t stream) {
+                      void *records, hipStream_t stream) {
   // widest output vector that M and the pointers allow (K > 1 keeps scalar outputs)
   const uintptr_t pw = reinterpret_cast<uintptr_t>(w), po = reinterpret_cast<uintptr_t>(out);
   if (d.K == 1 && d.M % 4 == 0 && pw % (4 * sizeof(Real)) == 0 && po % (4 * sizeof(Real)) == 0)
-    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, 4>(d, x, nodes, w, out, stream);
+    return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 4>(d, x, nodes, w, out, records, stream);
   if (d.K == 1 && d.M % 2 == 0 && pw % (2 * sizeof(Real)) == 0 && po % (2 * sizeof(Real)) == 0)
-    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, 2>(d, x, nodes, w, out, stream);
-  return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, 1>(d, x, nodes, w, out, stream);
+    return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 2>(d, x, nodes, w, out, records, stream);
+  return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 1>(d, x, nodes, w, out, records, stream);
 }
 
 // Four trees per thread with 16-bit parked keys where the depth allows it, else two trees with 32-bit keys: both keep
 // the per-pass results of a 1024-thread workgroup under the LDS left beside a 128 KB sample tile.
 template <typename Real, bool FERN, int BT, bool XLDS>
 int launch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                   hipStream_t stream) {
-  if (d.depth <= 16) return launch_forward_as<Real, FERN, BT, XLDS, 4, uint16_t>(d, x, nodes, w, out, stream);
-  return launch_forward_as<Real, FERN, BT, XLDS, 2, uint32_t>(d, x, nodes, w, out, stream);
+                   void *records, hipStream_t stream) {
+  if (d.depth <= 16) return launch_forward_as<Real, FERN, BT, XLDS, 4, uint16_t>(d, x, nodes, w, out, records, stream);
+  return launch_forward_as<Real, FERN, BT, XLDS, 2, uint32_t>(d, x, nodes, w, out, records, stream);
 }
 
 template <typename Real, bool FERN>
 int dispatch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                     hipStream_t stream) {
+                     void *records, hipStream_t stream) {
   // room for the per-pass results: (4 trees x 1024 threads + one pad column) x (|margin| + key)
   const size_t reserve = size_t(4) * kForestThreads * (sizeof(Real) + sizeof(uint32_t));
   int bt = pick_tile<Real>(d.F, reserve);
@@ -181,11 +206,11 @@ int dispatch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes
   // pass (longer contiguous row segments per store burst, half the barriers) and one row per wavefront.
   if (d.M >= 8 && bt >= 32) bt /= 2;
   switch (bt) {
-    case 64: return launch_forward<Real, FERN, 64, true>(d, x, nodes, w, out, stream);
-    case 32: return launch_forward<Real, FERN, 32, true>(d, x, nodes, w, out, stream);
-    case 16: return launch_forward<Real, FERN, 16, true>(d, x, nodes, w, out, stream);
-    case 8: return launch_forward<Real, FERN, 8, true>(d, x, nodes, w, out, stream);
-    default: return launch_forward<Real, FERN, 64, false>(d, x, nodes, w, out, stream);
+    case 64: return launch_forward<Real, FERN, 64, true>(d, x, nodes, w, out, records, stream);
+    case 32: return launch_forward<Real, FERN, 32, true>(d, x, nodes, w, out, records, stream);
+    case 16: return launch_forward<Real, FERN, 16, true>(d, x, nodes, w, out, records, stream);
+    case 8: return launch_forward<Real, FERN, 8, true>(d, x, nodes, w, out, records, stream);
+    default: return launch_forward<Real, FERN, 64, false>(d, x, nodes, w, out, records, stream);
   }
 }
 
@@ -213,15 +238,15 @@ size_t forest_forward_workspace(const ForestDims &d) {
 
 template <typename Real>
 int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                   Real *out, void *ws, size_t ws_bytes, hipStream_t stream) {
+                   Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream) {
   if (d.S == 0 || d.T == 0) return HT_OK;
   if (ws == nullptr || ws_bytes < packed_nodes_bytes<Real>(d))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the forward pass.");
   int rc = pack_nodes<Real>(d, thr, ord, ws, stream);
   if (rc != HT_OK) return rc;
   const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
-  return fern ? dispatch_forward<Real, true>(d, x, nodes, w, out, stream)
-              : dispatch_forward<Real, false>(d, x, nodes, w, out, stream);
+  return fern ? dispatch_forward<Real, true>(d, x, nodes, w, out, records, stream)
+              : dispatch_forward<Real, false>(d, x, nodes, w, out, records, stream);
 }
 
 #define HT_INSTANTIATE(Real)                                                                                          \
@@ -229,7 +254,7 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
   template int pack_nodes<Real>(const ForestDims &, const Real *, const int64_t *, void *, hipStream_t);              \
   template size_t forest_forward_workspace<Real>(const ForestDims &);                                                 \
   template int forest_forward<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,            \
-                                    const Real *, Real *, void *, size_t, hipStream_t);
+                                    const Real *, Real *, void *, void *, size_t, hipStream_t);
 HT_INSTANTIATE(float)
 HT_INSTANTIATE(double)
 #undef HT_INSTANTIATE

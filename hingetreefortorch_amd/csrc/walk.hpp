@@ -17,6 +17,7 @@ template <typename Real>
 struct WalkResult {
   uint32_t key;     // leaf key
   uint32_t vertex;  // index into thr/ord of the min-|margin| decision
+  uint32_t ord;     // the feature that decision tests
   Real margin;      // its signed margin
 };
 
@@ -61,6 +62,7 @@ __device__ __forceinline__ void walk_many(int depth, const Node<Real> *const (&n
     v[i] = 0;
     r[i].key = 0;
     r[i].vertex = 0;
+    r[i].ord = 0;
     r[i].margin = Real(0);
     best_abs[i] = Real(0);
   }
@@ -81,6 +83,7 @@ __device__ __forceinline__ void walk_many(int depth, const Node<Real> *const (&n
         best_abs[i] = a;
         r[i].margin = m[i];
         r[i].vertex = at;
+        r[i].ord = uint32_t(n[i].ord);
       }
       r[i].key |= bit << lvl;
       v[i] = 2u * v[i] + 1u + bit;
@@ -96,6 +99,7 @@ __device__ __forceinline__ WalkResult<Real> walk(int depth, NodeFn node, Feature
   uint32_t v = 0;
   r.key = 0;
   r.vertex = 0;
+  r.ord = 0;
   r.margin = Real(0);
   Real best_abs = Real(0);
   for (int lvl = 0; lvl < depth; ++lvl) {
@@ -110,6 +114,7 @@ __device__ __forceinline__ WalkResult<Real> walk(int depth, NodeFn node, Feature
       best_abs = a;
       r.margin = m;
       r.vertex = at;
+      r.ord = uint32_t(o);
     }
     r.key |= bit << lvl;
     v = 2u * v + 1u + bit;

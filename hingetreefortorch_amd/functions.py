@@ -28,16 +28,30 @@ class _ForestFunction(torch.autograd.Function):
 
     @staticmethod
     def _forward(cls, ctx, inData, inThresholds, inOrdinals, inWeights):
-        ctx.save_for_backward(inData, inThresholds, inOrdinals, inWeights)
-        return cls._op("forward")(inData, inThresholds, inOrdinals, inWeights)
+        # When a backward pass will follow, the forward pass also keeps what its tree walks found, so that the backward
+        # does not walk again (the reference's backward re-walks, hingetree_gpu.cu:619-730; same gradients).
+        records = None
+        if any(ctx.needs_input_grad) and inData.is_cuda:
+            out, records = cls._op("forward_records")(inData, inThresholds, inOrdinals, inWeights)
+        else:
+            out = cls._op("forward")(inData, inThresholds, inOrdinals, inWeights)
+        ctx.has_records = records is not None
+        if records is not None:
+            ctx.save_for_backward(inData, inThresholds, inOrdinals, inWeights, records)
+        else:
+            ctx.save_for_backward(inData, inThresholds, inOrdinals, inWeights)
+        return out
 
     @staticmethod
     def _backward(cls, ctx, outDataGrad):
-        inData, inThresholds, inOrdinals, inWeights = ctx.saved_tensors
+        inData, inThresholds, inOrdinals, inWeights = ctx.saved_tensors[:4]
         need = ctx.needs_input_grad
-        op = cls._op("backward_deterministic" if _is_deterministic() else "backward")
-        grads = op(inData, need[0], inThresholds, need[1], inOrdinals, need[2], inWeights, need[3],
-                   outDataGrad.contiguous())
+        args = (inData, need[0], inThresholds, need[1], inOrdinals, need[2], inWeights, need[3],
+                outDataGrad.contiguous())
+        if ctx.has_records:
+            grads = cls._op("backward_records")(ctx.saved_tensors[4], _is_deterministic(), *args)
+        else:
+            grads = cls._op("backward_deterministic" if _is_deterministic() else "backward")(*args)
         return tuple(grads)
 
     # static helpers of the reference classes

@@ -172,6 +172,47 @@ def _backward(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, 
     return [dx, dthr, None, dw]
 
 
+def _forward_records(kind, inData, inThresholds, inOrdinals, inWeights):
+    """Forward that also returns the walk records for `_backward_records` (None where the library does not offer
+    them). Not part of the reference's module: its backward walks the trees again (hingetree_gpu.cu:619-730)."""
+    _common_checks([inData, inThresholds, inWeights], inOrdinals, False)
+    shape, out_sizes = _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights)
+    lib = L.load()
+    rec_bytes = lib.ht_forest_records_bytes(ctypes.byref(shape))
+    if rec_bytes == 0 or inData.numel() == 0 or inWeights.numel() == 0:
+        return _forward(kind, inData, inThresholds, inOrdinals, inWeights), None
+    with torch.cuda.device(inData.device):
+        out = torch.empty(out_sizes, dtype=inData.dtype, device=inData.device)
+        records = torch.empty(rec_bytes, dtype=torch.uint8, device=inData.device)
+        nbytes = lib.ht_forest_forward_workspace(ctypes.byref(shape))
+        ws = _workspace(nbytes, inData.device)
+        L.check(lib.ht_forest_forward_records(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals),
+                                              _ptr(inWeights), _ptr(out), _ptr(records), rec_bytes, _ptr(ws), nbytes,
+                                              _stream(inData.device)))
+    return out, records
+
+
+def _backward_records(kind, mode, records, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals,
+                      bInOrdinalsGrad, inWeights, bInWeightsGrad, outDataGrad):
+    """`_backward` from the records of `_forward_records`; inData / inThresholds / inOrdinals only give shapes."""
+    _common_checks([inData, inThresholds, inWeights, outDataGrad], inOrdinals, True)
+    if bInOrdinalsGrad:
+        _runtime("Error: Gradient on inOrdinals is requested, but inOrdinals never has a gradient.")
+    shape, _ = _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights, outDataGrad)
+    with torch.cuda.device(inData.device):
+        dx = torch.empty_like(inData) if bInDataGrad else None
+        dthr = torch.empty_like(inThresholds) if bInThresholdsGrad else None
+        dw = torch.empty_like(inWeights) if bInWeightsGrad else None
+        lib = L.load()
+        nbytes = lib.ht_forest_backward_records_workspace(ctypes.byref(shape), mode, int(bool(bInDataGrad)),
+                                                          int(bool(bInThresholdsGrad)), int(bool(bInWeightsGrad)))
+        ws = _workspace(nbytes, inData.device)
+        L.check(lib.ht_forest_backward_records(ctypes.byref(shape), _ptr(inWeights), _ptr(outDataGrad), _ptr(records),
+                                               records.numel(), _ptr(dx), _ptr(dthr), _ptr(dw), mode, _ptr(ws), nbytes,
+                                               _stream(inData.device)))
+    return [dx, dthr, None, dw]
+
+
 def _maps(kind, inData, inThresholds, inOrdinals, inWeights, want):
     _common_checks([inData, inThresholds, inWeights], inOrdinals, False)
     shape, out_sizes = _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights)
@@ -272,6 +313,24 @@ def tree_forward(inData, inThresholds, inOrdinals, inWeights):
 
 def fern_forward(inData, inThresholds, inOrdinals, inWeights):
     return _forward(L.HT_FERN, inData, inThresholds, inOrdinals, inWeights)
+
+
+def tree_forward_records(inData, inThresholds, inOrdinals, inWeights):
+    return _forward_records(L.HT_TREE, inData, inThresholds, inOrdinals, inWeights)
+
+
+def fern_forward_records(inData, inThresholds, inOrdinals, inWeights):
+    return _forward_records(L.HT_FERN, inData, inThresholds, inOrdinals, inWeights)
+
+
+def tree_backward_records(records, deterministic, *args):
+    mode = L.HT_BACKWARD_DETERMINISTIC if deterministic else L.HT_BACKWARD_ATOMIC
+    return _backward_records(L.HT_TREE, mode, records, *args)
+
+
+def fern_backward_records(records, deterministic, *args):
+    mode = L.HT_BACKWARD_DETERMINISTIC if deterministic else L.HT_BACKWARD_ATOMIC
+    return _backward_records(L.HT_FERN, mode, records, *args)
 
 
 def tree_backward(inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad, inWeights,

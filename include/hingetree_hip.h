@@ -74,6 +74,23 @@ int ht_forest_backward(const ht_forest_shape *s, const void *x, const void *thr,
                        const void *gout, void *dx, void *dthr, void *dw, int mode, void *workspace,
                        size_t workspace_bytes, void *stream);
 
+/* Training path, no counterpart in the reference (whose backward walks every tree again, hingetree_gpu.cu:619-730):
+ * ht_forest_forward_records is ht_forest_forward that also writes what its walks found -- leaf key, selected vertex,
+ * its ordinal and the signed margin of every (tree, sample) pair -- into `records`, an opaque device buffer of
+ * ht_forest_records_bytes(s) bytes that the caller keeps until the matching ht_forest_backward_records call, which
+ * computes the same gradients as ht_forest_backward from w, the upstream gradient and the records alone (x, thr and ord
+ * are not read again). ht_forest_records_bytes returns 0 for shapes the records path does not serve (use the stateless
+ * pair then). The records are only valid for the x / thr / ord of the forward call that wrote them. */
+size_t ht_forest_records_bytes(const ht_forest_shape *s);
+int ht_forest_forward_records(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord,
+                              const void *w, void *out, void *records, size_t records_bytes, void *workspace,
+                              size_t workspace_bytes, void *stream);
+size_t ht_forest_backward_records_workspace(const ht_forest_shape *s, int mode, int need_dx, int need_dthr,
+                                            int need_dw);
+int ht_forest_backward_records(const ht_forest_shape *s, const void *w, const void *gout, const void *records,
+                               size_t records_bytes, void *dx, void *dthr, void *dw, int mode, void *workspace,
+                               size_t workspace_bytes, void *stream);
+
 /* Per-(b,t,k) leaf key / signed margin + selected ordinal / per-(t,leaf) visit counts; any output may be NULL.
  * Replaces hingetree_gpu_leafmap, _marginmap, _reachability (hingetree.cpp:54-60; hingetree_gpu.cu:732-933), which
  * return the leaf map and the counts as int64 on the GPU. */

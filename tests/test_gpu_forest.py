@@ -195,3 +195,35 @@ def test_errors(dev):
         ops.tree_backward(x, True, thr, True, ordn, True, w, True, gout)
     with pytest.raises(ValueError, match="outDataGrad.shape"):
         ops.tree_backward(x, True, thr, True, ordn, False, w, True, gout[:4].contiguous())
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("case", CASES, ids=[f"c{i}" for i in range(len(CASES))])
+def test_records_path(dev, case, dtype, fern):
+    """The training path (forward that keeps its walk records, backward from the records) against the oracle and the
+    stateless operators: same forward bits, deterministic gradients bit-identical to the stateless deterministic
+    backward, atomic gradients within tolerance."""
+    B, F, Kd, T, D, Md = case
+    x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype)
+    rdx, rdthr, rdw = ho.backward(x, thr, ordn, w, gout, fern=fern)
+    gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
+    pre = "fern_" if fern else "tree_"
+    out, records = getattr(ops, pre + "forward_records")(gx, gthr, gord, gw)
+    assert torch.equal(out.cpu(), ho.forward(x, thr, ordn, w, fern))
+    if records is None:
+        pytest.skip("the library does not offer records for this shape")
+    bwd = getattr(ops, pre + "backward_records")
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    dx, dthr, dord, dw = bwd(records, False, gx, True, gthr, True, gord, False, gw, True, gg)
+    assert dord is None
+    assert rel_err(dx.cpu(), rdx) <= tol and rel_err(dthr.cpu(), rdthr) <= tol and rel_err(dw.cpu(), rdw) <= tol
+    det = bwd(records, True, gx, True, gthr, True, gord, False, gw, True, gg)
+    ref = getattr(ops, pre + "backward_deterministic")(gx, True, gthr, True, gord, False, gw, True, gg)
+    for a, b in zip(det, ref):
+        assert (a is None and b is None) or torch.equal(a, b)
+    # subsets of the gradients
+    only_w = bwd(records, False, gx, False, gthr, False, gord, False, gw, True, gg)
+    assert only_w[0] is None and only_w[1] is None and rel_err(only_w[3].cpu(), rdw) <= tol
+    only_x = bwd(records, False, gx, True, gthr, False, gord, False, gw, False, gg)
+    assert only_x[3] is None and rel_err(only_x[0].cpu(), rdx) <= tol
