@@ -104,6 +104,10 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--mode", default="atomic", choices=["atomic", "deterministic"])
     ap.add_argument("--path", default="train", choices=["train", "stateless"])
+    ap.add_argument("--other-steps", type=int, default=-1,
+                    help="timed steps of the path not selected by --path (-1: a quarter of --steps, 0: skip)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run three 1 GiB device-to-device copies (what the HBM counters are scaled against)")
     ap.add_argument("--cpu-rows", type=int, default=32768, help="rows of the batch timed on the CPU (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -117,6 +121,14 @@ def main():
         sys.exit("bench.py: no GPU visible; the HIP library is the only back-end.")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        src = torch.ones(256 * 1024 * 1024, dtype=torch.float32, device=dev)   # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "3 x copy of 1 GiB (reads 1073741824 B, writes 1073741824 B per launch)"}))
+        return
     name = args.workload
     B, F, T, depth, M, kind, _, desc = WORKLOADS[name]
     x, thr, ordn, w, gout = make_inputs(torch, name, dev)
@@ -168,7 +180,10 @@ def main():
                 sum(e[1].elapsed_time(e[2]) for e in ev) / steps)
 
     other = "stateless" if args.path == "train" else "train"
-    o_ms, o_fwd, o_bwd = run(other, max(3, args.steps // 4), 2)
+    other_steps = max(3, args.steps // 4) if args.other_steps < 0 else args.other_steps
+    o_ms = o_fwd = o_bwd = None
+    if other_steps > 0:
+        o_ms, o_fwd, o_bwd = run(other, other_steps, 2)
     ms_per_step, fwd_ms, bwd_ms = run(args.path, args.steps, args.warmup)
 
     fwd_bytes, bwd_bytes = algorithmic_bytes(B, F, T, depth, M, kind)
@@ -194,9 +209,10 @@ def main():
         "backward": {"mode": args.mode, "ms": bwd_ms, "samples_per_s": B / (bwd_ms * 1e-3),
                      "algorithmic_bytes": bwd_bytes, "hbm_frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
         "step_hbm_frac": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "other_path": {"path": other, "ms_per_step": o_ms, "forward_ms": o_fwd, "backward_ms": o_bwd,
-                       "samples_per_s": B / (o_ms * 1e-3)},
     }
+    if o_ms is not None:
+        result["other_path"] = {"path": other, "ms_per_step": o_ms, "forward_ms": o_fwd, "backward_ms": o_bwd,
+                                "samples_per_s": B / (o_ms * 1e-3)}
     if args.cpu_rows > 0:
         result["cpu_baseline"] = cpu_baseline(torch, name, x, thr, ordn, w, gout, args.cpu_rows)
     print(json.dumps(result), flush=True)
