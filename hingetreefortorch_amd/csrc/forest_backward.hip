@@ -433,6 +433,197 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// tree-stationary dW + c, specialised: float, K == 1, compact records, M a compile-time constant, TB a power of two
+// ---------------------------------------------------------------------------------------------------------------
+// Same work split and data movement as tree_kernel; what differs is that everything that does not depend on the
+// data (which lane serves which pair, every address offset, which chunk elements a lane owns) is computed once per
+// lane outside the sample loop, and M / P are compile-time constants, so a 64-pair block costs about a quarter of
+// the generic kernel's vector instructions -- the generic kernel is bound by instruction issue, not by memory.
+//
+// A block is SPT = 64 / TB consecutive samples x TB trees = 64 pairs. Records are loaded one pair per lane (lane =
+// tree rt = lane / SPT, sample rj = lane % SPT: coalesced). The block is worked off in P sub-steps of NP = 64 / P
+// pairs; in sub-step u lane group g = lane / P serves pair pp = u * NP + g (sample pp / TB, tree pp % TB: sample
+// major, so adjacent lane groups read adjacent memory) and lane li = lane % P of the group owns CNT(li) of the M
+// elements. Lane li loads the 16-byte chunk starting at its first element, except that the lanes whose chunk would
+// pass the end of the row all load the row's last four elements.
+template <int M>
+struct LeanSplit {
+  static constexpr int VE = 4;
+  static constexpr int Q = (M + VE - 1) / VE;
+  static constexpr int P = Q <= 1 ? 1 : (Q <= 2 ? 2 : (Q <= 4 ? 4 : (Q <= 8 ? 8 : 16)));  // lanes per pair
+  static constexpr int BASE = M / P, EXTRA = M % P;  // lanes li < EXTRA own BASE + 1 elements
+  static constexpr int ROUNDS = BASE + (EXTRA ? 1 : 0);
+  static constexpr int LAST = M >= VE ? M - VE : 0;  // first element of the row's last chunk
+  __host__ __device__ static constexpr int begin(int li) { return li * BASE + (li < EXTRA ? li : EXTRA); }
+  __host__ __device__ static constexpr int count(int li) { return BASE + (li < EXTRA ? 1 : 0); }
+};
+
+typedef float Float4U __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int M, bool FIXED>
+__global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d, const float *__restrict__ w,
+                                                                   const float *__restrict__ gout,
+                                                                   Records<float, true> rec, float *dw,
+                                                                   unsigned long long *dw_fixed,
+                                                                   const DetHeader *hdr, int log2_tb,
+                                                                   long long part_size, bool need_c, bool dw_atomic,
+                                                                   int num_groups) {
+  typedef LeanSplit<M> Split;
+  constexpr int P = Split::P, NP = kWave / P, VE = Split::VE;
+  typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
+  extern __shared__ __align__(16) unsigned char smem[];
+  Acc *acc = reinterpret_cast<Acc *>(smem);
+  double scale = 1.0, inv_scale = 1.0;
+  if (FIXED) {
+    if (hdr->fallback_w) dw = nullptr;
+    scale = hdr->scale_w;
+    inv_scale = hdr->inv_scale_w;
+    if (!dw && !need_c) return;
+  }
+  const int TB = 1 << log2_tb;
+  const int per_xcd = (num_groups + kNumXCDs - 1) / kNumXCDs;
+  const int group = int(blockIdx.x % kNumXCDs) * per_xcd + int(blockIdx.x / kNumXCDs);
+  if (group >= num_groups) return;
+  const int t0 = group * TB;
+  const int nt = min(TB, d.T - t0);
+  const uint32_t LM = uint32_t(d.L) * M;
+  if (dw) {
+    for (uint32_t i = threadIdx.x; i < uint32_t(nt) * LM; i += kForestThreads) acc[i] = Acc(0);
+    __syncthreads();
+  }
+  const long long s_begin = (long long)blockIdx.y * part_size;
+  const long long s_end = min(d.S, s_begin + part_size);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  constexpr int kWaves = kForestThreads / kWave;
+  const int log2_spt = 6 - log2_tb;
+  const int SPT = 1 << log2_spt;
+
+  // ---- loop-invariant lane constants
+  const int rt = lane >> log2_spt, rj = lane & (SPT - 1);  // as a loader of records
+  const int li = lane & (P - 1), grp = lane / P;           // as a member of a lane group
+  const int my_begin = Split::begin(li), my_cnt = Split::count(li);
+  const int e0 = M >= VE ? min(my_begin, Split::LAST) : 0;
+  const bool shifted = my_begin != e0;  // this lane owns chunk elements [my_begin - LAST, ...) instead of [0, ...)
+  constexpr int SHIFT = Split::begin(P - 1) - Split::LAST > 0 ? Split::begin(P - 1) - Split::LAST : 0;
+  static_assert(M < VE || Split::begin(P - 1) + Split::count(P - 1) == M, "element split must cover the row");
+  static_assert(M < VE || P < 2 || Split::begin(P - 2) <= Split::LAST, "only the last lane of a group may be shifted");
+  int src[P];        // byte index (lane * 4) of the lane that loaded the record of sub-step u's pair
+  uint32_t goff[P];  // element offset of this lane's chunk of sub-step u inside the block's gradient rows
+  uint32_t woff[P];  // (tree * L) * M + e0 of sub-step u's pair, to which key * M is added
+  int jq[P], tq[P];
+#pragma unroll
+  for (int u = 0; u < P; ++u) {
+    const int pp = u * NP + grp;
+    jq[u] = pp >> log2_tb;
+    tq[u] = pp & (TB - 1);
+    src[u] = (tq[u] * SPT + jq[u]) * 4;
+    goff[u] = (uint32_t(jq[u]) * uint32_t(d.T) + uint32_t(tq[u])) * M + e0;
+    woff[u] = uint32_t(tq[u]) * LM + e0;
+  }
+  const int my_pp = rj * TB + rt;
+  const int my_sub = my_pp / NP, my_src = (my_pp - my_sub * NP) * P * 4;
+  const float *wbase = w + (long long)t0 * LM;
+  // a lane that owns elements i < my_cnt of its chunk, at chunk positions i (+ SHIFT for the shifted lanes)
+  auto pick = [&](const Float4U &v, int i) -> float {
+    if constexpr (M < VE) {
+      return v[i];
+    } else {
+      if constexpr (SHIFT == 0) return v[i];
+      const int k = i + SHIFT;
+      return shifted ? v[k < VE ? k : VE - 1] : v[i];
+    }
+  };
+  auto load_chunk = [&](const float *p, bool stream) -> Float4U {
+    Float4U v;
+    if constexpr (M >= VE) {
+      v = stream ? __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(p))
+                 : *reinterpret_cast<const Float4U *>(p);
+    } else {
+#pragma unroll
+      for (int k = 0; k < VE; ++k) v[k] = k < M ? p[k] : 0.f;
+    }
+    return v;
+  };
+
+  const long long first = s_begin + (long long)wave * SPT;
+  for (long long sblk = first; sblk < s_end; sblk += (long long)kWaves * SPT) {
+    const int ns = int(min<long long>(SPT, s_end - sblk));
+    const bool full = ns == SPT && nt == TB;  // wave uniform
+    const bool have = full || (rt < nt && rj < ns);
+    const long long at = (long long)(t0 + (have ? rt : 0)) * d.S + sblk + (have ? rj : 0);
+    const uint32_t a_r = rec.a[at];
+    const float mg_r = rec.margin[at];
+    const float *gbase = gout + (sblk * d.T + t0) * M;
+    Float4U gv[P], wv[P];
+    bool on[P];
+    float mg[P];
+    uint32_t rel[P];
+#pragma unroll
+    for (int u = 0; u < P; ++u) {
+      on[u] = full || (jq[u] < ns && tq[u] < nt);
+      gv[u] = load_chunk(gbase + (on[u] ? goff[u] : uint32_t(e0)), true);
+    }
+#pragma unroll
+    for (int u = 0; u < P; ++u) {
+      const uint32_t key = uint32_t(__builtin_amdgcn_ds_bpermute(src[u], int(a_r))) & 0xffffu;
+      mg[u] = __int_as_float(__builtin_amdgcn_ds_bpermute(src[u], __float_as_int(mg_r)));
+      rel[u] = woff[u] + key * M;
+      if (need_c) wv[u] = load_chunk(wbase + (on[u] ? rel[u] : uint32_t(e0)), false);
+    }
+    float c_mine = 0.f;
+#pragma unroll
+    for (int u = 0; u < P; ++u) {
+      if (dw && on[u]) {
+        Acc *cell = acc + (rel[u] - e0 + my_begin);
+#pragma unroll
+        for (int i = 0; i < Split::ROUNDS; ++i) {
+          if (i < my_cnt) {
+            const float term = ht_abs(mg[u]) * pick(gv[u], i);
+            if (FIXED)
+              atomicAdd(reinterpret_cast<unsigned long long *>(cell) + i, to_fixed(double(term), scale));
+            else
+              atomicAdd(reinterpret_cast<double *>(cell) + i, double(term));
+          }
+        }
+      }
+      if (need_c) {
+        float partial = 0.f;
+#pragma unroll
+        for (int i = 0; i < Split::ROUNDS; ++i)
+          if (i < my_cnt) partial = __builtin_fmaf(pick(wv[u], i), pick(gv[u], i), partial);
+        partial = group_sum<float>(on[u] ? partial : 0.f, P);
+        const float got = __int_as_float(__builtin_amdgcn_ds_bpermute(my_src, __float_as_int(partial)));
+        if (my_sub == u) c_mine = got;
+      }
+    }
+    if (need_c && have) rec.c[at] = ht_sign(mg_r) * c_mine;
+  }
+  if (dw) {
+    __syncthreads();
+    float *dst = dw + (long long)t0 * LM;
+    const uint32_t n = uint32_t(nt) * LM;
+    if (FIXED) {
+      const unsigned long long *q = reinterpret_cast<const unsigned long long *>(acc);
+      if (dw_atomic) {
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads)
+          if (q[i] != 0ull) atomicAdd(dw_fixed + (long long)t0 * LM + i, q[i]);
+      } else {
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = from_fixed<float>(q[i], inv_scale);
+      }
+    } else {
+      const double *q = reinterpret_cast<const double *>(acc);
+      if (dw_atomic) {
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads)
+          if (q[i] != 0.0) atomicAdd(dst + i, float(q[i]));
+      } else {
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = float(q[i]);
+      }
+    }
+  }
+}
+
 // dThr[t, v] = sum over samples with selected vertex v of -c. One workgroup per tree (x sample parts).
 template <typename Real, bool COMPACT, bool FIXED>
 __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dthr,
@@ -846,6 +1037,28 @@ template <typename Real, bool COMPACT, bool FIXED>
 int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, const Real *gout,
                        Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
                        bool need_c, hipStream_t stream) {
+  if constexpr (std::is_same<Real, float>::value && COMPACT) {
+    // the specialised kernel: contiguous rows, a power-of-two tree group, 32-bit offsets inside a block and a group
+    int log2_tb = 0;
+    while ((1 << (log2_tb + 1)) <= p.TB) ++log2_tb;
+    const bool fits = d.K == 1 && (1 << log2_tb) == p.TB && p.TB <= kWave &&
+                      (long long)kWave * d.T * d.M < (1ll << 31) && (long long)p.TB * d.L * d.M < (1ll << 31);
+    if (fits && (d.M == 10 || d.M == 1)) {
+      HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(d.M == 10 ? (const void *)tree_lean_kernel<10, FIXED>
+                                                                                : (const void *)tree_lean_kernel<1, FIXED>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(p.lds)));
+      const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
+      const dim3 grid((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts);
+      if (d.M == 10)
+        hipLaunchKernelGGL((tree_lean_kernel<10, FIXED>), grid, dim3(kForestThreads), p.lds, stream, d, w, gout, rec, dw,
+                           dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups);
+      else
+        hipLaunchKernelGGL((tree_lean_kernel<1, FIXED>), grid, dim3(kForestThreads), p.lds, stream, d, w, gout, rec, dw,
+                           dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups);
+      HT_LAUNCH_CHECK("forest backward (trees)");
+      return HT_OK;
+    }
+  }
   constexpr int VE = 16 / sizeof(Real);
   const int Q = d.M >= VE ? (d.M + VE - 1) / VE : 1;  // 16-byte chunks in one pair's values
   int P = 1;                                          // lanes per pair

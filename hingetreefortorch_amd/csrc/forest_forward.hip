@@ -8,6 +8,8 @@
 // (|margin|, leaf) in LDS, and then the workgroup writes the pass' outputs with the lane index running along the
 // contiguous (tree, m) -- or for K > 1 the contiguous (inner position, m) -- axis of `out`, so the dominant store
 // traffic is emitted as full-width rows.
+#include <type_traits>
+
 #include "forest_tile.hpp"
 #include "records.hpp"
 
@@ -140,6 +142,339 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// row kernel (K == 1): wavefront-autonomous walk + output
+// ---------------------------------------------------------------------------------------------------------------
+// Two-level vertices ("quads") of a float tree whose ordinals fit 10 bits: the vertex of an even level together with
+// its two children in one 16-byte word, so a walk costs one vector load per TWO levels. The vector memory pipeline
+// charges a divergent load per instruction and per distinct line, not per byte, which makes this the cheapest form
+// of the data-dependent vertex stream. Quads of level pair k (levels 2k, 2k+1) start at (4^k - 1) / 3; quad i of a
+// pair holds vertex (2^(2k) - 1) + i and its grandchildren are quads 4i .. 4i+3 of the next pair.
+struct __align__(16) QuadNode {
+  float thr, thr_left, thr_right;
+  uint32_t ords;  // ordinal | left ordinal << 10 | right ordinal << 20
+};
+constexpr int kQuadOrdinalBits = 10;
+
+static inline long long quads_per_tree(int depth) {
+  long long n = 0, level = 1;
+  for (int l = 0; l < depth; l += 2) {
+    n += level;
+    level *= 4;
+  }
+  return n;
+}
+
+__global__ __launch_bounds__(256) void pack_quads_kernel(const float *__restrict__ thr, const int64_t *__restrict__ ord,
+                                                         QuadNode *__restrict__ quads, int T, int V, int NQ, int F) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long long)T * NQ) return;
+  const int t = int(i / NQ), q = int(i - (long long)t * NQ);
+  int k = 0, base = 0, width = 1;
+  while (q >= base + width) {
+    base += width;
+    width *= 4;
+    ++k;
+  }
+  const long long v = ((1ll << (2 * k)) - 1) + (q - base);
+  const float *th = thr + (long long)t * V;
+  const int64_t *od = ord + (long long)t * V;
+  QuadNode n;
+  n.thr = th[v];
+  uint32_t o = uint32_t(clamp_ordinal(od[v], F));
+  n.thr_left = n.thr_right = 0.f;
+  if (2 * v + 2 < V) {
+    n.thr_left = th[2 * v + 1];
+    n.thr_right = th[2 * v + 2];
+    o |= uint32_t(clamp_ordinal(od[2 * v + 1], F)) << kQuadOrdinalBits;
+    o |= uint32_t(clamp_ordinal(od[2 * v + 2], F)) << (2 * kQuadOrdinalBits);
+  }
+  n.ords = o;
+  quads[i] = n;
+}
+
+// N interleaved walks over quads; xs_j = this lane's column of the feature-major sample tile (pitch BT).
+template <int N, int BT>
+__device__ __forceinline__ void walk_quads(int depth, const QuadNode *const (&quads)[N], const float *xs_j,
+                                           WalkResult<float> (&r)[N]) {
+  uint32_t idx[N];
+  float best_abs[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    idx[i] = 0;
+    r[i].key = 0;
+    r[i].vertex = 0;
+    r[i].ord = 0;
+    r[i].margin = 0.f;
+    best_abs[i] = 0.f;
+  }
+  uint32_t base = 0, width = 1;  // first quad / number of quads of the current level pair
+  constexpr uint32_t kMask = (1u << kQuadOrdinalBits) - 1;
+  for (int lvl = 0; lvl < depth; lvl += 2) {
+    QuadNode n[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) n[i] = quads[i][base + idx[i]];
+    float m0[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) m0[i] = xs_j[(n[i].ords & kMask) * BT] - n[i].thr;
+    const uint32_t first = (1u << lvl) - 1u;  // heap index of the level's first vertex
+    const bool two = lvl + 1 < depth;
+    float m1[N];
+    uint32_t o1[N], b0[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      b0[i] = (m0[i] > 0.f) ? 1u : 0u;
+      const float t1 = b0[i] ? n[i].thr_right : n[i].thr_left;
+      o1[i] = (n[i].ords >> (b0[i] ? 2 * kQuadOrdinalBits : kQuadOrdinalBits)) & kMask;
+      m1[i] = two ? xs_j[o1[i] * BT] - t1 : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const uint32_t v0 = first + idx[i];
+      const float a0 = ht_abs(m0[i]);
+      if (lvl == 0 || a0 < best_abs[i]) {
+        best_abs[i] = a0;
+        r[i].margin = m0[i];
+        r[i].vertex = v0;
+        r[i].ord = n[i].ords & kMask;
+      }
+      r[i].key |= b0[i] << lvl;
+      if (two) {
+        const uint32_t b1 = (m1[i] > 0.f) ? 1u : 0u;
+        const float a1 = ht_abs(m1[i]);
+        if (a1 < best_abs[i]) {
+          best_abs[i] = a1;
+          r[i].margin = m1[i];
+          r[i].vertex = 2u * v0 + 1u + b0[i];
+          r[i].ord = o1[i];
+        }
+        r[i].key |= b1 << (lvl + 1);
+        idx[i] = 4u * idx[i] + 2u * b0[i] + b1;
+      }
+    }
+    base += width;
+    width *= 4u;
+  }
+}
+
+constexpr int kRowIlp = 4;     // trees walked concurrently per lane
+constexpr int kRowUnroll = 5;  // output vectors per lane whose weight gathers are in flight together
+
+// One workgroup = one tile of BT samples (all features in LDS, feature major) x a range of trees, like
+// forward_kernel, but every wavefront works on its own: lanes = BT samples x 64/BT tree slots, each lane walks
+// kRowIlp trees, parks (|margin|, leaf) in a wavefront-private piece of LDS, and the same wavefront then writes the
+// TPW = 64/BT * kRowIlp trees' outputs of its samples, lanes running along the contiguous (tree, m) axis of a row.
+// There is no workgroup barrier after the tile load, so at any moment some wavefronts of a CU walk (vertex gathers)
+// while others store, and the two phases overlap instead of alternating across the whole device.
+//
+// QUAD selects two-level vertices (float trees, F <= 1024); otherwise Node<Real> is walked level by level.
+// GW = elements per weight gather and per store (divides M). RECORD: also write the walk records.
+template <typename Real, bool FERN, bool QUAD, int BT, int GW, bool RECORD, bool COMPACT>
+__global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims d, const Real *__restrict__ x,
+                                                                      const void *__restrict__ vertices, int NQ,
+                                                                      const Real *__restrict__ w,
+                                                                      Real *__restrict__ out,
+                                                                      Records<Real, COMPACT> rec,
+                                                                      int trees_per_block, FastDiv div_m,
+                                                                      FastDiv div_u_full) {
+  typedef Real Vec __attribute__((ext_vector_type(GW)));
+  constexpr int NT = kForestThreads;
+  constexpr int kWaves = NT / kWave;
+  constexpr int SLOTS = kWave / BT;        // tree slots of a wavefront
+  constexpr int TPW = SLOTS * kRowIlp;     // trees per wavefront step
+  constexpr int LDP = TPW + 1;             // odd pitch of the parked results, [sample][tree]
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *xs = reinterpret_cast<Real *>(smem);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  Real *p_abs = xs + size_t(d.F) * BT + size_t(wave) * (BT * LDP);
+  uint16_t *p_key = reinterpret_cast<uint16_t *>(xs + size_t(d.F) * BT + size_t(kWaves) * (BT * LDP)) +
+                    size_t(wave) * (BT * LDP);
+
+  const long long s0 = (long long)blockIdx.x * BT;
+  load_tile<Real, BT, NT>(xs, x, d, s0);
+  __syncthreads();
+
+  const int j = lane % BT, slot = lane / BT;
+  const long long s = s0 + j;
+  const bool live = s < d.S;
+  const int n_live = int(min<long long>(BT, d.S - s0));
+  const Real *xs_j = xs + j;
+  const int t_begin = blockIdx.y * trees_per_block;
+  const int t_end = min(d.T, t_begin + trees_per_block);
+  const uint32_t TM = uint32_t(d.T) * uint32_t(d.M);
+
+  for (int tb = t_begin + wave * TPW; tb < t_end; tb += kWaves * TPW) {
+    // ---- walk: this lane's sample through trees tb + slot + i * SLOTS
+    {
+      WalkResult<Real> r[kRowIlp];
+      int t[kRowIlp];
+#pragma unroll
+      for (int i = 0; i < kRowIlp; ++i) t[i] = min(tb + slot + i * SLOTS, t_end - 1);  // surplus slots re-walk, unused
+#ifdef HT_AB_NOWALK
+      for (int i = 0; i < kRowIlp; ++i) { r[i].key = (t[i] * 2654435761u + uint32_t(s) * 40503u) >> 22; r[i].margin = xs_j[(t[i] & 1023) * BT]; r[i].vertex = 1; r[i].ord = 2; }
+#else
+      if constexpr (QUAD) {
+        const QuadNode *qn[kRowIlp];
+#pragma unroll
+        for (int i = 0; i < kRowIlp; ++i) qn[i] = static_cast<const QuadNode *>(vertices) + (long long)t[i] * NQ;
+        walk_quads<kRowIlp, BT>(d.depth, qn, xs_j, r);
+      } else {
+        const Node<Real> *nd[kRowIlp];
+#pragma unroll
+        for (int i = 0; i < kRowIlp; ++i) nd[i] = static_cast<const Node<Real> *>(vertices) + (long long)t[i] * d.V;
+        walk_many<Real, FERN, kRowIlp>(d.depth, nd, [&](int, int f) { return xs_j[f * BT]; }, r);
+      }
+#endif
+#pragma unroll
+      for (int i = 0; i < kRowIlp; ++i) {
+        p_abs[j * LDP + slot + i * SLOTS] = ht_abs(r[i].margin);
+        p_key[j * LDP + slot + i * SLOTS] = uint16_t(r[i].key);
+        if (RECORD && live && tb + slot + i * SLOTS < t_end)
+          rec.put((long long)(tb + slot + i * SLOTS) * d.S + s, r[i].key, r[i].vertex, r[i].ord, r[i].margin);
+      }
+    }
+    // the parked results are read by other lanes of this wavefront only
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // ---- output: out[s0 + jj, tb .. tb + nt, 0 .. M) is one contiguous run per sample
+    const int nt = min(TPW, t_end - tb);
+    const int U = nt * d.M / GW;  // vectors per sample
+    FastDiv div_u = div_u_full;   // divisor TPW * M / GW, prepared by the host
+    if (nt != TPW) div_u = FastDiv(U);
+    const int total = n_live * U;
+    Real *obase = out + ((long long)s0 * d.T + tb) * d.M;
+    const Real *wbase = w + (long long)tb * d.L * d.M;
+    for (int u0 = lane; u0 < total; u0 += kWave * kRowUnroll) {
+      Real a[kRowUnroll];
+      Vec wv[kRowUnroll];
+      uint32_t off[kRowUnroll];
+#pragma unroll
+      for (int q = 0; q < kRowUnroll; ++q) {
+        const int u = min(u0 + q * kWave, total - 1);
+        const int jj = div_u.div(u);
+        const int e = (u - jj * U) * GW;
+        const int tt = div_m.div(e), m = e - tt * d.M;
+        const uint32_t key = p_key[jj * LDP + tt];
+        a[q] = p_abs[jj * LDP + tt];
+#ifdef HT_AB_NOGATHER
+        for (int i = 0; i < GW; ++i) wv[q][i] = Real(key + m);
+#else
+        wv[q] = *reinterpret_cast<const Vec *>(wbase + (uint32_t(tt) * uint32_t(d.L) + key) * uint32_t(d.M) + m);
+#endif
+        off[q] = uint32_t(jj) * TM + uint32_t(e);
+      }
+#pragma unroll
+      for (int q = 0; q < kRowUnroll; ++q) {
+        if (u0 + q * kWave < total) {
+          Vec o;
+#pragma unroll
+          for (int i = 0; i < GW; ++i) o[i] = a[q] * wv[q][i];
+#ifdef HT_AB_NOSTORE
+          if (o[0] == Real(123.456)) 
+#endif
+#ifdef HT_AB_T
+          *reinterpret_cast<Vec *>(obase + off[q]) = o;
+#else
+          // streaming store: the output is written once and not read here, so it should not displace the vertices
+          // and leaf weights that the gathers keep re-reading from L2 (measured: 1.45 -> 1.17 ms at the headline shape)
+          __builtin_nontemporal_store(o, reinterpret_cast<Vec *>(obase + off[q]));
+#endif
+        }
+      }
+    }
+    // the next step's parking writes follow this step's reads in program order; the LDS serves a wavefront's
+    // requests in order
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+template <typename Real>
+static inline size_t rows_lds_bytes(int F, int bt) {
+  const int tpw = kWave / bt * kRowIlp;
+  return size_t(F) * bt * sizeof(Real) +
+         size_t(kForestThreads / kWave) * bt * (tpw + 1) * (sizeof(Real) + sizeof(uint16_t));
+}
+
+template <typename Real>
+static inline int pick_rows_tile(int F) {
+  const int candidates[4] = {64, 32, 16, 8};
+  for (int bt : candidates)
+    if (rows_lds_bytes<Real>(F, bt) <= size_t(kLdsBytes)) return bt;
+  return 0;
+}
+
+// Shapes the row kernel serves: contiguous rows (K == 1), 16-bit parked keys, 32-bit element offsets inside a
+// wavefront step, and a sample tile that fits LDS.
+template <typename Real>
+static inline bool rows_ok(const ForestDims &d) {
+  if (d.K != 1 || d.depth > 16 || d.M < 1) return false;
+  if ((long long)d.T * d.M * 64 >= (1ll << 31)) return false;
+  if ((long long)kWave * kRowIlp * d.L * d.M >= (1ll << 31)) return false;
+  return pick_rows_tile<Real>(d.F) != 0;
+}
+
+template <typename Real>
+static inline bool quads_ok(const ForestDims &d, bool fern) {
+  return std::is_same<Real, float>::value && !fern && d.F <= (1 << kQuadOrdinalBits) &&
+         (long long)d.T * quads_per_tree(d.depth) < (1ll << 31);
+}
+
+template <typename Real, bool FERN, bool QUAD, int BT, int GW, bool RECORD, bool COMPACT>
+int launch_rows(const ForestDims &d, const Real *x, const void *vertices, const Real *w, Real *out, void *records,
+                hipStream_t stream) {
+  constexpr int TPW = kWave / BT * kRowIlp;
+  constexpr int TP = kForestThreads / kWave * TPW;
+  const size_t lds = rows_lds_bytes<Real>(d.F, BT);
+  const long long tiles = (d.S + BT - 1) / BT;
+  int trees_per_block, gy;
+  split_trees(tiles, d.T, TP, &trees_per_block, &gy);
+  if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
+  auto kernel = forward_rows_kernel<Real, FERN, QUAD, BT, GW, RECORD, COMPACT>;
+  Records<Real, COMPACT> rec{};
+  if (RECORD) rec = carve_records<Real, COMPACT>(d, records, nullptr);
+  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   int(lds)));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, vertices,
+                     int(quads_per_tree(d.depth)), w, out, rec, trees_per_block, FastDiv(d.M),
+                     FastDiv(TPW * d.M / GW));
+  HT_LAUNCH_CHECK("forest forward (rows)");
+  return HT_OK;
+}
+
+template <typename Real, bool FERN, bool QUAD, int BT, int GW>
+int launch_rows_rec(const ForestDims &d, const Real *x, const void *vertices, const Real *w, Real *out, void *records,
+                    hipStream_t stream) {
+  if (!records) return launch_rows<Real, FERN, QUAD, BT, GW, false, true>(d, x, vertices, w, out, records, stream);
+  if (compact_ok(d)) return launch_rows<Real, FERN, QUAD, BT, GW, true, true>(d, x, vertices, w, out, records, stream);
+  return launch_rows<Real, FERN, QUAD, BT, GW, true, false>(d, x, vertices, w, out, records, stream);
+}
+
+template <typename Real, bool FERN, bool QUAD, int BT>
+int launch_rows_gw(const ForestDims &d, const Real *x, const void *vertices, const Real *w, Real *out, void *records,
+                   hipStream_t stream) {
+  const uintptr_t pw = reinterpret_cast<uintptr_t>(w), po = reinterpret_cast<uintptr_t>(out);
+  if (d.M % 4 == 0 && pw % (4 * sizeof(Real)) == 0 && po % (4 * sizeof(Real)) == 0)
+    return launch_rows_rec<Real, FERN, QUAD, BT, 4>(d, x, vertices, w, out, records, stream);
+  if (d.M % 2 == 0 && pw % (2 * sizeof(Real)) == 0 && po % (2 * sizeof(Real)) == 0)
+    return launch_rows_rec<Real, FERN, QUAD, BT, 2>(d, x, vertices, w, out, records, stream);
+  return launch_rows_rec<Real, FERN, QUAD, BT, 1>(d, x, vertices, w, out, records, stream);
+}
+
+template <typename Real, bool FERN, bool QUAD>
+int dispatch_rows(const ForestDims &d, const Real *x, const void *vertices, const Real *w, Real *out, void *records,
+                  hipStream_t stream) {
+  switch (pick_rows_tile<Real>(d.F)) {
+    case 64: return launch_rows_gw<Real, FERN, QUAD, 64>(d, x, vertices, w, out, records, stream);
+    case 32: return launch_rows_gw<Real, FERN, QUAD, 32>(d, x, vertices, w, out, records, stream);
+    case 16: return launch_rows_gw<Real, FERN, QUAD, 16>(d, x, vertices, w, out, records, stream);
+    default: return launch_rows_gw<Real, FERN, QUAD, 8>(d, x, vertices, w, out, records, stream);
+  }
+}
+
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
 int launch_forward_rec(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
                        void *records, hipStream_t stream);
@@ -232,16 +567,39 @@ int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *d
 }
 
 template <typename Real>
+static size_t quads_bytes(const ForestDims &d) {
+  return align_up(size_t(d.T) * size_t(quads_per_tree(d.depth)) * sizeof(QuadNode), 256);
+}
+
+template <typename Real>
 size_t forest_forward_workspace(const ForestDims &d) {
-  return packed_nodes_bytes<Real>(d);
+  const size_t nodes = packed_nodes_bytes<Real>(d);
+  const size_t quads = (quads_ok<Real>(d, false) && rows_ok<Real>(d)) ? quads_bytes<Real>(d) : 0;
+  return nodes > quads ? nodes : quads;
 }
 
 template <typename Real>
 int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
                    Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream) {
   if (d.S == 0 || d.T == 0) return HT_OK;
-  if (ws == nullptr || ws_bytes < packed_nodes_bytes<Real>(d))
+  if (ws == nullptr || ws_bytes < forest_forward_workspace<Real>(d))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the forward pass.");
+  if (rows_ok<Real>(d)) {
+    if constexpr (std::is_same<Real, float>::value) {
+      if (quads_ok<Real>(d, fern)) {
+        const int NQ = int(quads_per_tree(d.depth));
+        const long long n = (long long)d.T * NQ;
+        hipLaunchKernelGGL(pack_quads_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, thr, ord,
+                           static_cast<QuadNode *>(ws), d.T, d.V, NQ, d.F);
+        HT_LAUNCH_CHECK("pack two-level vertices");
+        return dispatch_rows<Real, false, true>(d, x, ws, w, out, records, stream);
+      }
+    }
+    int rc = pack_nodes<Real>(d, thr, ord, ws, stream);
+    if (rc != HT_OK) return rc;
+    return fern ? dispatch_rows<Real, true, false>(d, x, ws, w, out, records, stream)
+                : dispatch_rows<Real, false, false>(d, x, ws, w, out, records, stream);
+  }
   int rc = pack_nodes<Real>(d, thr, ord, ws, stream);
   if (rc != HT_OK) return rc;
   const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
