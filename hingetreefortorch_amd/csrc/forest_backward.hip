@@ -436,30 +436,53 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
 // ---------------------------------------------------------------------------------------------------------------
 // tree-stationary dW + c, specialised: float, K == 1, compact records, M a compile-time constant, TB a power of two
 // ---------------------------------------------------------------------------------------------------------------
-// Same work split and data movement as tree_kernel; what differs is that everything that does not depend on the
-// data (which lane serves which pair, every address offset, which chunk elements a lane owns) is computed once per
-// lane outside the sample loop, and M / P are compile-time constants, so a 64-pair block costs about a quarter of
-// the generic kernel's vector instructions -- the generic kernel is bound by instruction issue, not by memory.
+// Same work split as tree_kernel; what differs is that everything that does not depend on the data (which lane
+// serves which pair, every address offset, which chunk elements a lane owns) is computed once per lane outside the
+// sample loop, M / P are compile-time constants, and a lane group finds its records inside its own quad, so a 64-pair
+// block costs a fraction of the generic kernel's vector and LDS instructions -- the generic kernel is bound by
+// instruction issue and by the LDS pipeline (atomics + cross-lane permutes), not by memory.
 //
-// A block is SPT = 64 / TB consecutive samples x TB trees = 64 pairs. Records are loaded one pair per lane (lane =
-// tree rt = lane / SPT, sample rj = lane % SPT: coalesced). The block is worked off in P sub-steps of NP = 64 / P
-// pairs; in sub-step u lane group g = lane / P serves pair pp = u * NP + g (sample pp / TB, tree pp % TB: sample
-// major, so adjacent lane groups read adjacent memory) and lane li = lane % P of the group owns CNT(li) of the M
-// elements. Lane li loads the 16-byte chunk starting at its first element, except that the lanes whose chunk would
-// pass the end of the row all load the row's last four elements.
+// A block is SPT = 64 / TB consecutive samples x TB trees = 64 pairs. It is worked off in P sub-steps of 64 / P
+// pairs; lane li = lane % P of a lane group owns CNT(li) of a pair's M elements and loads the 16-byte chunk that
+// starts at its first element, except that the last lane's chunk is the row's last four elements. A record reaches
+// the lanes of its group through a DPP quad broadcast (a plain vector instruction) instead of an LDS permute.
 template <int M>
 struct LeanSplit {
   static constexpr int VE = 4;
   static constexpr int Q = (M + VE - 1) / VE;
-  static constexpr int P = Q <= 1 ? 1 : (Q <= 2 ? 2 : (Q <= 4 ? 4 : (Q <= 8 ? 8 : 16)));  // lanes per pair
-  static constexpr int BASE = M / P, EXTRA = M % P;  // lanes li < EXTRA own BASE + 1 elements
+  static constexpr int P = Q <= 1 ? 1 : (Q <= 2 ? 2 : 4);  // lanes per pair (M <= 16)
+  static constexpr int BASE = M / P, EXTRA = M % P;         // lanes li < EXTRA own BASE + 1 elements
   static constexpr int ROUNDS = BASE + (EXTRA ? 1 : 0);
-  static constexpr int LAST = M >= VE ? M - VE : 0;  // first element of the row's last chunk
+  static constexpr int LAST = M >= VE ? M - VE : 0;         // first element of the row's last chunk
   __host__ __device__ static constexpr int begin(int li) { return li * BASE + (li < EXTRA ? li : EXTRA); }
   __host__ __device__ static constexpr int count(int li) { return BASE + (li < EXTRA ? 1 : 0); }
+  // chunk position of the last lane's first own element
+  static constexpr int SHIFT = (M >= VE && begin(P - 1) > LAST) ? begin(P - 1) - LAST : 0;
 };
 
 typedef float Float4U __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+// Value of lane (group base + U) of each aligned group of P lanes (P <= 4), to every lane of the group.
+template <int P, int U>
+__device__ __forceinline__ int group_bcast(int v) {
+  if constexpr (P == 1) {
+    return v;
+  } else if constexpr (P == 2) {
+    constexpr int ctrl = U | (U << 2) | ((2 + U) << 4) | ((2 + U) << 6);  // quad_perm [U, U, 2+U, 2+U]
+    return __builtin_amdgcn_update_dpp(0, v, ctrl, 0xF, 0xF, true);
+  } else {
+    constexpr int ctrl = U * 0x55;  // quad_perm [U, U, U, U]
+    return __builtin_amdgcn_update_dpp(0, v, ctrl, 0xF, 0xF, true);
+  }
+}
 
 template <int M, bool FIXED>
 __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d, const float *__restrict__ w,
@@ -470,7 +493,11 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
                                                                    long long part_size, bool need_c, bool dw_atomic,
                                                                    int num_groups) {
   typedef LeanSplit<M> Split;
-  constexpr int P = Split::P, NP = kWave / P, VE = Split::VE;
+  constexpr int P = Split::P, VE = Split::VE, ROUNDS = Split::ROUNDS, SHIFT = Split::SHIFT;
+  static_assert(M <= 16, "at most four lanes per pair");
+  static_assert(M < VE || Split::begin(P - 1) + Split::count(P - 1) == M, "element split must cover the row");
+  static_assert(M < VE || P < 2 || Split::begin(P - 2) <= Split::LAST, "only the last lane of a group is shifted");
+  static_assert(SHIFT + Split::count(P - 1) <= VE, "the last lane's elements lie inside its chunk");
   typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
   extern __shared__ __align__(16) unsigned char smem[];
   Acc *acc = reinterpret_cast<Acc *>(smem);
@@ -497,42 +524,46 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   constexpr int kWaves = kForestThreads / kWave;
-  const int log2_spt = 6 - log2_tb;
-  const int SPT = 1 << log2_spt;
+  const int SPT = kWave >> log2_tb;
 
   // ---- loop-invariant lane constants
-  const int rt = lane >> log2_spt, rj = lane & (SPT - 1);  // as a loader of records
-  const int li = lane & (P - 1), grp = lane / P;           // as a member of a lane group
+  const int li = lane & (P - 1), grp = lane / P;
   const int my_begin = Split::begin(li), my_cnt = Split::count(li);
   const int e0 = M >= VE ? min(my_begin, Split::LAST) : 0;
-  const bool shifted = my_begin != e0;  // this lane owns chunk elements [my_begin - LAST, ...) instead of [0, ...)
-  constexpr int SHIFT = Split::begin(P - 1) - Split::LAST > 0 ? Split::begin(P - 1) - Split::LAST : 0;
-  static_assert(M < VE || Split::begin(P - 1) + Split::count(P - 1) == M, "element split must cover the row");
-  static_assert(M < VE || P < 2 || Split::begin(P - 2) <= Split::LAST, "only the last lane of a group may be shifted");
-  int src[P];        // byte index (lane * 4) of the lane that loaded the record of sub-step u's pair
-  uint32_t goff[P];  // element offset of this lane's chunk of sub-step u inside the block's gradient rows
-  uint32_t woff[P];  // (tree * L) * M + e0 of sub-step u's pair, to which key * M is added
-  int jq[P], tq[P];
-#pragma unroll
-  for (int u = 0; u < P; ++u) {
-    const int pp = u * NP + grp;
-    jq[u] = pp >> log2_tb;
-    tq[u] = pp & (TB - 1);
-    src[u] = (tq[u] * SPT + jq[u]) * 4;
-    goff[u] = (uint32_t(jq[u]) * uint32_t(d.T) + uint32_t(tq[u])) * M + e0;
-    woff[u] = uint32_t(tq[u]) * LM + e0;
-  }
-  const int my_pp = rj * TB + rt;
-  const int my_sub = my_pp / NP, my_src = (my_pp - my_sub * NP) * P * 4;
+  const bool shifted = SHIFT != 0 && li == P - 1;
+  // Records are loaded one pair per lane, coalesced: lane = tree * SPT + sample. P divides SPT (TB <= 16), so the P
+  // lanes of a group hold P consecutive samples of ONE tree, and those are the pairs the group serves in its P
+  // sub-steps: sub-step u works on the pair whose record lane (group base + u) loaded.
+  const int log2_spt = 6 - log2_tb;
+  const int tq = lane >> log2_spt;                     // tree of this lane's group (and of its record)
+  const int jq0 = (grp * P) & (SPT - 1);               // sample of the group's sub-step 0
+  const int rec_t = tq, rec_j = jq0 + li;              // the pair whose record this lane loads and whose c it stores
+  const uint32_t goff = (uint32_t(jq0) * uint32_t(d.T) + uint32_t(tq)) * M + e0;  // this lane's chunk, sub-step 0
+  const uint32_t gstep = uint32_t(d.T) * M;                                        // ... and per further sub-step
+  const uint32_t woff = uint32_t(tq) * LM + e0;  // (tree * L) * M + e0, to which key * M is added
+  constexpr int jstep = 1;
   const float *wbase = w + (long long)t0 * LM;
-  // a lane that owns elements i < my_cnt of its chunk, at chunk positions i (+ SHIFT for the shifted lanes)
-  auto pick = [&](const Float4U &v, int i) -> float {
-    if constexpr (M < VE) {
-      return v[i];
+  const uint32_t key_mask = rec.key_mask();
+
+  // The ROUNDS elements this lane owns, out of a loaded chunk: positions 0.. for all lanes but the shifted one, which
+  // takes SHIFT.. instead. The empty asm keeps the four components apart, so each own element costs one select with
+  // a loop-invariant condition.
+  auto own_elements = [&](Float4U v, float (&e)[ROUNDS]) {
+    float c0 = v[0], c1 = v[1], c2 = v[2], c3 = v[3];
+    if constexpr (SHIFT != 0) {
+      asm volatile("" : "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3));
+      static_for<ROUNDS>([&](auto i_tag) {
+        constexpr int i = decltype(i_tag)::value;
+        constexpr int k = i + SHIFT < VE ? i + SHIFT : VE - 1;
+        const float plain = i == 0 ? c0 : (i == 1 ? c1 : (i == 2 ? c2 : c3));
+        const float moved = k == 0 ? c0 : (k == 1 ? c1 : (k == 2 ? c2 : c3));
+        e[i] = shifted ? moved : plain;
+      });
     } else {
-      if constexpr (SHIFT == 0) return v[i];
-      const int k = i + SHIFT;
-      return shifted ? v[k < VE ? k : VE - 1] : v[i];
+      static_for<ROUNDS>([&](auto i_tag) {
+        constexpr int i = decltype(i_tag)::value;
+        e[i] = i == 0 ? c0 : (i == 1 ? c1 : (i == 2 ? c2 : c3));
+      });
     }
   };
   auto load_chunk = [&](const float *p, bool stream) -> Float4U {
@@ -547,40 +578,51 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     return v;
   };
 
-  const long long first = s_begin + (long long)wave * SPT;
-  for (long long sblk = first; sblk < s_end; sblk += (long long)kWaves * SPT) {
-    const int ns = int(min<long long>(SPT, s_end - sblk));
-    const bool full = ns == SPT && nt == TB;  // wave uniform
-    const bool have = full || (rt < nt && rj < ns);
-    const long long at = (long long)(t0 + (have ? rt : 0)) * d.S + sblk + (have ? rj : 0);
-    const uint32_t a_r = rec.a[at];
-    const float mg_r = rec.margin[at];
-    const float *gbase = gout + (sblk * d.T + t0) * M;
+  // A block's state between the moment its loads are issued and the moment it is consumed.
+  struct Stage {
+    uint32_t a_r;   // record words of the pair this lane loads (key | vertex << 16, margin)
+    float mg_r;
+    float mg_own;   // copy of mg_r that survives the reuse of a_r / mg_r for a later block
+    float mg[P];    // per sub-step: margin of the pair this lane's group serves
+    uint32_t rel[P];  // ... and its element offset (tree, leaf, first chunk element) in the group's weights
     Float4U gv[P], wv[P];
-    bool on[P];
-    float mg[P];
-    uint32_t rel[P];
+  };
+  auto record_index = [&](long long sblk, bool have) -> long long {
+    return (long long)(t0 + (have ? rec_t : 0)) * d.S + sblk + (have ? rec_j : 0);
+  };
+  auto issue_rec = [&](Stage &st, long long sblk, bool have) {
+    const long long at = record_index(sblk, have);
+    st.a_r = rec.a[at];
+    st.mg_r = rec.margin[at];
+  };
+  auto issue_g = [&](Stage &st, long long sblk, const bool (&on)[P]) {
+    const float *gbase = gout + (sblk * d.T + t0) * M;
 #pragma unroll
-    for (int u = 0; u < P; ++u) {
-      on[u] = full || (jq[u] < ns && tq[u] < nt);
-      gv[u] = load_chunk(gbase + (on[u] ? goff[u] : uint32_t(e0)), true);
-    }
-#pragma unroll
-    for (int u = 0; u < P; ++u) {
-      const uint32_t key = uint32_t(__builtin_amdgcn_ds_bpermute(src[u], int(a_r))) & 0xffffu;
-      mg[u] = __int_as_float(__builtin_amdgcn_ds_bpermute(src[u], __float_as_int(mg_r)));
-      rel[u] = woff[u] + key * M;
-      if (need_c) wv[u] = load_chunk(wbase + (on[u] ? rel[u] : uint32_t(e0)), false);
-    }
+    for (int u = 0; u < P; ++u) st.gv[u] = load_chunk(on[u] ? gbase + u * gstep + goff : gbase + e0, false);
+  };
+  auto issue_w = [&](Stage &st, const bool (&on)[P]) {
+    st.mg_own = st.mg_r;
+    static_for<P>([&](auto u_tag) {
+      constexpr int u = decltype(u_tag)::value;
+      const uint32_t key = uint32_t(group_bcast<P, u>(int(st.a_r))) & key_mask;
+      st.mg[u] = __int_as_float(group_bcast<P, u>(__float_as_int(st.mg_r)));
+      st.rel[u] = woff + key * M;
+      if (need_c) st.wv[u] = load_chunk(wbase + (on[u] ? st.rel[u] : uint32_t(e0)), false);
+    });
+  };
+  auto compute = [&](Stage &st, long long sblk, bool have, const bool (&on)[P], auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
     float c_mine = 0.f;
 #pragma unroll
     for (int u = 0; u < P; ++u) {
-      if (dw && on[u]) {
-        Acc *cell = acc + (rel[u] - e0 + my_begin);
+      float g[ROUNDS];
+      own_elements(st.gv[u], g);
+      if (dw && (FULL || on[u])) {
+        Acc *cell = acc + (st.rel[u] - e0 + my_begin);
 #pragma unroll
-        for (int i = 0; i < Split::ROUNDS; ++i) {
-          if (i < my_cnt) {
-            const float term = ht_abs(mg[u]) * pick(gv[u], i);
+        for (int i = 0; i < ROUNDS; ++i) {
+          if (i < Split::BASE || i < my_cnt) {
+            const float term = ht_abs(st.mg[u]) * g[i];
             if (FIXED)
               atomicAdd(reinterpret_cast<unsigned long long *>(cell) + i, to_fixed(double(term), scale));
             else
@@ -589,16 +631,68 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
         }
       }
       if (need_c) {
+        float wl[ROUNDS];
+        own_elements(st.wv[u], wl);
         float partial = 0.f;
 #pragma unroll
-        for (int i = 0; i < Split::ROUNDS; ++i)
-          if (i < my_cnt) partial = __builtin_fmaf(pick(wv[u], i), pick(gv[u], i), partial);
-        partial = group_sum<float>(on[u] ? partial : 0.f, P);
-        const float got = __int_as_float(__builtin_amdgcn_ds_bpermute(my_src, __float_as_int(partial)));
-        if (my_sub == u) c_mine = got;
+        for (int i = 0; i < ROUNDS; ++i) {
+          const float term = __builtin_fmaf(wl[i], g[i], partial);
+          partial = (i < Split::BASE || i < my_cnt) ? term : partial;
+        }
+        partial = group_sum<float>((FULL || on[u]) ? partial : 0.f, P);
+        c_mine = (li == u) ? partial : c_mine;
       }
     }
-    if (need_c && have) rec.c[at] = ht_sign(mg_r) * c_mine;
+    if (need_c && (FULL || have)) rec.c[record_index(sblk, have)] = ht_sign(st.mg_own) * c_mine;
+  };
+
+  // This wavefront's blocks start at first, first + stride, ...; nfull of them are complete (64 existing pairs).
+  const long long stride = (long long)kWaves * SPT;
+  const long long first = s_begin + (long long)wave * SPT;
+  long long nblk = first < s_end ? (s_end - first + stride - 1) / stride : 0;
+  long long nfull = 0;
+  if (nt == TB && first + SPT <= s_end) nfull = (s_end - SPT - first) / stride + 1;
+  if (nt != TB) nfull = 0;
+
+  // ---- complete blocks, software pipelined: while block b is consumed, the gradient rows and weights of block b + 1
+  // and the records of block b + 2 are in flight (the kernel is otherwise bound by the latency of two dependent
+  // round trips per block: records -> weights).
+  if (nfull > 0) {
+    bool all_on[P];
+#pragma unroll
+    for (int u = 0; u < P; ++u) all_on[u] = true;
+    auto block_at = [&](long long b) { return first + (b < nfull ? b : nfull - 1) * stride; };  // clamped: re-reads
+    Stage s0, s1;
+    issue_rec(s0, block_at(0), true);
+    issue_g(s0, block_at(0), all_on);
+    issue_rec(s1, block_at(1), true);
+    issue_w(s0, all_on);
+    auto iteration = [&](Stage &cur, Stage &nxt, long long b) {
+      issue_rec(cur, block_at(b + 2), true);  // cur's record words were consumed by its issue_w
+      issue_g(nxt, block_at(b + 1), all_on);
+      issue_w(nxt, all_on);
+      compute(cur, block_at(b), true, all_on, std::true_type{});
+    };
+    long long b = 0;
+    for (; b + 1 < nfull; b += 2) {
+      iteration(s0, s1, b);
+      iteration(s1, s0, b + 1);
+    }
+    if (b < nfull) iteration(s0, s1, b);
+  }
+  // ---- the incomplete tail (at most one block per wavefront unless the tree group itself is incomplete)
+  for (long long bi = nfull; bi < nblk; ++bi) {
+    const long long sblk = first + bi * stride;
+    const int ns = int(min<long long>(SPT, s_end - sblk));
+    const bool have = rec_t < nt && rec_j < ns;
+    bool on[P];
+#pragma unroll
+    for (int u = 0; u < P; ++u) on[u] = jq0 + u * jstep < ns && tq < nt;
+    Stage st;
+    issue_rec(st, sblk, have);
+    issue_g(st, sblk, on);
+    issue_w(st, on);
+    compute(st, sblk, have, on, std::false_type{});
   }
   if (dw) {
     __syncthreads();
@@ -1041,7 +1135,7 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
     // the specialised kernel: contiguous rows, a power-of-two tree group, 32-bit offsets inside a block and a group
     int log2_tb = 0;
     while ((1 << (log2_tb + 1)) <= p.TB) ++log2_tb;
-    const bool fits = d.K == 1 && (1 << log2_tb) == p.TB && p.TB <= kWave &&
+    const bool fits = d.K == 1 && (1 << log2_tb) == p.TB && p.TB <= 16 &&
                       (long long)kWave * d.T * d.M < (1ll << 31) && (long long)p.TB * d.L * d.M < (1ll << 31);
     if (fits && (d.M == 10 || d.M == 1)) {
       HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(d.M == 10 ? (const void *)tree_lean_kernel<10, FIXED>

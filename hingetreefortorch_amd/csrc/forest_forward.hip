@@ -258,8 +258,14 @@ __device__ __forceinline__ void walk_quads(int depth, const QuadNode *const (&qu
   }
 }
 
-constexpr int kRowIlp = 4;     // trees walked concurrently per lane
-constexpr int kRowUnroll = 5;  // output vectors per lane whose weight gathers are in flight together
+#ifndef HT_ROW_ILP
+#define HT_ROW_ILP 4
+#endif
+#ifndef HT_ROW_UNROLL
+#define HT_ROW_UNROLL 5
+#endif
+constexpr int kRowIlp = HT_ROW_ILP;        // trees walked concurrently per lane
+constexpr int kRowUnroll = HT_ROW_UNROLL;  // output vectors per lane whose weight gathers are in flight together
 
 // One workgroup = one tile of BT samples (all features in LDS, feature major) x a range of trees, like
 // forward_kernel, but every wavefront works on its own: lanes = BT samples x 64/BT tree slots, each lane walks
@@ -402,8 +408,12 @@ static inline size_t rows_lds_bytes(int F, int bt) {
 template <typename Real>
 static inline int pick_rows_tile(int F) {
   const int candidates[4] = {64, 32, 16, 8};
-  for (int bt : candidates)
+  for (int bt : candidates) {
+#ifdef HT_ROW_MAXBT
+    if (bt > HT_ROW_MAXBT) continue;
+#endif
     if (rows_lds_bytes<Real>(F, bt) <= size_t(kLdsBytes)) return bt;
+  }
   return 0;
 }
 
