@@ -327,10 +327,37 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
         for (int i = 0; i < kRowIlp; ++i) qn[i] = static_cast<const QuadNode *>(vertices) + (long long)t[i] * NQ;
         walk_quads<kRowIlp, BT>(d.depth, qn, xs_j, r);
       } else {
-        const Node<Real> *nd[kRowIlp];
+        const Node<Real> *all = static_cast<const Node<Real> *>(vertices);
+        bool staged = false;
+        if constexpr (FERN) {
+          // A fern's vertex is the same for every sample, so a vector load of it would fetch one address per tree
+          // slot and still cost a full trip through the vector memory pipeline per level. Instead the wavefront
+          // copies the vertices of its TPW ferns into LDS once per step -- into the space of the parked results,
+          // which nobody reads before this step's walks are over -- and the walk reads them as LDS broadcasts.
+          Node<Real> *stage = reinterpret_cast<Node<Real> *>(p_abs);
+          if (size_t(TPW) * d.depth * sizeof(Node<Real>) <= size_t(BT) * LDP * sizeof(Real)) {
+            staged = true;
+            for (int i = lane; i < TPW * d.depth; i += kWave) {
+              const int tt = i / d.depth, lv = i - tt * d.depth;
+              stage[i] = all[(long long)min(tb + tt, t_end - 1) * d.V + lv];
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            walk_many_fn<Real, true, kRowIlp>(
+                d.depth, [&](int i, uint32_t at) { return stage[(slot + i * SLOTS) * d.depth + at]; },
+                [&](int, int f) { return xs_j[f * BT]; }, r);
+            // every lane has read its vertices before any lane overwrites them with results
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+          }
+        }
+        if (!staged) {
+          const Node<Real> *nd[kRowIlp];
 #pragma unroll
-        for (int i = 0; i < kRowIlp; ++i) nd[i] = static_cast<const Node<Real> *>(vertices) + (long long)t[i] * d.V;
-        walk_many<Real, FERN, kRowIlp>(d.depth, nd, [&](int, int f) { return xs_j[f * BT]; }, r);
+          for (int i = 0; i < kRowIlp; ++i) nd[i] = all + (long long)t[i] * d.V;
+          walk_many<Real, FERN, kRowIlp>(d.depth, nd, [&](int, int f) { return xs_j[f * BT]; }, r);
+        }
       }
 #endif
 #pragma unroll

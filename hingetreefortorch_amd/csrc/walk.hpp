@@ -51,10 +51,10 @@ struct __align__(16) Node<double> {
 };
 
 // N independent walks advanced level by level in one loop, so that their dependent load chains overlap.
-// `nodes[i]` is the packed vertex array of walk i, `feature(i, f)` returns walk i's sample value of feature f.
-template <typename Real, bool FERN, int N, typename FeatureFn>
-__device__ __forceinline__ void walk_many(int depth, const Node<Real> *const (&nodes)[N], FeatureFn feature,
-                                          WalkResult<Real> (&r)[N]) {
+// `node(i, at)` returns the packed vertex `at` (heap index, or level for a fern) of walk i, `feature(i, f)` returns
+// walk i's sample value of feature f.
+template <typename Real, bool FERN, int N, typename NodeFn, typename FeatureFn>
+__device__ __forceinline__ void walk_many_fn(int depth, NodeFn node, FeatureFn feature, WalkResult<Real> (&r)[N]) {
   uint32_t v[N];
   Real best_abs[N];
 #pragma unroll
@@ -69,7 +69,7 @@ __device__ __forceinline__ void walk_many(int depth, const Node<Real> *const (&n
   for (int lvl = 0; lvl < depth; ++lvl) {
     Node<Real> n[N];
 #pragma unroll
-    for (int i = 0; i < N; ++i) n[i] = nodes[i][FERN ? uint32_t(lvl) : v[i]];
+    for (int i = 0; i < N; ++i) n[i] = node(i, FERN ? uint32_t(lvl) : v[i]);
     Real m[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) m[i] = feature(i, int(n[i].ord)) - n[i].thr;
@@ -89,6 +89,13 @@ __device__ __forceinline__ void walk_many(int depth, const Node<Real> *const (&n
       v[i] = 2u * v[i] + 1u + bit;
     }
   }
+}
+
+// The same with the vertices of walk i in the array nodes[i].
+template <typename Real, bool FERN, int N, typename FeatureFn>
+__device__ __forceinline__ void walk_many(int depth, const Node<Real> *const (&nodes)[N], FeatureFn feature,
+                                          WalkResult<Real> (&r)[N]) {
+  walk_many_fn<Real, FERN, N>(depth, [&](int i, uint32_t at) { return nodes[i][at]; }, feature, r);
 }
 
 // Single walk over separate threshold / ordinal arrays (used where the vertices are not packed).
