@@ -23,6 +23,7 @@ struct ConvGeom {
 
 constexpr int kConvThreads = 256;
 constexpr int kMaxRegM = 16;
+constexpr int kConvIlp = 4;  // channels whose walks a thread of the tiled kernels interleaves (hides LDS latency)
 
 // Offsets of tap j relative to the patch anchor, per dim (already multiplied by the dilation): tapc[j * 3 + d].
 __device__ __forceinline__ void fill_tap_table(int *tapc, const ConvGeom &g) {
@@ -183,6 +184,335 @@ __global__ __launch_bounds__(kConvThreads) void conv_backward_kernel(ConvGeom g,
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// tiled kernels for 1 and 2 spatial dims
+// ---------------------------------------------------------------------------------------------------------------
+// A workgroup of 256 threads owns a TY x TX tile of output positions of one image (one thread per position) and keeps
+// the input region that tile reads -- all C channels, zeros where the region leaves the image -- in LDS. The trees of
+// one out channel (C trees) are staged in LDS as (threshold, tile offset of the tap) pairs, so a walk step is two LDS
+// reads and no address arithmetic beyond one add, and the padding needs no test. Every byte of x is read from memory
+// once per tile instead of once per (out channel, vertex visit).
+struct ConvTile {
+  int H, W, OH, OW;
+  int kh, kw, sy, sx, py, px, dy, dx;
+  int TY, TX, log2_tx;  // output tile, TY * TX == kConvThreads
+  int IH, IW, TSZ;      // input region of a tile, TSZ = IH * IW
+  int tiles_y, tiles_x;
+  int taps;
+};
+
+static bool make_tile(const ConvGeom &g, ConvTile *t) {
+  if (g.nd > 2) return false;
+  const int a = g.nd == 2 ? 0 : -1;  // index of the row dimension, none for 1-d
+  t->H = a < 0 ? 1 : g.size[0];
+  t->OH = a < 0 ? 1 : g.osz[0];
+  t->kh = a < 0 ? 1 : g.ker[0];
+  t->sy = a < 0 ? 1 : g.str[0];
+  t->py = a < 0 ? 0 : g.pad[0];
+  t->dy = a < 0 ? 1 : g.dil[0];
+  const int c = g.nd - 1;
+  t->W = g.size[c];
+  t->OW = g.osz[c];
+  t->kw = g.ker[c];
+  t->sx = g.str[c];
+  t->px = g.pad[c];
+  t->dx = g.dil[c];
+  int tx = kConvThreads;  // widest power-of-two tile row that the output needs
+  while (tx > 32 && tx / 2 >= t->OW) tx /= 2;
+  if (t->OH > 1 && tx > 32) tx = 32;
+  t->TX = tx;
+  t->TY = kConvThreads / tx;
+  t->log2_tx = 0;
+  while ((1 << t->log2_tx) < tx) ++t->log2_tx;
+  t->IH = (t->TY - 1) * t->sy + (t->kh - 1) * t->dy + 1;
+  t->IW = (t->TX - 1) * t->sx + (t->kw - 1) * t->dx + 1;
+  const long long tsz = (long long)t->IH * t->IW;
+  if (tsz > (1 << 20)) return false;
+  t->TSZ = int(tsz);
+  t->tiles_y = (t->OH + t->TY - 1) / t->TY;
+  t->tiles_x = (t->OW + t->TX - 1) / t->TX;
+  t->taps = g.taps;
+  return true;
+}
+
+// Cooperative load of the input region of tile (tyi, txi) of image b, all channels: a thread owns one or two cells of
+// the region and copies them channel by channel (the coordinate arithmetic is done once per cell, not per element).
+template <typename Real>
+__device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restrict__ x, const ConvTile &g, int C,
+                                               long long b, int tyi, int txi) {
+  const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
+  const long long chan = (long long)g.H * g.W;
+  const Real *img = x + b * C * chan;
+  for (int e = threadIdx.x; e < g.TSZ; e += kConvThreads) {
+    const int iy = e / g.IW, ix = e - iy * g.IW;
+    const int gy = iy0 + iy, gx = ix0 + ix;
+    Real *q = tile + e;
+    if (gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) {
+      const Real *p = img + (long long)gy * g.W + gx;
+#pragma unroll 4
+      for (int c = 0; c < C; ++c) q[c * g.TSZ] = p[c * chan];
+    } else {
+      for (int c = 0; c < C; ++c) q[c * g.TSZ] = Real(0);
+    }
+  }
+}
+
+// Trees (and optionally leaf weights) of out channel j into LDS.
+template <typename Real>
+__device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, const ConvTile &g, int C, int V, int LM,
+                                                 int j, const Real *__restrict__ thr, const int64_t *__restrict__ ord,
+                                                 const Real *__restrict__ w) {
+  const long long first = (long long)j * C * V;
+  for (int i = threadIdx.x; i < C * V; i += kConvThreads) {
+    const int tap = clamp_ordinal(ord[first + i], g.taps);
+    const int ky = tap / g.kw, kx = tap - ky * g.kw;
+    Node<Real> n;
+    n.thr = thr[first + i];
+    n.ord = ky * g.dy * g.IW + kx * g.dx;
+    nodes[i] = n;
+  }
+  if (wl) {
+    const long long wfirst = (long long)j * C * LM;
+    for (int i = threadIdx.x; i < C * LM; i += kConvThreads) wl[i] = w[wfirst + i];
+  }
+}
+
+struct ConvLds {
+  size_t tile, acc_x, nodes, wl, acc_w, acc_t, total;
+};
+
+template <typename Real>
+static ConvLds conv_lds_layout(const ConvTile &t, int C, int V, int LM, bool dx_acc, bool tree_acc, bool w_lds) {
+  ConvLds l{};
+  size_t at = 0;
+  l.tile = at;
+  at += align_up(size_t(C) * t.TSZ * sizeof(Real), 16);
+  l.acc_x = at;
+  if (dx_acc) at += align_up(size_t(C) * t.TSZ * sizeof(double), 16);
+  l.nodes = at;
+  at += align_up(size_t(C) * V * sizeof(Node<Real>), 16);
+  l.wl = at;
+  if (w_lds) at += align_up(size_t(C) * LM * sizeof(Real), 16);
+  l.acc_w = at;
+  if (tree_acc) at += align_up(size_t(C) * LM * sizeof(double), 16);
+  l.acc_t = at;
+  if (tree_acc) at += align_up(size_t(C) * V * sizeof(double), 16);
+  l.total = at;
+  return l;
+}
+
+// MREG = outputs per leaf kept in registers per pass over the channels (1, 4 or 16: the smallest that holds M, so the
+// common single-output case carries no per-output loop at all).
+template <typename Real, bool FERN, int MREG>
+__global__ __launch_bounds__(kConvThreads) void conv_tiled_forward_kernel(ConvTile g, ConvLds lay, int C, int Cout,
+                                                                          int depth, int V, int L, int M, int j_per,
+                                                                          const Real *__restrict__ x,
+                                                                          const Real *__restrict__ thr,
+                                                                          const int64_t *__restrict__ ord,
+                                                                          const Real *__restrict__ w,
+                                                                          Real *__restrict__ out) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *tile = reinterpret_cast<Real *>(smem + lay.tile);
+  Node<Real> *nodes = reinterpret_cast<Node<Real> *>(smem + lay.nodes);
+  Real *wl = reinterpret_cast<Real *>(smem + lay.wl);
+  const int tyi = blockIdx.x / g.tiles_x, txi = blockIdx.x - tyi * g.tiles_x;
+  const long long b = blockIdx.z;
+  load_conv_tile<Real>(tile, x, g, C, b, tyi, txi);
+  const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
+  const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
+  const bool live = oy < g.OH && ox < g.OW;
+  const Real *mine = tile + ty * g.sy * g.IW + tx * g.sx;
+  const int LM = L * M;
+  const int j_begin = blockIdx.y * j_per, j_end = min(Cout, j_begin + j_per);
+  for (int j = j_begin; j < j_end; ++j) {
+    __syncthreads();  // the tile is complete / the previous out channel's trees are no longer read
+    stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w);
+    __syncthreads();
+    if (!live) continue;
+    Real *o = out + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+    for (int m0 = 0; m0 < M; m0 += MREG) {
+      const int mc = min(MREG, M - m0);
+      Real acc[MREG];
+#pragma unroll
+      for (int m = 0; m < MREG; ++m) acc[m] = Real(0);
+      for (int c = 0; c < C; c += kConvIlp) {
+        // several channels' walks interleaved; their terms are still added in ascending channel order
+        WalkResult<Real> r[kConvIlp];
+        const Node<Real> *nd[kConvIlp];
+        const Real *px[kConvIlp];
+#pragma unroll
+        for (int i = 0; i < kConvIlp; ++i) {
+          const int ci = min(c + i, C - 1);  // surplus slots re-walk the last channel, unused
+          nd[i] = nodes + ci * V;
+          px[i] = mine + ci * g.TSZ;
+        }
+        walk_paths<Real, FERN, false, kConvIlp>(
+            depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
+#pragma unroll
+        for (int i = 0; i < kConvIlp; ++i) {
+          if (c + i >= C) break;
+          const Real a = r[i].margin;  // |margin|
+          const Real *row = wl + ((c + i) * L + r[i].key) * M + m0;
+#pragma unroll
+          for (int m = 0; m < MREG; ++m)
+            if (MREG == 1 || m < mc) acc[m] = acc[m] + row[m] * a;
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < MREG; ++m)
+        if (MREG == 1 || m < mc) o[m0 + m] = acc[m];
+    }
+  }
+}
+
+// dX: tile-stationary over all out channels; c = sign(margin) * sum_m w * g goes into an fp64 LDS image of the tile's
+// input region (fp64 because that is the fast LDS floating-point atomic on gfx950), flushed once with global atomics
+// (regions of neighbouring tiles overlap). Cells outside the image are dropped like the reference drops padded taps.
+template <typename Real, bool FERN>
+__global__ __launch_bounds__(kConvThreads) void conv_tiled_dx_kernel(ConvTile g, ConvLds lay, int C, int Cout,
+                                                                     int depth, int V, int L, int M, int j_per,
+                                                                     const Real *__restrict__ x,
+                                                                     const Real *__restrict__ thr,
+                                                                     const int64_t *__restrict__ ord,
+                                                                     const Real *__restrict__ w,
+                                                                     const Real *__restrict__ gout, Real *dx) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *tile = reinterpret_cast<Real *>(smem + lay.tile);
+  double *acc = reinterpret_cast<double *>(smem + lay.acc_x);
+  Node<Real> *nodes = reinterpret_cast<Node<Real> *>(smem + lay.nodes);
+  Real *wl = reinterpret_cast<Real *>(smem + lay.wl);
+  const int tyi = blockIdx.x / g.tiles_x, txi = blockIdx.x - tyi * g.tiles_x;
+  const long long b = blockIdx.z;
+  load_conv_tile<Real>(tile, x, g, C, b, tyi, txi);
+  for (int i = threadIdx.x; i < C * g.TSZ; i += kConvThreads) acc[i] = 0.0;
+  const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
+  const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
+  const bool live = oy < g.OH && ox < g.OW;
+  const int base = ty * g.sy * g.IW + tx * g.sx;
+  const Real *mine = tile + base;
+  const int LM = L * M;
+  const int j_begin = blockIdx.y * j_per, j_end = min(Cout, j_begin + j_per);
+  for (int j = j_begin; j < j_end; ++j) {
+    __syncthreads();
+    stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w);
+    __syncthreads();
+    if (!live) continue;
+    const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+    for (int c = 0; c < C; c += kConvIlp) {
+      WalkResult<Real> r[kConvIlp];
+      const Node<Real> *nd[kConvIlp];
+      const Real *px[kConvIlp];
+#pragma unroll
+      for (int i = 0; i < kConvIlp; ++i) {
+        const int ci = min(c + i, C - 1);
+        nd[i] = nodes + ci * V;
+        px[i] = mine + ci * g.TSZ;
+      }
+      walk_paths<Real, FERN, true, kConvIlp>(
+          depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
+#pragma unroll
+      for (int i = 0; i < kConvIlp; ++i) {
+        if (c + i >= C) break;
+        const Real *row = wl + ((c + i) * L + r[i].key) * M;
+        Real cs = Real(0);
+        for (int m = 0; m < M; ++m) cs += row[m] * gp[m];
+        cs = ht_sign(r[i].margin) * cs;
+        atomicAdd(acc + (c + i) * g.TSZ + base + int(r[i].ord), double(cs));  // r.ord is the tap's tile offset
+      }
+    }
+  }
+  __syncthreads();
+  const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
+  for (int i = threadIdx.x; i < C * g.TSZ; i += kConvThreads) {
+    const double v = acc[i];
+    if (v == 0.0) continue;
+    const int c = i / g.TSZ, r = i - c * g.TSZ;
+    const int iy = r / g.IW, ix = r - iy * g.IW;
+    const int gy = iy0 + iy, gx = ix0 + ix;
+    if (gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) atomicAdd(dx + ((b * C + c) * g.H + gy) * (long long)g.W + gx, Real(v));
+  }
+}
+
+// dThr and dW: a workgroup owns out channel blockIdx.x and visits every blockIdx.y-th (image, tile); the gradients of
+// its C trees are accumulated in fp64 LDS tables over all of those visits and flushed once.
+template <typename Real, bool FERN>
+__global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile g, ConvLds lay, int C, int Cout,
+                                                                        int depth, int V, int L, int M, long long items,
+                                                                        const Real *__restrict__ x,
+                                                                        const Real *__restrict__ thr,
+                                                                        const int64_t *__restrict__ ord,
+                                                                        const Real *__restrict__ w,
+                                                                        const Real *__restrict__ gout, Real *dthr,
+                                                                        Real *dw) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *tile = reinterpret_cast<Real *>(smem + lay.tile);
+  Node<Real> *nodes = reinterpret_cast<Node<Real> *>(smem + lay.nodes);
+  Real *wl = reinterpret_cast<Real *>(smem + lay.wl);
+  double *acc_w = reinterpret_cast<double *>(smem + lay.acc_w);
+  double *acc_t = reinterpret_cast<double *>(smem + lay.acc_t);
+  const int j = blockIdx.x;
+  const int LM = L * M;
+  stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w);
+  for (int i = threadIdx.x; i < C * LM; i += kConvThreads) acc_w[i] = 0.0;
+  for (int i = threadIdx.x; i < C * V; i += kConvThreads) acc_t[i] = 0.0;
+  const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
+  const Real *mine = tile + ty * g.sy * g.IW + tx * g.sx;
+  const int tiles = g.tiles_y * g.tiles_x;
+  for (long long it = blockIdx.y; it < items; it += gridDim.y) {
+    const long long b = it / tiles;
+    const int t = int(it - b * tiles);
+    const int tyi = t / g.tiles_x, txi = t - tyi * g.tiles_x;
+    __syncthreads();  // the previous tile is no longer read (first pass: the staged trees are complete)
+    load_conv_tile<Real>(tile, x, g, C, b, tyi, txi);
+    __syncthreads();
+    const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
+    if (oy >= g.OH || ox >= g.OW) continue;
+    const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+    for (int c = 0; c < C; c += kConvIlp) {
+      WalkResult<Real> r[kConvIlp];
+      const Node<Real> *nd[kConvIlp];
+      const Real *px[kConvIlp];
+#pragma unroll
+      for (int i = 0; i < kConvIlp; ++i) {
+        const int ci = min(c + i, C - 1);
+        nd[i] = nodes + ci * V;
+        px[i] = mine + ci * g.TSZ;
+      }
+      walk_paths<Real, FERN, true, kConvIlp>(
+          depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
+#pragma unroll
+      for (int i = 0; i < kConvIlp; ++i) {
+        if (c + i >= C) break;
+        const Real a = ht_abs(r[i].margin);
+        const int cell = ((c + i) * L + int(r[i].key)) * M;
+        Real cs = Real(0);
+        for (int m = 0; m < M; ++m) {
+          const Real gv = gp[m];
+          cs += wl[cell + m] * gv;
+          if (dw) atomicAdd(acc_w + cell + m, double(a * gv));
+        }
+        if (dthr) atomicAdd(acc_t + (c + i) * V + int(r[i].vertex), -double(ht_sign(r[i].margin) * cs));
+      }
+    }
+  }
+  __syncthreads();
+  if (dw)
+    for (int i = threadIdx.x; i < C * LM; i += kConvThreads)
+      if (acc_w[i] != 0.0) atomicAdd(dw + (long long)j * C * LM + i, Real(acc_w[i]));
+  if (dthr)
+    for (int i = threadIdx.x; i < C * V; i += kConvThreads)
+      if (acc_t[i] != 0.0) atomicAdd(dthr + (long long)j * C * V + i, Real(acc_t[i]));
+}
+
+constexpr size_t kConvTiledLdsMax = 160 * 1024;  // LDS of a CU
+
+// Out channels per workgroup of the tile-stationary kernels: all of them unless that leaves the device underfilled.
+static int conv_j_per(long long tiles_total, int Cout) {
+  long long want = tiles_total >= 4 * kNumCUs ? 1 : (4 * kNumCUs + tiles_total - 1) / (tiles_total > 0 ? tiles_total : 1);
+  if (want > Cout) want = Cout;
+  return int((Cout + want - 1) / want);
+}
+
 int make_geom(const ht_conv_shape &s, ConvGeom *g) {
   if (s.nd < 1 || s.nd > HT_MAX_CONV_DIMS)
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: convolution supports 1, 2 or 3 spatial dimensions.");
@@ -240,6 +570,25 @@ int conv_forward(const ht_conv_shape &s, const Real *x, const Real *thr, const i
   const bool fern = s.kind == HT_FERN;
   const int V = fern ? int(s.depth) : int((1LL << s.depth) - 1), L = int(1LL << s.depth);
   if (s.C == 0) return zero_fill(out, size_t(s.B) * s.Cout * g.rows * s.M * sizeof(Real), stream);
+  ConvTile t;
+  if (make_tile(g, &t)) {
+    const int LM = L * int(s.M);
+    const ConvLds lay = conv_lds_layout<Real>(t, int(s.C), V, LM, false, false, true);
+    if (lay.total <= kConvTiledLdsMax && (long long)t.tiles_y * t.tiles_x <= 0x7fffffffLL) {
+      const long long tiles = (long long)t.tiles_y * t.tiles_x;
+      const int j_per = conv_j_per(tiles * s.B, int(s.Cout));
+      const dim3 tgrid((unsigned)tiles, (unsigned)((s.Cout + j_per - 1) / j_per), (unsigned)s.B);
+      auto kernel = fern ? conv_tiled_forward_kernel<Real, true, 16> : conv_tiled_forward_kernel<Real, false, 16>;
+      if (s.M == 1) kernel = fern ? conv_tiled_forward_kernel<Real, true, 1> : conv_tiled_forward_kernel<Real, false, 1>;
+      else if (s.M <= 4) kernel = fern ? conv_tiled_forward_kernel<Real, true, 4> : conv_tiled_forward_kernel<Real, false, 4>;
+      HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lay.total)));
+      hipLaunchKernelGGL(kernel, tgrid, dim3(kConvThreads), lay.total, stream, t, lay, int(s.C), int(s.Cout),
+                         int(s.depth), V, L, int(s.M), j_per, x, thr, ord, w, out);
+      HT_LAUNCH_CHECK("conv forward (tiled)");
+      return HT_OK;
+    }
+  }
   const dim3 grid((g.rows + kConvThreads - 1) / kConvThreads, (unsigned)s.Cout, (unsigned)s.B);
   const size_t lds = size_t(g.taps) * 3 * sizeof(int);
   if (fern)
@@ -278,6 +627,40 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
   if (dthr && (rc = zero_fill(dthr, size_t(s.Cout) * s.C * V * sizeof(Real), stream)) != HT_OK) return rc;
   if (dw && (rc = zero_fill(dw, size_t(s.Cout) * s.C * L * s.M * sizeof(Real), stream)) != HT_OK) return rc;
   if (s.B == 0 || s.Cout == 0 || s.C == 0 || g.rows == 0 || (!dx && !dthr && !dw)) return HT_OK;
+  ConvTile t;
+  if (make_tile(g, &t)) {
+    const int LM = L * int(s.M);
+    const ConvLds lay_x = conv_lds_layout<Real>(t, int(s.C), V, LM, true, false, true);
+    const ConvLds lay_t = conv_lds_layout<Real>(t, int(s.C), V, LM, false, true, true);
+    const long long tiles = (long long)t.tiles_y * t.tiles_x;
+    if (lay_x.total <= kConvTiledLdsMax && lay_t.total <= kConvTiledLdsMax && tiles <= 0x7fffffffLL) {
+      if (dx) {
+        const int j_per = conv_j_per(tiles * s.B, int(s.Cout));
+        const dim3 grid((unsigned)tiles, (unsigned)((s.Cout + j_per - 1) / j_per), (unsigned)s.B);
+        auto kernel = fern ? conv_tiled_dx_kernel<Real, true> : conv_tiled_dx_kernel<Real, false>;
+        HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(lay_x.total)));
+        hipLaunchKernelGGL(kernel, grid, dim3(kConvThreads), lay_x.total, stream, t, lay_x, int(s.C), int(s.Cout),
+                           int(s.depth), V, L, int(s.M), j_per, x, thr, ord, w, gout, dx);
+        HT_LAUNCH_CHECK("conv backward (dX, tiled)");
+      }
+      if (dthr || dw) {
+        const long long items = tiles * s.B;
+        long long parts = (4 * kNumCUs + s.Cout - 1) / s.Cout;  // ~4 workgroups per CU
+        if (parts > items) parts = items;
+        if (parts > 65535) parts = 65535;
+        if (parts < 1) parts = 1;
+        const dim3 grid((unsigned)s.Cout, (unsigned)parts);
+        auto kernel = fern ? conv_tiled_trees_kernel<Real, true> : conv_tiled_trees_kernel<Real, false>;
+        HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(lay_t.total)));
+        hipLaunchKernelGGL(kernel, grid, dim3(kConvThreads), lay_t.total, stream, t, lay_t, int(s.C), int(s.Cout),
+                           int(s.depth), V, L, int(s.M), items, x, thr, ord, w, gout, dthr, dw);
+        HT_LAUNCH_CHECK("conv backward (trees, tiled)");
+      }
+      return HT_OK;
+    }
+  }
   const size_t tap_bytes = align_up(size_t(g.taps) * 3 * sizeof(int), 16);
   const size_t acc_bytes = (size_t(V) + size_t(L) * s.M) * sizeof(Real);
   const bool lds_acc = acc_bytes <= 48 * 1024;

@@ -98,6 +98,52 @@ __device__ __forceinline__ void walk_many(int depth, const Node<Real> *const (&n
   walk_many_fn<Real, FERN, N>(depth, [&](int i, uint32_t at) { return nodes[i][at]; }, feature, r);
 }
 
+// Leaner form of walk_many_fn for walks whose vertices and features both sit in LDS (little latency to hide, so the
+// instruction count is what matters). The decisions are collected most significant bit first in `path` -- which is
+// also the index of the current vertex inside its level, so the heap index needs no separate update -- and the leaf
+// key (decision of level i in bit i) is the bit reversal of the finished path. TRACK = false skips the selected
+// vertex / ordinal / signed margin (forward pass): r.margin then holds |margin|.
+template <typename Real, bool FERN, bool TRACK, int N, typename NodeFn, typename FeatureFn>
+__device__ __forceinline__ void walk_paths(int depth, NodeFn node, FeatureFn feature, WalkResult<Real> (&r)[N]) {
+  uint32_t path[N];
+  Real best_abs[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    path[i] = 0;
+    best_abs[i] = Real(0);
+    r[i].vertex = 0;
+    r[i].ord = 0;
+    r[i].margin = Real(0);
+  }
+  for (int lvl = 0; lvl < depth; ++lvl) {
+    const uint32_t first = FERN ? uint32_t(lvl) : (1u << lvl) - 1u;  // wave uniform
+    Node<Real> n[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) n[i] = node(i, FERN ? first : first + path[i]);
+    Real m[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) m[i] = feature(i, int(n[i].ord)) - n[i].thr;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const Real a = ht_abs(m[i]);
+      if (lvl == 0 || a < best_abs[i]) {
+        best_abs[i] = a;
+        if (TRACK) {
+          r[i].margin = m[i];
+          r[i].vertex = FERN ? first : first + path[i];
+          r[i].ord = uint32_t(n[i].ord);
+        }
+      }
+      path[i] = path[i] + path[i] + ((m[i] > Real(0)) ? 1u : 0u);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    r[i].key = __brev(path[i]) >> (32 - depth);
+    if (!TRACK) r[i].margin = best_abs[i];
+  }
+}
+
 // Single walk over separate threshold / ordinal arrays (used where the vertices are not packed).
 // `node(i)` returns (threshold, ordinal) of decision i; `feature(f)` returns this sample's value of feature f.
 template <typename Real, bool FERN, typename NodeFn, typename FeatureFn>
