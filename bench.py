@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: RandomHingeForest fp32 forward+backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c1] [--mode atomic|deterministic]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c1|c4] [--mode atomic|deterministic]
                     [--path train|stateless]
 
 One step = one forward plus one backward (all three gradients requested, atomic mode) over one batch of synthetic input
@@ -12,6 +12,11 @@ tree_backward), whose backward walks the trees again. The other path is timed to
 The default workload is the configuration the metric is quoted on: x ~ N(0,1) [65536, 1024], 1000 trees, depth 10,
 extra_outputs = 10 (out [65536, 1000, 10]); thresholds ~ U(-3,3) made consistent like the module constructor does,
 ordinals ~ U{0..1023}, leaf weights ~ N(0,1), upstream gradient ~ N(0,1).
+
+`--workload c4` times the convolutional operator instead (tree_conv2d_forward / tree_conv2d_backward on images
+[32,16,128,128], 64 out channels, depth 6, 3x3 taps: 64 x 16 trees over the 9 taps of one channel each, summed over
+the channels); it is bound by LDS reads and vector instructions, not by HBM, so its line reports images/s and vertex
+visits/s with the HBM fraction for information only.
 
 Prints ONE JSON line. `value` is samples/s over the timed steps (wall clock between device synchronisations);
 `roofline` prices the dominant kernel (the forward kernel: tree_forward launches it plus a ~7 us vertex-packing
@@ -96,12 +101,65 @@ def cpu_baseline(torch, name, x, thr, ordn, w, gout, budget_rows):
             "host_cores": os.cpu_count()}
 
 
+def bench_conv(torch, ops, dev, args):
+    """HingeTreeConv2d forward+backward on the convolutional benchmark shape."""
+    B, C, Cout, H, W, depth = 32, 16, 64, 128, 128, 6
+    V, L = 2 ** depth - 1, 2 ** depth
+    g = torch.Generator().manual_seed(6112)
+    thr = (6.0 * torch.rand([Cout, C, V], generator=g) - 3.0).to(dev)
+    ordn = torch.randint(0, 9, [Cout, C, V], generator=g, dtype=torch.int64).to(dev)
+    w = torch.randn([Cout, C, L], generator=g).to(dev)
+    gg = torch.Generator(device=dev).manual_seed(6113)
+    x = torch.randn([B, C, H, W], generator=gg, device=dev)
+    gout = torch.randn([B, Cout, H, W], generator=gg, device=dev)
+    geo = ([3, 3], [1, 1], [1, 1], [1, 1])
+
+    def step(ev=None):
+        if ev: ev[0].record()
+        ops.tree_conv2d_forward(x, thr, ordn, w, *geo)
+        if ev: ev[1].record()
+        ops.tree_conv2d_backward(x, True, thr, True, ordn, False, w, True, gout, *geo)
+        if ev: ev[2].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(ev[i])
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    walks = B * Cout * C * H * W
+    fwd_bytes = 4 * (x.numel() + thr.numel() + w.numel() + gout.numel()) + 8 * ordn.numel()
+    bwd_bytes = fwd_bytes + 4 * (x.numel() + thr.numel() + w.numel())
+    return {
+        "metric": "conv fwd+bwd images/s (HingeTreeConv2d [32,16,128,128] -> 64 channels, depth 6, 3x3)",
+        "value": B / (ms * 1e-3), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "c4: 64 x 16 trees of depth 6 over the 9 taps of one input channel each, summed over "
+                               "the 16 channels; stride 1, padding 1, dilation 1", "B": B, "C": C, "Cout": Cout,
+                   "H": H, "W": W, "depth": depth},
+        "forward": {"ms": fwd_ms, "vertex_visits_per_s": walks * depth / (fwd_ms * 1e-3),
+                    "hbm_frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "backward": {"ms": bwd_ms, "hbm_frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "roofline": {"bound": "hbm", "kernel": "conv_tiled_forward_kernel",
+                     "achieved": fwd_bytes / (fwd_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "note": "informational: the kernel is bound by LDS reads and vector instructions "
+                             "(3.2e9 vertex visits per pass), not by HBM"},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4"])
     ap.add_argument("--mode", default="atomic", choices=["atomic", "deterministic"])
     ap.add_argument("--path", default="train", choices=["train", "stateless"])
     ap.add_argument("--other-steps", type=int, default=-1,
@@ -130,6 +188,9 @@ def main():
         print(json.dumps({"calibration": "3 x copy of 1 GiB (reads 1073741824 B, writes 1073741824 B per launch)"}))
         return
     name = args.workload
+    if name == "c4":
+        print(json.dumps(bench_conv(torch, ops, dev, args)), flush=True)
+        return
     B, F, T, depth, M, kind, _, desc = WORKLOADS[name]
     x, thr, ordn, w, gout = make_inputs(torch, name, dev)
     pre = "fern_" if kind == "fern" else "tree_"
@@ -203,7 +264,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{name}: {desc}", "backward_mode": args.mode, "path": args.path, "B": B, "F": F, "T": T, "depth": depth,
                    "extra_outputs": M},
-        "roofline": {"bound": "hbm", "kernel": "forward_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": "forward_rows_kernel" if name != "c1" else "forward", "achieved": achieved, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get(name),
                      "algorithmic_bytes": fwd_bytes, "ms": fwd_ms, "samples_per_s": B / (fwd_ms * 1e-3)},
         "backward": {"mode": args.mode, "ms": bwd_ms, "samples_per_s": B / (bwd_ms * 1e-3),

@@ -737,12 +737,25 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
   __syncthreads();
   const long long s_begin = (long long)blockIdx.y * part_size;
   const long long s_end = min(d.S, s_begin + part_size);
-  for (long long s = s_begin + threadIdx.x; s < s_end; s += 256) {
-    const long long at = (long long)t * d.S + s;
-    if (FIXED)
-      atomicAdd(reinterpret_cast<unsigned long long *>(acc) + rec.vertex(at), to_fixed(-double(rec.c[at]), scale));
-    else
-      atomicAdd(reinterpret_cast<double *>(acc) + rec.vertex(at), -double(rec.c[at]));
+  constexpr int kBatch = 8;  // loads in flight per thread
+  for (long long s0 = s_begin + threadIdx.x; s0 < s_end; s0 += 256 * kBatch) {
+    uint32_t v[kBatch];
+    Real cv[kBatch];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      const long long s = min(s0 + i * 256, s_end - 1);
+      const long long at = (long long)t * d.S + s;
+      v[i] = rec.vertex(at);
+      cv[i] = rec.c[at];
+    }
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      if (s0 + i * 256 >= s_end) break;
+      if (FIXED)
+        atomicAdd(reinterpret_cast<unsigned long long *>(acc) + v[i], to_fixed(-double(cv[i]), scale));
+      else
+        atomicAdd(reinterpret_cast<double *>(acc) + v[i], -double(cv[i]));
+    }
   }
   __syncthreads();
   Real *dst = dthr + (long long)t * d.V;
@@ -788,13 +801,26 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
   const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
   const long long s = s0 + j;
   if (s < d.S) {
-    for (int t = tt; t < d.T; t += TC) {
-      const long long at = (long long)t * d.S + s;
-      if (FIXED)
-        atomicAdd(reinterpret_cast<unsigned long long *>(acc) + rec.ord(at) * LD + j,
-                  to_fixed(double(rec.c[at]), scale));
-      else
-        lds_add(reinterpret_cast<Real *>(acc) + rec.ord(at) * LD + j, rec.c[at]);
+    // the loads of several trees are issued together: the loop is otherwise bound by one memory round trip per tree
+    constexpr int kBatch = 8;
+    for (int t0 = tt; t0 < d.T; t0 += TC * kBatch) {
+      uint32_t o[kBatch];
+      Real cv[kBatch];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        const int t = min(t0 + i * TC, d.T - 1);
+        const long long at = (long long)t * d.S + s;
+        o[i] = rec.ord(at);
+        cv[i] = __builtin_nontemporal_load(rec.c + at);
+      }
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        if (t0 + i * TC >= d.T) break;
+        if (FIXED)
+          atomicAdd(reinterpret_cast<unsigned long long *>(acc) + o[i] * LD + j, to_fixed(double(cv[i]), scale));
+        else
+          lds_add(reinterpret_cast<Real *>(acc) + o[i] * LD + j, cv[i]);
+      }
     }
   }
   __syncthreads();
