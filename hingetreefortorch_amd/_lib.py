@@ -51,6 +51,11 @@ SIGNATURES = {
     "ht_conv_output_size": (_I, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int64)]),
     "ht_conv_forward": (_I, [ctypes.POINTER(ConvShape), _P, _P, _P, _P, _P, _P]),
     "ht_conv_backward": (_I, [ctypes.POINTER(ConvShape), _P, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "ht_projection_workspace": (_SZ, [ctypes.c_int64]),
+    "ht_projection_forward": (_I, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _P, _P, ctypes.c_double, _P, _P, _P,
+                                   _P, _P, _SZ, _P]),
+    "ht_projection_backward": (_I, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _P, _P, _P, _P, _P, _P, _P, _P,
+                                    _SZ, _P]),
     "ht_check_thresholds": (_I, [_P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),
     "ht_fix_thresholds": (_I, [_P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),
 }

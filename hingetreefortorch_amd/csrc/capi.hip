@@ -287,6 +287,29 @@ static int thresholds_common(int64_t T, int64_t depth, int32_t dtype, int32_t ki
   return HT_OK;
 }
 
+size_t ht_projection_workspace(int64_t N) { return N < 0 ? 0 : projection_workspace(N); }
+
+int ht_projection_forward(int64_t B, int64_t K, int64_t N, const float *x, const float *lin, double eps, float *zhat,
+                          float *mean, float *rstd, float *var, void *workspace, size_t workspace_bytes, void *stream) {
+  if (B < 0 || K < 0 || N < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if (N > 0 && (!mean || !rstd || !workspace)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (B > 0 && N > 0 && (!zhat || (K > 0 && (!x || !lin)))) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (workspace_bytes < projection_workspace(N))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the projection.");
+  return projection_forward(B, K, N, x, lin, eps, zhat, mean, rstd, var, workspace, static_cast<hipStream_t>(stream));
+}
+
+int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, const float *lin, const float *zhat,
+                           const float *rstd, float *g, float *dlin, float *dx, void *workspace,
+                           size_t workspace_bytes, void *stream) {
+  if (B < 0 || K < 0 || N < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if (B > 0 && N > 0 && (!zhat || !rstd || !g || !workspace || (dlin && !x) || (dx && !lin)))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (workspace_bytes < projection_workspace(N))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the projection.");
+  return projection_backward(B, K, N, x, lin, zhat, rstd, g, dlin, dx, workspace, static_cast<hipStream_t>(stream));
+}
+
 int ht_check_thresholds(const void *thr, const int64_t *ord, int64_t T, int64_t depth, int32_t dtype, int32_t kind,
                         uint8_t *flags) {
   int64_t V;

@@ -109,6 +109,13 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
                   const Real *gout, Real *dx, Real *dthr, Real *dw, hipStream_t stream);
 
 int conv_output_size(const ht_conv_shape &s, int64_t *out_size);
+
+// Dense projection + batch normalisation in front of a forest (projection.hip), fp32.
+size_t projection_workspace(long long N);
+int projection_forward(long long B, long long K, long long N, const float *x, const float *lin, double eps,
+                       float *zhat, float *mean, float *rstd, float *var, void *ws, hipStream_t stream);
+int projection_backward(long long B, long long K, long long N, const float *x, const float *lin, const float *zhat,
+                        const float *rstd, float *g, float *dlin, float *dx, void *ws, hipStream_t stream);
 int ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, hipStream_t stream);
 
 // Fills `bytes` bytes with zero through a kernel (safe to record into a HIP graph, unlike a memset node).

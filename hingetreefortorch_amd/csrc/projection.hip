@@ -1,0 +1,342 @@
+// Dense projection in front of a forest: z = x * lin^T on the matrix cores, batch statistics of z in the same pass,
+// normalisation in place, and the matching backward (batch-norm backward + dLin = dz^T * x, dX = dz * lin).
+//
+// This is the Linear -> BatchNorm1d(affine=False) -> RandomHingeForest composition of the reference's README
+// (README.md:117-129, experiments/run_letter_seq.py:45-52) with the two dense stages written for gfx950: the only
+// place of this library where MFMA applies. fp32 in, fp32 accumulate (v_mfma_f32_32x32x2_f32).
+//
+// GEMM tiling: a workgroup of 256 threads (4 wavefronts, 2 x 2) owns a 128 x 128 tile of the result; a wavefront
+// owns 64 x 64 of it as 2 x 2 MFMA tiles (64 accumulator registers per lane). The reduction runs in steps of 16:
+// both operand tiles are staged in LDS reduction-major (tile[r][i], pitch 132), so the MFMA operand of lane l
+// (row l % 32, reduction index l / 32) is one conflict-free ds_read_b32, and the next step's global loads are in
+// flight while the current step is multiplied (register double buffering).
+#include "common.hpp"
+
+namespace ht {
+namespace {
+
+typedef float Acc16 __attribute__((ext_vector_type(16)));
+typedef float Vec4 __attribute__((ext_vector_type(4)));
+
+constexpr int kGemmThreads = 256;
+constexpr int kTile = 128;  // result tile edge
+constexpr int kRed = 16;    // reduction step
+constexpr int kPitch = kTile + 4;
+
+// Operand access patterns. An operand is a [rows x red] matrix that contributes tile[r][i] = op(i0 + i, r0 + r).
+//   RED_CONTIG  : element (i, r) at p[i * ld + r]   (reduction index contiguous: x and lin in z = x * lin^T)
+//   otherwise   : element (i, r) at p[r * ld + i]   (row index contiguous: dz and x in dLin = dz^T * x)
+// Each thread moves 2 x float4 per operand and step.
+struct Fetch {
+  Vec4 v[2];
+};
+
+template <bool RED_CONTIG>
+__device__ __forceinline__ void fetch_tile(Fetch &f, const float *__restrict__ p, long long ld, int i0, int n_i,
+                                           int r0, int n_r, bool vec_ok) {
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    Vec4 v = {0.f, 0.f, 0.f, 0.f};
+    if (RED_CONTIG) {
+      // thread -> (row i = t / 4 + 64 h, reduction quad q = t % 4)
+      const int i = i0 + t / 4 + 64 * h, r = r0 + (t % 4) * 4;
+      if (i < n_i) {
+        const float *src = p + (long long)i * ld + r;
+        if (vec_ok && r + 3 < n_r) {
+          v = *reinterpret_cast<const Vec4 *>(src);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (r + e < n_r) v[e] = src[e];
+        }
+      }
+    } else {
+      // thread -> (reduction index r = t / 32 + 8 h, row quad q = t % 32)
+      const int r = r0 + t / 32 + 8 * h, i = i0 + (t % 32) * 4;
+      if (r < n_r) {
+        const float *src = p + (long long)r * ld + i;
+        if (vec_ok && i + 3 < n_i) {
+          v = *reinterpret_cast<const Vec4 *>(src);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (i + e < n_i) v[e] = src[e];
+        }
+      }
+    }
+    f.v[h] = v;
+  }
+}
+
+template <bool RED_CONTIG>
+__device__ __forceinline__ void stash_tile(float *tile, const Fetch &f) {
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    if (RED_CONTIG) {
+      const int i = t / 4 + 64 * h, r = (t % 4) * 4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) tile[(r + e) * kPitch + i] = f.v[h][e];
+    } else {
+      const int r = t / 32 + 8 * h, i = (t % 32) * 4;
+      *reinterpret_cast<Vec4 *>(tile + r * kPitch + i) = f.v[h];
+    }
+  }
+}
+
+// C[i, j] = sum_r A(i, r) * B(j, r), i < n_i, j < n_j, r < n_r; C row-major with leading dimension ldc.
+// STATS: also accumulate per column j the sum and the sum of squares of C over i into stats[j], stats[n_j + j] (fp64
+// atomics; the batch statistics of the projection).
+template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS>
+__global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const float *__restrict__ A, long long lda,
+                                                            const float *__restrict__ B, long long ldb,
+                                                            float *__restrict__ C, long long ldc, int n_i, int n_j,
+                                                            int n_r, bool vec_a, bool vec_b, double *stats) {
+  __shared__ float As[2][kRed * kPitch];
+  __shared__ float Bs[2][kRed * kPitch];
+  const int i0 = blockIdx.y * kTile, j0 = blockIdx.x * kTile;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wavefront's 64 x 64 corner
+  const int lr = lane & 31, lk = lane >> 5;
+
+  Acc16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+
+  Fetch fa, fb;
+  fetch_tile<A_RED_CONTIG>(fa, A, lda, i0, n_i, 0, n_r, vec_a);
+  fetch_tile<B_RED_CONTIG>(fb, B, ldb, j0, n_j, 0, n_r, vec_b);
+  stash_tile<A_RED_CONTIG>(As[0], fa);
+  stash_tile<B_RED_CONTIG>(Bs[0], fb);
+  __syncthreads();
+  const int steps = (n_r + kRed - 1) / kRed;
+  for (int s = 0; s < steps; ++s) {
+    const int cur = s & 1;
+    if (s + 1 < steps) {
+      fetch_tile<A_RED_CONTIG>(fa, A, lda, i0, n_i, (s + 1) * kRed, n_r, vec_a);
+      fetch_tile<B_RED_CONTIG>(fb, B, ldb, j0, n_j, (s + 1) * kRed, n_r, vec_b);
+    }
+    const float *as = As[cur], *bs = Bs[cur];
+#pragma unroll
+    for (int kk = 0; kk < kRed; kk += 2) {
+      const float a0 = as[(kk + lk) * kPitch + wi + lr], a1 = as[(kk + lk) * kPitch + wi + 32 + lr];
+      const float b0 = bs[(kk + lk) * kPitch + wj + lr], b1 = bs[(kk + lk) * kPitch + wj + 32 + lr];
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    }
+    if (s + 1 < steps) {
+      stash_tile<A_RED_CONTIG>(As[cur ^ 1], fa);
+      stash_tile<B_RED_CONTIG>(Bs[cur ^ 1], fb);
+    }
+    __syncthreads();
+  }
+
+  // accumulator element e of lane l is C(row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32) of its 32 x 32 tile
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const int j = j0 + wj + 32 * b + lr;
+    double s1 = 0.0, s2 = 0.0;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int i = i0 + wi + 32 * a + 8 * (e / 4) + 4 * lk + (e % 4);
+        const float v = acc[a][b][e];
+        if (i < n_i && j < n_j) {
+          C[(long long)i * ldc + j] = v;
+          if (STATS) {
+            s1 += double(v);
+            s2 += double(v) * double(v);
+          }
+        }
+      }
+    }
+    if (STATS) {
+      s1 += __shfl_xor(s1, 32, 64);
+      s2 += __shfl_xor(s2, 32, 64);
+      if (lk == 0 && j < n_j) {
+        atomicAdd(stats + j, s1);
+        atomicAdd(stats + n_j + j, s2);
+      }
+    }
+  }
+}
+
+// mean, rstd (and the biased variance) of every column from the accumulated sums.
+__global__ void bn_finalize_kernel(const double *__restrict__ stats, int N, long long B, double eps, float *mean,
+                                   float *rstd, float *var) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= N) return;
+  const double m = stats[j] / double(B);
+  double v = stats[N + j] / double(B) - m * m;
+  if (v < 0.0) v = 0.0;
+  mean[j] = float(m);
+  rstd[j] = float(1.0 / sqrt(v + eps));
+  if (var) var[j] = float(v);
+}
+
+// z <- (z - mean) * rstd, in place, row-major [B x N]. One thread per 4 consecutive columns of 8 rows.
+__global__ __launch_bounds__(256) void bn_apply_kernel(float *z, long long B, int N, const float *__restrict__ mean,
+                                                       const float *__restrict__ rstd) {
+  const int j = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (j >= N) return;
+  float m[4], r[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    m[e] = j + e < N ? mean[j + e] : 0.f;
+    r[e] = j + e < N ? rstd[j + e] : 0.f;
+  }
+  const bool vec = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(z) % 16 == 0);
+  for (long long i = blockIdx.y; i < B; i += gridDim.y) {
+    float *p = z + i * N + j;
+    if (vec) {
+      Vec4 v = *reinterpret_cast<Vec4 *>(p);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (v[e] - m[e]) * r[e];
+      *reinterpret_cast<Vec4 *>(p) = v;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (j + e < N) p[e] = (p[e] - m[e]) * r[e];
+    }
+  }
+}
+
+// Column sums of g and of g * zhat over the rows (fp64 atomics into sums[j], sums[N + j]).
+__global__ __launch_bounds__(256) void bn_backward_sums_kernel(const float *__restrict__ g,
+                                                               const float *__restrict__ zhat, long long B, int N,
+                                                               double *sums) {
+  const int j = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (j >= N) return;
+  double s1[4] = {0, 0, 0, 0}, s2[4] = {0, 0, 0, 0};
+  const bool vec = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(g) % 16 == 0) &&
+                   (reinterpret_cast<uintptr_t>(zhat) % 16 == 0);
+  for (long long i = blockIdx.y; i < B; i += gridDim.y) {
+    float gv[4], zv[4];
+    if (vec) {
+      const Vec4 a = *reinterpret_cast<const Vec4 *>(g + i * N + j), b = *reinterpret_cast<const Vec4 *>(zhat + i * N + j);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) gv[e] = a[e], zv[e] = b[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        gv[e] = j + e < N ? g[i * N + j + e] : 0.f;
+        zv[e] = j + e < N ? zhat[i * N + j + e] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      s1[e] += double(gv[e]);
+      s2[e] += double(gv[e]) * double(zv[e]);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    if (j + e < N) {
+      atomicAdd(sums + j + e, s1[e]);
+      atomicAdd(sums + N + j + e, s2[e]);
+    }
+}
+
+// g <- rstd * (g - mean(g) - zhat * mean(g * zhat)), in place (batch-norm backward without affine parameters).
+__global__ __launch_bounds__(256) void bn_backward_apply_kernel(float *g, const float *__restrict__ zhat, long long B,
+                                                                int N, const float *__restrict__ rstd,
+                                                                const double *__restrict__ sums) {
+  const int j = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (j >= N) return;
+  float r[4], m1[4], m2[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const bool in = j + e < N;
+    r[e] = in ? rstd[j + e] : 0.f;
+    m1[e] = in ? float(sums[j + e] / double(B)) : 0.f;
+    m2[e] = in ? float(sums[N + j + e] / double(B)) : 0.f;
+  }
+  const bool vec = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(g) % 16 == 0) &&
+                   (reinterpret_cast<uintptr_t>(zhat) % 16 == 0);
+  for (long long i = blockIdx.y; i < B; i += gridDim.y) {
+    float *p = g + i * N + j;
+    const float *q = zhat + i * N + j;
+    if (vec) {
+      Vec4 a = *reinterpret_cast<Vec4 *>(p);
+      const Vec4 b = *reinterpret_cast<const Vec4 *>(q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) a[e] = r[e] * (a[e] - m1[e] - b[e] * m2[e]);
+      *reinterpret_cast<Vec4 *>(p) = a;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (j + e < N) p[e] = r[e] * (p[e] - m1[e] - q[e] * m2[e]);
+    }
+  }
+}
+
+bool aligned16(const void *p, long long ld) { return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0; }
+
+template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS>
+int launch_gemm(const float *A, long long lda, const float *B, long long ldb, float *C, long long ldc, long long n_i,
+                long long n_j, long long n_r, double *stats, hipStream_t stream) {
+  if (n_i <= 0 || n_j <= 0) return HT_OK;
+  const long long gi = (n_i + kTile - 1) / kTile, gj = (n_j + kTile - 1) / kTile;
+  if (gi > 65535 || gj > 0x7fffffffLL || n_r > 0x7fffffffLL || n_i > 0x7fffffffLL || n_j > 0x7fffffffLL)
+    return fail(HT_ERR_RUNTIME, "Error: projection too large for this build.");
+  hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS>), dim3((unsigned)gj, (unsigned)gi), dim3(kGemmThreads), 0, stream,
+                     A, lda, B, ldb, C, ldc, int(n_i), int(n_j), int(n_r), aligned16(A, lda), aligned16(B, ldb), stats);
+  HT_LAUNCH_CHECK("projection (matrix cores)");
+  return HT_OK;
+}
+
+long long rows_grid(long long B) { return B < 64 ? (B < 1 ? 1 : B) : 64; }
+
+}  // namespace
+
+size_t projection_workspace(long long N) { return align_up(size_t(2) * size_t(N) * sizeof(double), 256); }
+
+// zhat [B x N] = normalised (x [B x K] * lin [N x K]^T); mean, rstd, var [N] out; ws: projection_workspace(N).
+int projection_forward(long long B, long long K, long long N, const float *x, const float *lin, double eps,
+                       float *zhat, float *mean, float *rstd, float *var, void *ws, hipStream_t stream) {
+  int rc;
+  double *stats = static_cast<double *>(ws);
+  if ((rc = zero_fill(stats, size_t(2) * N * sizeof(double), stream)) != HT_OK) return rc;
+  if (B == 0 || N == 0) return HT_OK;
+  if ((rc = launch_gemm<true, true, true>(x, K, lin, K, zhat, N, B, N, K, stats, stream)) != HT_OK) return rc;
+  hipLaunchKernelGGL(bn_finalize_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, stats, int(N), B, eps,
+                     mean, rstd, var);
+  HT_LAUNCH_CHECK("batch statistics");
+  hipLaunchKernelGGL(bn_apply_kernel, dim3((unsigned)((N + 1023) / 1024), (unsigned)rows_grid(B)), dim3(256), 0, stream,
+                     zhat, B, int(N), mean, rstd);
+  HT_LAUNCH_CHECK("normalisation");
+  return HT_OK;
+}
+
+// g [B x N] holds dL/dzhat on entry and dL/dz on return. dlin [N x K] and / or dx [B x K] out (either may be null).
+int projection_backward(long long B, long long K, long long N, const float *x, const float *lin, const float *zhat,
+                        const float *rstd, float *g, float *dlin, float *dx, void *ws, hipStream_t stream) {
+  int rc;
+  double *sums = static_cast<double *>(ws);
+  if ((rc = zero_fill(sums, size_t(2) * N * sizeof(double), stream)) != HT_OK) return rc;
+  if (B == 0 || N == 0) {
+    if (dlin && (rc = zero_fill(dlin, size_t(N) * K * sizeof(float), stream)) != HT_OK) return rc;
+    if (dx && (rc = zero_fill(dx, size_t(B) * K * sizeof(float), stream)) != HT_OK) return rc;
+    return HT_OK;
+  }
+  const dim3 grid((unsigned)((N + 1023) / 1024), (unsigned)rows_grid(B));
+  hipLaunchKernelGGL(bn_backward_sums_kernel, grid, dim3(256), 0, stream, g, zhat, B, int(N), sums);
+  HT_LAUNCH_CHECK("batch-norm backward (sums)");
+  hipLaunchKernelGGL(bn_backward_apply_kernel, grid, dim3(256), 0, stream, g, zhat, B, int(N), rstd, sums);
+  HT_LAUNCH_CHECK("batch-norm backward");
+  // dlin[n, k] = sum_b g[b, n] * x[b, k]: both operands row contiguous, reduction over the batch
+  if (dlin && (rc = launch_gemm<false, false, false>(g, N, x, K, dlin, K, N, K, B, nullptr, stream)) != HT_OK) return rc;
+  // dx[b, k] = sum_n g[b, n] * lin[n, k]: g has the reduction index n contiguous, lin the row index k
+  if (dx && (rc = launch_gemm<true, false, false>(g, N, lin, K, dx, K, B, K, N, nullptr, stream)) != HT_OK) return rc;
+  return HT_OK;
+}
+
+}  // namespace ht

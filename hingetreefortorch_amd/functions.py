@@ -141,3 +141,25 @@ HingeTreeConv3d = _conv_function("HingeTreeConv3d", "tree", 3, "tree")
 HingeFernConv1d = _conv_function("HingeFernConv1d", "fern", 1, "fern")
 HingeFernConv2d = _conv_function("HingeFernConv2d", "fern", 2, "fern")
 HingeFernConv3d = _conv_function("HingeFernConv3d", "fern", 3, "fern")
+
+
+class LinearBatchNorm(torch.autograd.Function):
+    """zhat = BatchNorm1d(affine=False, training)(Linear(bias=False)(x)) as one operator on the HIP library: the dense
+    front of the reference's README model (README.md:117-129). forward(ctx, inData, inLinearWeights, eps) returns
+    (zhat, mean, var); mean and the biased batch variance are for the caller's running statistics and carry no
+    gradient."""
+
+    @staticmethod
+    def forward(ctx, inData, inLinearWeights, eps):
+        zhat, mean, rstd, var = _ops.linear_bn_forward(inData, inLinearWeights, eps)
+        ctx.save_for_backward(inData, inLinearWeights, zhat, rstd)
+        ctx.mark_non_differentiable(mean, var)
+        return zhat, mean, var
+
+    @staticmethod
+    def backward(ctx, outDataGrad, _mean_grad, _var_grad):
+        inData, inLinearWeights, zhat, rstd = ctx.saved_tensors
+        g = outDataGrad.contiguous().clone()  # the operator works in place on the upstream gradient
+        dx, dlin = _ops.linear_bn_backward(inData, ctx.needs_input_grad[0], inLinearWeights, ctx.needs_input_grad[1],
+                                           zhat, rstd, g)
+        return dx, dlin, None

@@ -97,6 +97,63 @@ def _validate_ordinals(ordinals, limit):
     _range_ok[key] = (ref, ordinals._version, bound)
 
 
+# ---- dense projection + batch normalisation in front of a forest ------------------------------------------------
+def linear_bn_forward(inData, inLinearWeights, eps=1e-5):
+    """zhat = batch_norm(inData @ inLinearWeights.T) in training mode without affine parameters: the Linear(bias=False)
+    -> BatchNorm1d(affine=False) front of the reference's README model (README.md:117-129), with the product on the
+    matrix cores and the batch sums taken by the same kernel. Returns [zhat, mean, rstd, var] (var: biased)."""
+    if inData.dtype != torch.float32 or inLinearWeights.dtype != torch.float32:
+        _invalid("Error: the projection supports torch.float32 only.")
+    if inData.device != inLinearWeights.device:
+        _invalid("Error: All tensors are expected to be on the same device.")
+    if not inData.is_cuda:
+        _runtime("Error: this build has no CPU back-end; tensors must be on a GPU.")
+    if not inData.is_contiguous() or not inLinearWeights.is_contiguous():
+        _invalid("Error: All tensors are expected to be contiguous.")
+    if inData.dim() != 2 or inLinearWeights.dim() != 2 or inData.shape[1] != inLinearWeights.shape[1]:
+        _invalid("Error: inData must be [batch, in_features] and inLinearWeights [out_features, in_features].")
+    B, K = inData.shape
+    N = inLinearWeights.shape[0]
+    lib = L.load()
+    with torch.cuda.device(inData.device):
+        zhat = torch.empty([B, N], dtype=torch.float32, device=inData.device)
+        mean, rstd, var = (torch.empty([N], dtype=torch.float32, device=inData.device) for _ in range(3))
+        nbytes = lib.ht_projection_workspace(N)
+        ws = _workspace(nbytes, inData.device)
+        L.check(lib.ht_projection_forward(B, K, N, _ptr(inData), _ptr(inLinearWeights), float(eps), _ptr(zhat),
+                                          _ptr(mean), _ptr(rstd), _ptr(var), _ptr(ws), nbytes,
+                                          _stream(inData.device)))
+    return [zhat, mean, rstd, var]
+
+
+def linear_bn_backward(inData, bInDataGrad, inLinearWeights, bInLinearWeightsGrad, zhat, rstd, outDataGrad):
+    """Gradients of linear_bn_forward for an upstream gradient on zhat. `outDataGrad` is overwritten (it becomes the
+    gradient with respect to the un-normalised product). Returns [dData | None, dLinearWeights | None]."""
+    for t in (inData, inLinearWeights, zhat, rstd, outDataGrad):
+        if t.dtype != torch.float32:
+            _invalid("Error: the projection supports torch.float32 only.")
+        if not t.is_contiguous():
+            _invalid("Error: All tensors are expected to be contiguous.")
+        if t.device != inData.device:
+            _invalid("Error: All tensors are expected to be on the same device.")
+    if not inData.is_cuda:
+        _runtime("Error: this build has no CPU back-end; tensors must be on a GPU.")
+    B, K = inData.shape
+    N = inLinearWeights.shape[0]
+    if zhat.shape != (B, N) or outDataGrad.shape != (B, N) or rstd.shape != (N,):
+        _invalid("Error: shapes of zhat / rstd / outDataGrad do not match the projection.")
+    lib = L.load()
+    with torch.cuda.device(inData.device):
+        dx = torch.empty_like(inData) if bInDataGrad else None
+        dlin = torch.empty_like(inLinearWeights) if bInLinearWeightsGrad else None
+        nbytes = lib.ht_projection_workspace(N)
+        ws = _workspace(nbytes, inData.device)
+        L.check(lib.ht_projection_backward(B, K, N, _ptr(inData), _ptr(inLinearWeights), _ptr(zhat), _ptr(rstd),
+                                           _ptr(outDataGrad), _ptr(dlin), _ptr(dx), _ptr(ws), nbytes,
+                                           _stream(inData.device)))
+    return [dx, dlin]
+
+
 # ---- forest / fern ------------------------------------------------------------------------------------------------
 def _common_checks(tensors, ordinals, with_grad):
     data = tensors[0]
@@ -519,4 +576,4 @@ for _name in ["sparse_tree_backward", "sparse_fern_backward", "tree_init_medians
               "fern_fusion_fused_linear_backward", "contract", "expand"]:
     globals()[_name] = _outside(_name)
 
-__all__ = [n for n in list(globals()) if n.split("_")[0] in ("tree", "fern", "sparse", "trie", "contract", "expand")]
+__all__ = [n for n in list(globals()) if n.split("_")[0] in ("tree", "fern", "sparse", "trie", "contract", "expand", "linear")]

@@ -192,3 +192,36 @@ class HingeFernConv2d(_ConvBase):
 
 class HingeFernConv3d(_ConvBase):
     _function, _nd, _fern = _fn.HingeFernConv3d, 3, True
+
+
+class LinearHingeForest(nn.Module):
+    """Linear(bias=False) -> BatchNorm1d(affine=False) -> RandomHingeForest(init_type="sequential") as one module: the
+    model of the reference's README (README.md:117-129; experiments/run_letter_seq.py:45-52), where the linear layer
+    produces one private feature per decision vertex (out_channels * (2^depth - 1) of them). The projection and the
+    batch statistics run in one matrix-core kernel of the HIP library; in eval mode the running statistics are used.
+
+    Sub-module names and parameter shapes equal those of the three separate torch / reference modules (`fc.weight`,
+    `bn.running_mean`, `bn.running_var`, `bn.num_batches_tracked`, `forest.weights`, `forest.thresholds`,
+    `forest.ordinals`), so a state dict moves between the two forms unchanged."""
+
+    def __init__(self, in_features: int, out_channels: int, depth: int, extra_outputs=None, eps: float = 1e-5,
+                 momentum: float = 0.1):
+        super().__init__()
+        hidden = out_channels * (2 ** depth - 1)
+        self.fc = nn.Linear(in_features, hidden, bias=False)
+        self.bn = nn.BatchNorm1d(hidden, eps=eps, momentum=momentum, affine=False)
+        self.forest = RandomHingeForest(hidden, out_channels, depth, extra_outputs=extra_outputs,
+                                        init_type="sequential")
+
+    def forward(self, x):
+        if not self.training or not x.is_cuda or x.dtype != torch.float32:
+            return self.forest(self.bn(self.fc(x)))
+        zhat, mean, var = _fn.LinearBatchNorm.apply(x.contiguous(), self.fc.weight, self.bn.eps)
+        if self.bn.track_running_stats:
+            with torch.no_grad():
+                n = x.shape[0]
+                self.bn.num_batches_tracked += 1
+                m = self.bn.momentum if self.bn.momentum is not None else 1.0 / float(self.bn.num_batches_tracked)
+                self.bn.running_mean.mul_(1 - m).add_(mean, alpha=m)
+                self.bn.running_var.mul_(1 - m).add_(var * (n / max(n - 1, 1)), alpha=m)
+        return self.forest(zhat)

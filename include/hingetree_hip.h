@@ -110,6 +110,24 @@ int ht_conv_forward(const ht_conv_shape *s, const void *x, const void *thr, cons
 int ht_conv_backward(const ht_conv_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
                      const void *gout, void *dx, void *dthr, void *dw, void *stream);
 
+/* ---- dense projection + batch normalisation in front of a forest (fp32) --------------------------------------------
+ * The reference has no operator for this stage: its README and experiments compose torch.nn.Linear(bias=False),
+ * torch.nn.BatchNorm1d(affine=False) and RandomHingeForest (README.md:117-129, experiments/run_letter_seq.py:45-52).
+ * These two calls replace the first two modules of that composition in training mode; the forest operators above
+ * consume zhat unchanged.
+ *   forward : zhat [B, N] = (z - mean) * rstd with z = x [B, K] * lin [N, K]^T computed on the matrix cores; the batch
+ *             sums of z are accumulated by the same kernel. mean, rstd, var [N] are outputs (var: biased variance, for
+ *             the caller's running statistics; may be NULL).
+ *   backward: g [B, N] holds dL/dzhat on entry and is overwritten with dL/dz; dlin [N, K] and dx [B, K] receive the
+ *             parameter / input gradients (either may be NULL).
+ * workspace: ht_projection_workspace(N) bytes. */
+size_t ht_projection_workspace(int64_t N);
+int ht_projection_forward(int64_t B, int64_t K, int64_t N, const float *x, const float *lin, double eps, float *zhat,
+                          float *mean, float *rstd, float *var, void *workspace, size_t workspace_bytes, void *stream);
+int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, const float *lin, const float *zhat,
+                           const float *rstd, float *g, float *dlin, float *dx, void *workspace,
+                           size_t workspace_bytes, void *stream);
+
 /* Host-side (CPU pointers) threshold consistency, in place for _fix. One flag byte per tree is written to `flags`
  * (check: 1 = consistent; fix: 1 = changed). Ferns are always consistent and never change.
  * Replaces hingetree_cpu_check_thresholds / _fix_thresholds (hingetree.cpp:513-581, HingeTreeCommon.h:211-287); the

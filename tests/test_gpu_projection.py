@@ -1,0 +1,102 @@
+"""GPU checks of the dense projection + batch normalisation front (matrix-core GEMM with fused batch sums) and of the
+LinearHingeForest module built on it.
+
+Nothing in the reference pins the results of this stage (its README composes torch.nn.Linear and BatchNorm1d, whose
+outputs depend on the installed BLAS): parity unpinned beyond fp32 tolerance. The checks are therefore against what the
+mathematics fixes: an fp64 matrix product, batch statistics of exactly mean 0 / variance 1, and the closed-form
+batch-norm and linear gradients, all within 1e-5 relative to the largest entry; the forest stage behind the projection is
+checked bit-exactly against the CPU oracle on the very zhat the projection produced.
+"""
+import pytest
+import torch
+
+from conftest import rel_err
+from oracle import hinge_oracle as ho
+import hingetree_cpp as ops
+from hingetreefortorch_amd import LinearHingeForest
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(1, 1, 1), (7, 5, 3), (64, 16, 128), (200, 37, 130), (300, 784, 381), (129, 40, 257)]
+
+
+def _reference(x, lin, eps):
+    z = x.double() @ lin.double().t()
+    mean = z.mean(0)
+    var = z.var(0, unbiased=False)
+    rstd = 1.0 / torch.sqrt(var + eps)
+    return (z - mean) * rstd, mean, rstd, var
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=[f"{b}x{k}x{n}" for b, k, n in SHAPES])
+def test_projection_forward_backward(dev, shape):
+    B, K, N = shape
+    g = torch.Generator().manual_seed(11)
+    x = torch.rand([B, K], generator=g)
+    lin = torch.randn([N, K], generator=g) / K ** 0.5
+    up = torch.randn([B, N], generator=g)
+    eps = 1e-5
+    zhat, mean, rstd, var = ops.linear_bn_forward(x.to(dev), lin.to(dev), eps)
+    rz, rmean, rrstd, rvar = _reference(x, lin, eps)
+    assert rel_err(zhat.cpu().double(), rz) <= 2e-5
+    assert rel_err(mean.cpu().double(), rmean) <= 1e-5 and rel_err(var.cpu().double(), rvar) <= 1e-5
+    if B > 1:
+        assert rel_err(rstd.cpu().double(), rrstd) <= 1e-4
+    # closed-form gradients in fp64: dz = rstd * (g - mean(g) - zhat * mean(g * zhat)); dlin = dz^T x; dx = dz lin
+    gd = up.double()
+    dz = rrstd * (gd - gd.mean(0) - rz * (gd * rz).mean(0))
+    rdlin, rdx = dz.t() @ x.double(), dz @ lin.double()
+    gbuf = up.to(dev).clone()
+    dx, dlin = ops.linear_bn_backward(x.to(dev), True, lin.to(dev), True, zhat, rstd, gbuf)
+    scale = max(float(rrstd.abs().max()), 1.0)   # near-constant columns amplify rounding by rstd
+    assert rel_err(dlin.cpu().double(), rdlin) <= 2e-5 * scale
+    assert rel_err(dx.cpu().double(), rdx) <= 2e-5 * scale
+    only = ops.linear_bn_backward(x.to(dev), False, lin.to(dev), True, zhat, rstd, up.to(dev).clone())
+    assert only[0] is None and rel_err(only[1].cpu().double(), rdlin) <= 2e-5 * scale
+
+
+def test_projection_rejects_bad_input(dev):
+    x = torch.rand([4, 3], device=dev)
+    lin = torch.rand([5, 2], device=dev)
+    with pytest.raises(ValueError):
+        ops.linear_bn_forward(x, lin)
+    with pytest.raises(ValueError):
+        ops.linear_bn_forward(x.double(), torch.rand([5, 3], device=dev).double())
+    with pytest.raises(RuntimeError):
+        ops.linear_bn_forward(x.cpu(), torch.rand([5, 3]))
+
+
+def test_linear_hinge_forest_matches_composition(dev):
+    """The fused module against torch.nn.Linear -> BatchNorm1d -> RandomHingeForest with the same parameters: zhat within
+    fp32 tolerance, the forest stage bit-exact on the module's own zhat, gradients within tolerance, running statistics
+    updated like BatchNorm1d does."""
+    torch.manual_seed(5)
+    B, K, T, depth, M = 96, 20, 6, 3, 4
+    model = LinearHingeForest(K, T, depth, extra_outputs=M).to(dev)
+    ref_fc = torch.nn.Linear(K, T * 7, bias=False).to(dev)
+    ref_bn = torch.nn.BatchNorm1d(T * 7, affine=False).to(dev)
+    ref_fc.weight.data.copy_(model.fc.weight.data)
+    x = torch.rand([B, K], device=dev)
+    model.train()
+    out = model(x)
+    zref = ref_bn(ref_fc(x))
+    zhat, _, _, _ = ops.linear_bn_forward(x, model.fc.weight.detach().contiguous(), model.bn.eps)
+    assert rel_err(zhat.cpu(), zref.detach().cpu()) <= 2e-5
+    assert rel_err(model.bn.running_mean.cpu(), ref_bn.running_mean.cpu()) <= 1e-5
+    assert rel_err(model.bn.running_var.cpu(), ref_bn.running_var.cpu()) <= 1e-5
+    want = ho.forward(zhat.cpu(), model.forest.thresholds.detach().cpu(), model.forest.ordinals.cpu(),
+                      model.forest.weights.detach().cpu(), False)
+    assert torch.equal(out.detach().cpu(), want)
+    up = torch.randn_like(out)
+    out.backward(up)
+    # gradient of the projection weights through the closed form, from the forest's own input gradient
+    zl = zhat.detach().clone().requires_grad_(True)
+    o2 = model.forest(zl)
+    o2.backward(up)
+    gd, rz = zl.grad.double().cpu(), zhat.double().cpu()
+    z = x.double().cpu() @ model.fc.weight.detach().double().cpu().t()
+    rstd = 1.0 / torch.sqrt(z.var(0, unbiased=False) + model.bn.eps)
+    dz = rstd * (gd - gd.mean(0) - rz * (gd * rz).mean(0))
+    assert rel_err(model.fc.weight.grad.double().cpu(), dz.t() @ x.double().cpu()) <= 5e-5
+    model.eval()
+    assert model(x).shape == out.shape
