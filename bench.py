@@ -18,6 +18,9 @@ ordinals ~ U{0..1023}, leaf weights ~ N(0,1), upstream gradient ~ N(0,1).
 the channels); it is bound by LDS reads and vector instructions, not by HBM, so its line reports images/s and vertex
 visits/s with the HBM fraction for information only.
 
+`--workload c5` times the README model's dense front plus forest (linear_bn_forward -> tree_forward ->
+tree_backward -> linear_bn_backward); its roofline object prices the projection against the fp32 matrix-core peak.
+
 Prints ONE JSON line. `value` is samples/s over the timed steps (wall clock between device synchronisations);
 `roofline` prices the dominant kernel (the forward kernel: tree_forward launches it plus a ~7 us vertex-packing
 pre-pass) against the 8 TB/s HBM peak using its algorithmic bytes (every input read once, every output written once)
@@ -154,12 +157,75 @@ def bench_conv(torch, ops, dev, args):
     }
 
 
+MFMA_FP32_PEAK_TFLOPS = 157.3
+
+
+def bench_projection(torch, ops, dev, args):
+    """Linear(784 -> 12700, no bias) -> BatchNorm1d(affine=False) -> forest (100 trees, depth 7, sequential ordinals,
+    10 outputs per leaf), forward+backward with gradients for the projection, the thresholds and the leaf weights."""
+    B, K, T, depth, M = 16384, 784, 100, 7, 10
+    V, L = 2 ** depth - 1, 2 ** depth
+    N = T * V
+    g = torch.Generator().manual_seed(6112)
+    x = torch.rand([B, K], generator=g).to(dev)
+    lin = (torch.randn([N, K], generator=g) / K ** 0.5).to(dev)
+    thr = 6.0 * torch.rand([T, V], generator=g) - 3.0
+    ordn = torch.arange(N, dtype=torch.int64).reshape(T, V)
+    w = torch.randn([T, L, M], generator=g)
+    ops.tree_fix_thresholds(thr, ordn, w)
+    thr, ordn, w = thr.to(dev), ordn.to(dev), w.to(dev)
+    gout = torch.randn([B, T, M], generator=torch.Generator(device=dev).manual_seed(6113), device=dev)
+
+    def step(ev=None):
+        if ev: ev[0].record()
+        zhat, mean, rstd, var = ops.linear_bn_forward(x, lin, 1e-5)
+        if ev: ev[1].record()
+        out = ops.tree_forward(zhat, thr, ordn, w)
+        if ev: ev[2].record()
+        dz, dthr, _, dw = ops.tree_backward(zhat, True, thr, True, ordn, False, w, True, gout)
+        if ev: ev[3].record()
+        ops.linear_bn_backward(x, False, lin, True, zhat, rstd, dz)
+        if ev: ev[4].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(ev[i])
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    seg = [sum(e[i].elapsed_time(e[i + 1]) for e in ev) / args.steps for i in range(4)]
+    flops = 2.0 * B * K * N
+    tf_fwd, tf_bwd = flops / (seg[0] * 1e-3) / 1e12, flops / (seg[3] * 1e-3) / 1e12
+    return {
+        "metric": "fwd+bwd samples/s (Linear 784->12700 + BatchNorm + forest T=100,D=7,M=10, B=16384)",
+        "value": B / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "c5: x~U[0,1) [16384,784], bias-free linear to 12700 = 100 x 127 private vertex features, "
+                               "batch norm without affine, forest 100 trees depth 7 sequential ordinals, 10 outputs "
+                               "per leaf; gradients: linear weights, thresholds, leaf weights", "B": B, "K": K, "N": N,
+                   "T": T, "depth": depth, "extra_outputs": M},
+        "projection_forward": {"ms": seg[0], "tflops": tf_fwd,
+                               "note": "GEMM with fused batch sums + statistics + in-place normalisation"},
+        "forest_forward_ms": seg[1], "forest_backward_ms": seg[2],
+        "projection_backward": {"ms": seg[3], "tflops": tf_bwd,
+                                "note": "batch-norm backward (two passes over [B, N]) + dLin = dz^T x GEMM"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel (projection forward)", "achieved": tf_fwd,
+                     "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf_fwd / MFMA_FP32_PEAK_TFLOPS,
+                     "traffic": None, "flops": flops,
+                     "note": "the timed span also holds the statistics and normalisation kernels"},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "c5"])
     ap.add_argument("--mode", default="atomic", choices=["atomic", "deterministic"])
     ap.add_argument("--path", default="train", choices=["train", "stateless"])
     ap.add_argument("--other-steps", type=int, default=-1,
@@ -190,6 +256,9 @@ def main():
     name = args.workload
     if name == "c4":
         print(json.dumps(bench_conv(torch, ops, dev, args)), flush=True)
+        return
+    if name == "c5":
+        print(json.dumps(bench_projection(torch, ops, dev, args)), flush=True)
         return
     B, F, T, depth, M, kind, _, desc = WORKLOADS[name]
     x, thr, ordn, w, gout = make_inputs(torch, name, dev)
