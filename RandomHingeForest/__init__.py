@@ -9,4 +9,5 @@ from hingetreefortorch_amd.modules import (  # noqa: F401
     HingeFernConv1d,
     HingeFernConv2d,
     HingeFernConv3d,
+    LinearHingeForest,
 )
