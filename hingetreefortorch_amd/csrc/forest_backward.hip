@@ -845,6 +845,19 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
   }
 }
 
+// dX for feature spaces too wide for an LDS tile (atomic mode): one global atomic per (tree, sample) pair straight
+// into the pre-cleared dX. With F in the thousands two pairs of one sample rarely meet, so the atomics do not
+// contend; the pair count, not the feature count, sets the cost.
+template <typename Real, bool COMPACT>
+__global__ __launch_bounds__(256) void dx_scatter_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dx) {
+  const long long pairs = (long long)d.T * d.S;
+  for (long long at = (long long)blockIdx.x * 256 + threadIdx.x; at < pairs; at += (long long)gridDim.x * 256) {
+    const long long s = at % d.S;
+    const Real c = rec.c[at];
+    if (c != Real(0)) atomicAdd(dx + (s / d.K) * d.FK + (long long)rec.ord(at) * d.K + (s % d.K), c);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // fused kernel with global atomics (small problems, depth > 16, F > 65536, huge leaf tables)
 // ---------------------------------------------------------------------------------------------------------------
@@ -1218,7 +1231,8 @@ bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw, bool fixed) {
   if ((long long)d.T * d.M * kWave >= (1ll << 31)) return false;
   if (need_dw && size_t(d.L) * d.M * sizeof(double) > size_t(kLdsBytes)) return false;
   if (size_t(d.V) * sizeof(double) > size_t(kLdsBytes)) return false;
-  if (need_dx && pick_dx_tile(d.F, fixed ? sizeof(unsigned long long) : sizeof(Real)) == 0) return false;
+  // (atomic mode serves a feature space too wide for the dX tile with one global atomic per pair instead)
+  if (need_dx && fixed && pick_dx_tile(d.F, sizeof(unsigned long long)) == 0) return false;
   return true;
 }
 
@@ -1351,7 +1365,15 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
       case 64: rc = launch_dx<Real, 64, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
       case 32: rc = launch_dx<Real, 32, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
       case 16: rc = launch_dx<Real, 16, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
-      default: rc = launch_dx<Real, 8, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
+      case 8: rc = launch_dx<Real, 8, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
+      default: {  // no tile fits (atomic mode only, see staged_ok); dX was cleared by the caller
+        const long long pairs = (long long)d.T * d.S;
+        long long blocks = (pairs + 255) / 256;
+        if (blocks > 16 * kNumCUs) blocks = 16 * kNumCUs;
+        hipLaunchKernelGGL((dx_scatter_kernel<Real, COMPACT>), dim3((unsigned)blocks), dim3(256), 0, stream, d, rec, dx);
+        HT_LAUNCH_CHECK("forest backward (dX, scattered)");
+        break;
+      }
     }
     if (rc != HT_OK) return rc;
     if (FIXED) {
@@ -1451,7 +1473,7 @@ template <typename Real>
 int clear_gradients(const ForestDims &d, Route route, Real *dx, Real *dthr, Real *dw, hipStream_t stream, bool *done) {
   int rc;
   const bool empty = d.S == 0 || d.T == 0;
-  const bool clear_dx = route != Route::kStaged || empty;
+  const bool clear_dx = route != Route::kStaged || empty || pick_dx_tile(d.F, sizeof(Real)) == 0;
   if (dx && clear_dx && (rc = zero_fill(dx, size_t(d.S) * d.F * sizeof(Real), stream)) != HT_OK) return rc;
   if (dthr && (rc = zero_fill(dthr, size_t(d.T) * d.V * sizeof(Real), stream)) != HT_OK) return rc;
   if (dw && (rc = zero_fill(dw, size_t(d.T) * d.L * d.M * sizeof(Real), stream)) != HT_OK) return rc;

@@ -33,6 +33,9 @@ CASES = [
     (2100, 33, [], 126, 4, []),
     (600, 16, [], 450, 3, [8, 8]),         # 64 outputs per leaf: 16 lanes per pair with 4-wide loads
     (520, 12, [], 520, 3, [70]),           # more outputs per leaf than a wavefront has lanes: fused kernel
+    # staged backward with a feature space too wide for the dX tile: dX by one global atomic per pair
+    (600, 6000, [], 500, 4, [10]),
+    (40, 5000, [8], 900, 3, [2]),
 ]
 
 
