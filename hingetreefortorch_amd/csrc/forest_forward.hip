@@ -194,9 +194,15 @@ __global__ __launch_bounds__(256) void pack_quads_kernel(const float *__restrict
   quads[i] = n;
 }
 
+constexpr int kTopQuads = 5;  // quads of the first two level pairs (levels 0..3): 1 + 4
+
 // N interleaved walks over quads; xs_j = this lane's column of the feature-major sample tile (pitch BT).
-template <int N, int BT>
-__device__ __forceinline__ void walk_quads(int depth, const QuadNode *const (&quads)[N], const float *xs_j,
+// TOP_LDS: top[i] is an LDS copy of the first kTopQuads quads of walk i's tree; levels 0..3 are then read from LDS
+// (the same for all samples of a tree slot: broadcasts), which takes two of the five dependent memory round trips
+// out of a depth-10 walk.
+template <int N, int BT, bool TOP_LDS>
+__device__ __forceinline__ void walk_quads(int depth, const QuadNode *const (&quads)[N],
+                                           const QuadNode *const (&top)[N], const float *xs_j,
                                            WalkResult<float> (&r)[N]) {
   uint32_t idx[N];
   float best_abs[N];
@@ -213,8 +219,13 @@ __device__ __forceinline__ void walk_quads(int depth, const QuadNode *const (&qu
   constexpr uint32_t kMask = (1u << kQuadOrdinalBits) - 1;
   for (int lvl = 0; lvl < depth; lvl += 2) {
     QuadNode n[N];
+    if (TOP_LDS && lvl < 4) {
 #pragma unroll
-    for (int i = 0; i < N; ++i) n[i] = quads[i][base + idx[i]];
+      for (int i = 0; i < N; ++i) n[i] = top[i][base + idx[i]];
+    } else {
+#pragma unroll
+      for (int i = 0; i < N; ++i) n[i] = quads[i][base + idx[i]];
+    }
     float m0[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) m0[i] = xs_j[(n[i].ords & kMask) * BT] - n[i].thr;
@@ -322,10 +333,33 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
       for (int i = 0; i < kRowIlp; ++i) { r[i].key = (t[i] * 2654435761u + uint32_t(s) * 40503u) >> 22; r[i].margin = xs_j[(t[i] & 1023) * BT]; r[i].vertex = 1; r[i].ord = 2; }
 #else
       if constexpr (QUAD) {
+        const QuadNode *all = static_cast<const QuadNode *>(vertices);
         const QuadNode *qn[kRowIlp];
 #pragma unroll
-        for (int i = 0; i < kRowIlp; ++i) qn[i] = static_cast<const QuadNode *>(vertices) + (long long)t[i] * NQ;
-        walk_quads<kRowIlp, BT>(d.depth, qn, xs_j, r);
+        for (int i = 0; i < kRowIlp; ++i) qn[i] = all + (long long)t[i] * NQ;
+        // The top of every tree is the same for all samples: the wavefront copies the first quads of its TPW trees
+        // into LDS once per step (into the space of the parked results, which nobody reads before this step's walks
+        // are over), where they fit.
+        constexpr bool kTopFits = size_t(TPW) * kTopQuads * sizeof(QuadNode) <= size_t(BT) * LDP * sizeof(Real);
+        if (kTopFits && NQ >= kTopQuads) {
+          QuadNode *stage = reinterpret_cast<QuadNode *>(p_abs);
+          for (int i = lane; i < TPW * kTopQuads; i += kWave) {
+            const int tt = i / kTopQuads, q = i - tt * kTopQuads;
+            stage[i] = all[(long long)min(tb + tt, t_end - 1) * NQ + q];
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          const QuadNode *top[kRowIlp];
+#pragma unroll
+          for (int i = 0; i < kRowIlp; ++i) top[i] = stage + (slot + i * SLOTS) * kTopQuads;
+          walk_quads<kRowIlp, BT, true>(d.depth, qn, top, xs_j, r);
+          // every lane has read its quads before any lane overwrites them with results
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+        } else {
+          walk_quads<kRowIlp, BT, false>(d.depth, qn, qn, xs_j, r);
+        }
       } else {
         const Node<Real> *all = static_cast<const Node<Real> *>(vertices);
         bool staged = false;
