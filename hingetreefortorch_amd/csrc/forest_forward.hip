@@ -3,11 +3,11 @@
 // A tiny pre-pass packs (threshold, ordinal) of every vertex into one aligned word pair (ordinals narrowed from the
 // API's int64 and clamped into range), so a walk step costs one vertex load plus one LDS gather.
 //
-// One workgroup = one tile of BT samples (all features in LDS, feature major) x a range of trees. Per pass every
-// thread walks TWO trees for its sample (interleaved, so the two dependent load chains overlap), parks
-// (|margin|, leaf) in LDS, and then the workgroup writes the pass' outputs with the lane index running along the
-// contiguous (tree, m) -- or for K > 1 the contiguous (inner position, m) -- axis of `out`, so the dominant store
-// traffic is emitted as full-width rows.
+// One workgroup = one tile of BT samples (all features in LDS, feature major) x a range of trees. Two kernels:
+//   forward_rows_kernel  (K == 1, the common case) every wavefront walks and writes on its own, see below;
+//   forward_kernel       (any K) per pass every thread walks several trees for its sample, parks (|margin|, leaf) in
+//                        LDS, and then the workgroup writes the pass' outputs with the lane index running along the
+//                        contiguous (tree, m) -- or for K > 1 the contiguous (inner position, m) -- axis of `out`.
 #include <type_traits>
 
 #include "forest_tile.hpp"
@@ -269,14 +269,8 @@ __device__ __forceinline__ void walk_quads(int depth, const QuadNode *const (&qu
   }
 }
 
-#ifndef HT_ROW_ILP
-#define HT_ROW_ILP 4
-#endif
-#ifndef HT_ROW_UNROLL
-#define HT_ROW_UNROLL 5
-#endif
-constexpr int kRowIlp = HT_ROW_ILP;        // trees walked concurrently per lane
-constexpr int kRowUnroll = HT_ROW_UNROLL;  // output vectors per lane whose weight gathers are in flight together
+constexpr int kRowIlp = 4;     // trees walked concurrently per lane
+constexpr int kRowUnroll = 5;  // output vectors per lane whose weight gathers are in flight together
 
 // One workgroup = one tile of BT samples (all features in LDS, feature major) x a range of trees, like
 // forward_kernel, but every wavefront works on its own: lanes = BT samples x 64/BT tree slots, each lane walks
@@ -329,9 +323,6 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
       int t[kRowIlp];
 #pragma unroll
       for (int i = 0; i < kRowIlp; ++i) t[i] = min(tb + slot + i * SLOTS, t_end - 1);  // surplus slots re-walk, unused
-#ifdef HT_AB_NOWALK
-      for (int i = 0; i < kRowIlp; ++i) { r[i].key = (t[i] * 2654435761u + uint32_t(s) * 40503u) >> 22; r[i].margin = xs_j[(t[i] & 1023) * BT]; r[i].vertex = 1; r[i].ord = 2; }
-#else
       if constexpr (QUAD) {
         const QuadNode *all = static_cast<const QuadNode *>(vertices);
         const QuadNode *qn[kRowIlp];
@@ -393,7 +384,6 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
           walk_many<Real, FERN, kRowIlp>(d.depth, nd, [&](int, int f) { return xs_j[f * BT]; }, r);
         }
       }
-#endif
 #pragma unroll
       for (int i = 0; i < kRowIlp; ++i) {
         p_abs[j * LDP + slot + i * SLOTS] = ht_abs(r[i].margin);
@@ -427,11 +417,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
         const int tt = div_m.div(e), m = e - tt * d.M;
         const uint32_t key = p_key[jj * LDP + tt];
         a[q] = p_abs[jj * LDP + tt];
-#ifdef HT_AB_NOGATHER
-        for (int i = 0; i < GW; ++i) wv[q][i] = Real(key + m);
-#else
         wv[q] = *reinterpret_cast<const Vec *>(wbase + (uint32_t(tt) * uint32_t(d.L) + key) * uint32_t(d.M) + m);
-#endif
         off[q] = uint32_t(jj) * TM + uint32_t(e);
       }
 #pragma unroll
@@ -440,16 +426,9 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
           Vec o;
 #pragma unroll
           for (int i = 0; i < GW; ++i) o[i] = a[q] * wv[q][i];
-#ifdef HT_AB_NOSTORE
-          if (o[0] == Real(123.456)) 
-#endif
-#ifdef HT_AB_T
-          *reinterpret_cast<Vec *>(obase + off[q]) = o;
-#else
           // streaming store: the output is written once and not read here, so it should not displace the vertices
           // and leaf weights that the gathers keep re-reading from L2 (measured: 1.45 -> 1.17 ms at the headline shape)
           __builtin_nontemporal_store(o, reinterpret_cast<Vec *>(obase + off[q]));
-#endif
         }
       }
     }
@@ -469,12 +448,8 @@ static inline size_t rows_lds_bytes(int F, int bt) {
 template <typename Real>
 static inline int pick_rows_tile(int F) {
   const int candidates[4] = {64, 32, 16, 8};
-  for (int bt : candidates) {
-#ifdef HT_ROW_MAXBT
-    if (bt > HT_ROW_MAXBT) continue;
-#endif
+  for (int bt : candidates)
     if (rows_lds_bytes<Real>(F, bt) <= size_t(kLdsBytes)) return bt;
-  }
   return 0;
 }
 
