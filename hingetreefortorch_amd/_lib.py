@@ -29,6 +29,12 @@ class ConvShape(ctypes.Structure):
                 ("dilation", ctypes.c_int64 * HT_MAX_CONV_DIMS)]
 
 
+class TileShape(ctypes.Structure):
+    _fields_ = [("planes", ctypes.c_int64), ("nd", ctypes.c_int32), ("elem_size", ctypes.c_int32),
+                ("size", ctypes.c_int64 * 3), ("tiles", ctypes.c_int64 * 3), ("window", ctypes.c_int64 * 3),
+                ("padding", ctypes.c_int64 * 3)]
+
+
 _P = ctypes.c_void_p
 _SZ = ctypes.c_size_t
 _I = ctypes.c_int
@@ -51,6 +57,8 @@ SIGNATURES = {
     "ht_conv_output_size": (_I, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int64)]),
     "ht_conv_forward": (_I, [ctypes.POINTER(ConvShape), _P, _P, _P, _P, _P, _P]),
     "ht_conv_backward": (_I, [ctypes.POINTER(ConvShape), _P, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "ht_contract": (_I, [ctypes.POINTER(TileShape), _P, _P, _P]),
+    "ht_expand": (_I, [ctypes.POINTER(TileShape), _P, _P, _P]),
     "ht_projection_workspace": (_SZ, [ctypes.c_int64]),
     "ht_projection_forward": (_I, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _P, _P, ctypes.c_double, _P, _P, _P,
                                    _P, _P, _SZ, _P]),

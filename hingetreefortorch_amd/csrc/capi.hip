@@ -287,6 +287,16 @@ static int thresholds_common(int64_t T, int64_t depth, int32_t dtype, int32_t ki
   return HT_OK;
 }
 
+int ht_contract(const ht_tile_shape *s, const void *image, void *tiles, void *stream) {
+  if (s && s->planes > 0 && (!image || !tiles)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return tile_contract(s, image, tiles, static_cast<hipStream_t>(stream));
+}
+
+int ht_expand(const ht_tile_shape *s, const void *tiles, void *image, void *stream) {
+  if (s && s->planes > 0 && (!image || !tiles)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return tile_expand(s, tiles, image, static_cast<hipStream_t>(stream));
+}
+
 size_t ht_projection_workspace(int64_t N) { return N < 0 ? 0 : projection_workspace(N); }
 
 int ht_projection_forward(int64_t B, int64_t K, int64_t N, const float *x, const float *lin, double eps, float *zhat,

@@ -110,6 +110,10 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
 
 int conv_output_size(const ht_conv_shape &s, int64_t *out_size);
 
+// Tile <-> image permutation (expand.hip).
+int tile_contract(const ht_tile_shape *s, const void *in, void *out, hipStream_t stream);
+int tile_expand(const ht_tile_shape *s, const void *in, void *out, hipStream_t stream);
+
 // Dense projection + batch normalisation in front of a forest (projection.hip), fp32.
 size_t projection_workspace(long long N);
 int projection_forward(long long B, long long K, long long N, const float *x, const float *lin, double eps,

@@ -163,3 +163,74 @@ class LinearBatchNorm(torch.autograd.Function):
         dx, dlin = _ops.linear_bn_backward(inData, ctx.needs_input_grad[0], inLinearWeights, ctx.needs_input_grad[1],
                                            zhat, rstd, g)
         return dx, dlin, None
+
+
+def contract(inData, window, padding=0):
+    """HingeTree/_HingeTree.py:32-39."""
+    if isinstance(window, int):
+        window = [window] * (inData.dim() - 2)
+    if isinstance(padding, int):
+        padding = [padding] * (inData.dim() - 2)
+    return _ops.contract(inData, window, padding)
+
+
+def expand(inData, padding=0):
+    """HingeTree/_HingeTree.py:40-44."""
+    if isinstance(padding, int):
+        padding = [padding] * ((inData.dim() - 2) // 2)
+    return _ops.expand(inData, padding)
+
+
+class _Expand(torch.autograd.Function):
+    """Tiles -> image; the gradient is the contraction of the upstream gradient (_HingeTree.py:46-59)."""
+
+    @staticmethod
+    def forward(ctx, inData, padding):
+        dim = (inData.dim() - 2) // 2
+        ctx.window = list(inData.shape[-dim:])
+        ctx.padding = padding
+        return expand(inData, padding)
+
+    @staticmethod
+    def backward(ctx, outDataGrad):
+        if ctx.needs_input_grad[0]:
+            return contract(outDataGrad.contiguous(), ctx.window, ctx.padding), None
+        return None, None
+
+
+class _Contract(torch.autograd.Function):
+    """Image -> tiles; the gradient is the expansion of the upstream gradient (_HingeTree.py:61-73)."""
+
+    @staticmethod
+    def forward(ctx, inData, window, padding=0):
+        ctx.padding = padding
+        return contract(inData, window, padding)
+
+    @staticmethod
+    def backward(ctx, outDataGrad):
+        if ctx.needs_input_grad[0]:
+            return expand(outDataGrad.contiguous(), ctx.padding), None, None
+        return None, None, None
+
+
+class Expand(torch.nn.Module):
+    """_HingeTree.py:75-81."""
+
+    def __init__(self, padding=0):
+        super().__init__()
+        self.padding = padding
+
+    def forward(self, inData):
+        return _Expand.apply(inData, self.padding)
+
+
+class Contract(torch.nn.Module):
+    """_HingeTree.py:83-90."""
+
+    def __init__(self, window, padding=0):
+        super().__init__()
+        self.window = window
+        self.padding = padding
+
+    def forward(self, inData):
+        return _Contract.apply(inData, self.window, self.padding)

@@ -97,6 +97,73 @@ def _validate_ordinals(ordinals, limit):
     _range_ok[key] = (ref, ordinals._version, bound)
 
 
+# ---- contract / expand ---------------------------------------------------------------------------------------------
+_TILE_DTYPES = (torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64, torch.float32, torch.float64)
+
+
+def _tile_call(fn_name, inData, nd, size, tiles, window, padding, out_sizes):
+    if not inData.is_cuda:
+        _runtime("Error: this build has no CPU back-end; tensors must be on a GPU.")
+    shape = L.TileShape()
+    shape.planes = int(inData.shape[0]) * int(inData.shape[1])
+    shape.nd = nd
+    shape.elem_size = inData.element_size()
+    for i in range(nd):
+        shape.size[i], shape.tiles[i], shape.window[i], shape.padding[i] = size[i], tiles[i], window[i], padding[i]
+    with torch.cuda.device(inData.device):
+        out = torch.empty(out_sizes, dtype=inData.dtype, device=inData.device)
+        L.check(getattr(L.load(), fn_name)(ctypes.byref(shape), _ptr(inData), _ptr(out), _stream(inData.device)))
+    return out
+
+
+def contract(inData, window, padding):
+    """Batched 2-d / 3-d image [B, C, *size] -> image of tiles [B, C, *tiles, *window] (expand.cpp:37-163,366-463:
+    same checks, messages and output size; positions of a tile that lie in the padding are 0)."""
+    window, padding = [int(v) for v in window], [int(v) for v in padding]
+    if len(window) == 0 or len(window) != len(padding):
+        _invalid("Error: window and padding must be non-empty and the same size.")
+    if not inData.is_contiguous():
+        _invalid("Error: All tensors are expected to be contiguous.")
+    if inData.dtype not in _TILE_DTYPES:
+        _invalid("Error: Only torch.{uint8,int8,int16,int32,int64,float32,float64} are supported.")
+    nd = len(window)
+    if nd not in (2, 3):
+        _invalid("Error: Only 2D and 3D window sizes are supported.")
+    if inData.dim() != nd + 2 or any(p < 0 for p in padding):
+        _invalid(f"Error: inData must have {nd + 2} dimensions. Padding must be non-negative.")
+    size = [int(v) for v in inData.shape[2:]]
+    if any(w < 1 or w > n + 2 * p for w, n, p in zip(window, size, padding)):
+        _invalid("Error: Window dimensions must be at least 1 but no greater than the size of the padded image.")
+    tiles = [(n + 2 * p - w) // w + 1 for w, n, p in zip(window, size, padding)]
+    return _tile_call("ht_contract", inData, nd, size, tiles, window, padding,
+                      list(inData.shape[:2]) + tiles + window)
+
+
+def expand(inData, padding):
+    """Image of tiles [B, C, *tiles, *window] -> image [B, C, *size] with size = tiles * window - (2 * padding // window)
+    * window (expand.cpp:169-330,474-570); image positions that no tile covers are 0."""
+    padding = [int(v) for v in padding]
+    if len(padding) == 0:
+        _invalid("Error: padding must be non-empty.")
+    if not inData.is_contiguous():
+        _invalid("Error: All tensors are expected to be contiguous.")
+    if inData.dtype not in _TILE_DTYPES:
+        _invalid("Error: Only torch.{uint8,int8,int16,int32,int64,float32,float64} are supported.")
+    nd = len(padding)
+    if nd not in (2, 3):
+        _invalid("Error: Only 2D and 3D padding sizes are supported.")
+    if inData.dim() != 2 * nd + 2 or any(p < 0 for p in padding):
+        _invalid(f"Error: inData must have {2 * nd + 2} dimensions. Padding must be non-negative.")
+    tiles = [int(v) for v in inData.shape[2:2 + nd]]
+    window = [int(v) for v in inData.shape[2 + nd:]]
+    if any(w < 1 for w in window):
+        _invalid("Error: The expanded size of the image must be non-empty.")
+    size = [t * w - ((2 * p) // w) * w for t, w, p in zip(tiles, window, padding)]
+    if any(n < 1 for n in size):
+        _invalid("Error: The expanded size of the image must be non-empty.")
+    return _tile_call("ht_expand", inData, nd, size, tiles, window, padding, list(inData.shape[:2]) + size)
+
+
 # ---- dense projection + batch normalisation in front of a forest ------------------------------------------------
 def linear_bn_forward(inData, inLinearWeights, eps=1e-5):
     """zhat = batch_norm(inData @ inLinearWeights.T) in training mode without affine parameters: the Linear(bias=False)
@@ -573,7 +640,7 @@ for _name in ["sparse_tree_backward", "sparse_fern_backward", "tree_init_medians
               "fern_fused_linear_backward", "sparse_fern_fused_linear_backward", "tree_fusion_forward",
               "tree_fusion_backward", "fern_fusion_forward", "fern_fusion_backward", "tree_fusion_fused_linear_forward",
               "tree_fusion_fused_linear_backward", "fern_fusion_fused_linear_forward",
-              "fern_fusion_fused_linear_backward", "contract", "expand"]:
+              "fern_fusion_fused_linear_backward"]:
     globals()[_name] = _outside(_name)
 
 __all__ = [n for n in list(globals()) if n.split("_")[0] in ("tree", "fern", "sparse", "trie", "contract", "expand", "linear")]

@@ -48,6 +48,14 @@ typedef struct ht_conv_shape {
       dilation[HT_MAX_CONV_DIMS];
 } ht_conv_shape;
 
+/* Tile <-> image permutation (contract / expand): image [planes, size...] <-> tiles [planes, tiles..., window...]. */
+typedef struct ht_tile_shape {
+  int64_t planes;    /* batch * channels */
+  int32_t nd;        /* 2 or 3 spatial dims */
+  int32_t elem_size; /* 1, 2, 4 or 8 bytes: the elements are moved, never interpreted */
+  int64_t size[3], tiles[3], window[3], padding[3];
+} ht_tile_shape;
+
 /* Message of the last failing call on this thread ("" if none). */
 const char *ht_last_error(void);
 /* ABI version of this header; bumped on any signature change. */
@@ -127,6 +135,14 @@ int ht_projection_forward(int64_t B, int64_t K, int64_t N, const float *x, const
 int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, const float *lin, const float *zhat,
                            const float *rstd, float *g, float *dlin, float *dx, void *workspace,
                            size_t workspace_bytes, void *stream);
+
+/* ---- contract / expand -----------------------------------------------------------------------------------------------
+ * Replace contract2d/3d and expand2d/3d of the reference (expand.cpp:37-227 on the CPU, expand_gpu.cu:110-172 on the
+ * GPU; exported as `contract` / `expand`, hingetree.cpp:2029-2030). Tile j of a dimension covers image positions
+ * [j * window - padding, j * window - padding + window); what lies outside the image (contract) or is covered by no
+ * tile (expand) is 0. Every element of `out` is written. */
+int ht_contract(const ht_tile_shape *s, const void *image, void *tiles, void *stream);
+int ht_expand(const ht_tile_shape *s, const void *tiles, void *image, void *stream);
 
 /* Host-side (CPU pointers) threshold consistency, in place for _fix. One flag byte per tree is written to `flags`
  * (check: 1 = consistent; fix: 1 = changed). Ferns are always consistent and never change.

@@ -199,3 +199,46 @@ def conv_backward(x, thr, ord_, w, gout, kernel, stride, padding, dilation, need
     if rc != 0:
         raise ValueError("invalid convolution geometry")
     return dx, dthr, dw
+
+
+def contract(x, window, padding):
+    """Image [B, C, *size] -> tiles [B, C, *tiles, *window]; restates contract2d_cpu / contract3d_cpu
+    (expand.cpp:37-163): tile j of a dimension covers [j * w - p, j * w - p + w), the part outside the image stays 0."""
+    nd = len(window)
+    size = list(x.shape[2:])
+    tiles = [(n + 2 * p - w) // w + 1 for n, w, p in zip(size, window, padding)]
+    out = torch.zeros(list(x.shape[:2]) + tiles + list(window), dtype=x.dtype)
+    import itertools
+    for j in itertools.product(*[range(t) for t in tiles]):
+        src, dst = [slice(None), slice(None)], [slice(None), slice(None)] + list(j)
+        empty = False
+        for d in range(nd):
+            b = j[d] * window[d] - padding[d]
+            lo, hi = max(0, b), min(size[d], b + window[d])
+            empty = empty or lo >= hi
+            src.append(slice(lo, hi))
+            dst.append(slice(lo - b, hi - b))
+        if not empty:
+            out[tuple(dst)] = x[tuple(src)]
+    return out
+
+
+def expand(x, padding):
+    """Tiles [B, C, *tiles, *window] -> image [B, C, *size]; restates expand2d_cpu / expand3d_cpu (expand.cpp:169-330)."""
+    nd = len(padding)
+    tiles, window = list(x.shape[2:2 + nd]), list(x.shape[2 + nd:])
+    size = [t * w - ((2 * p) // w) * w for t, w, p in zip(tiles, window, padding)]
+    out = torch.zeros(list(x.shape[:2]) + size, dtype=x.dtype)
+    import itertools
+    for j in itertools.product(*[range(t) for t in tiles]):
+        dst, src = [slice(None), slice(None)], [slice(None), slice(None)] + list(j)
+        empty = False
+        for d in range(nd):
+            b = j[d] * window[d] - padding[d]
+            lo, hi = max(0, b), min(size[d], b + window[d])
+            empty = empty or lo >= hi
+            dst.append(slice(lo, hi))
+            src.append(slice(lo - b, hi - b))
+        if not empty:
+            out[tuple(dst)] = x[tuple(src)]
+    return out

@@ -1,7 +1,8 @@
 """Writes tests/golden/*.npz from the reference's own CPU build (oracle/_ref/hingetree_cpp.so, made by
 `make -C oracle ref` from the sources under /root/reference). Run in the authoring container only:
 
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py            # everything
+    python tests/golden/make_golden.py tiles      # only the contract / expand fixtures
 
 Each file holds seeded inputs and the reference's outputs for one small case; tests compare the oracle (CPU) and the
 HIP path (GPU) against them. The fixtures are data only.
@@ -37,11 +38,33 @@ CONV_CASES = {
     "conv3d_fern": (1, 2, 2, [5, 4, 6], 3, [2], [2, 2, 3], [1, 2, 1], [0, 1, 1], [1, 1, 1], True, torch.float32),
 }
 
+TILE_CASES = {
+    # name: (shape, window, padding, dtype)
+    "tiles2d_f32": ([2, 3, 9, 11], [4, 3], [1, 2], torch.float32),
+    "tiles2d_u8_exact": ([1, 2, 8, 12], [2, 4], [0, 0], torch.uint8),
+    "tiles3d_i16": ([2, 1, 5, 6, 7], [2, 3, 2], [1, 0, 1], torch.int16),
+    "tiles3d_f64_big_pad": ([1, 2, 4, 5, 3], [3, 2, 2], [2, 1, 2], torch.float64),
+}
+
+
+def write_tiles(ref):
+    for name, (shape, window, padding, dtype) in TILE_CASES.items():
+        g = torch.Generator().manual_seed(23)
+        x = (200.0 * torch.rand(shape, generator=g) - 50.0).to(dtype)
+        tiles = ref.contract(x, window, padding)
+        image = ref.expand(tiles, padding)
+        np.savez_compressed(os.path.join(HERE, name + ".npz"), x=x.numpy(), window=np.array(window),
+                            padding=np.array(padding), tiles=tiles.numpy(), image=image.numpy())
+
 
 def main():
     ref = ho.reference_module()
     if ref is None:
         raise SystemExit("oracle/_ref/hingetree_cpp.so is missing: run `make -C oracle ref` first")
+    write_tiles(ref)
+    if sys.argv[1:] == ["tiles"]:
+        print("wrote", sorted(f for f in os.listdir(HERE) if f.startswith("tiles")))
+        return
     for name, (B, F, Kd, T, D, Md, fern, dtype, dist) in FOREST_CASES.items():
         x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype, seed=11, x_dist=dist)
         pre = "fern_" if fern else "tree_"

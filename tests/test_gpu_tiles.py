@@ -1,0 +1,86 @@
+"""GPU parity of contract / expand against the CPU oracle (bit-exact: pure data movement), for every dtype the
+reference accepts, the golden fixtures written from the reference's own build, the autograd pair and the modules."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT
+from oracle import hinge_oracle as ho
+import hingetree_cpp as ops
+from HingeTree import Contract, Expand, contract, expand
+
+pytestmark = pytest.mark.gpu
+
+CASES = [([2, 3, 8, 12], [2, 3], [0, 0]), ([1, 2, 7, 9], [3, 2], [1, 2]), ([2, 1, 5, 6, 7], [2, 3, 2], [1, 0, 1]),
+         ([1, 1, 4, 4], [4, 4], [2, 2]), ([1, 2, 9, 9], [4, 5], [3, 1]), ([1, 1, 3, 10, 4], [3, 4, 1], [0, 3, 2]),
+         ([3, 5, 64, 48], [8, 8], [0, 0])]
+DTYPES = [torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64, torch.float32, torch.float64]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=[str(d).split(".")[1] for d in DTYPES])
+@pytest.mark.parametrize("case", CASES, ids=[f"t{i}" for i in range(len(CASES))])
+def test_contract_expand_bit_exact(dev, case, dtype):
+    shape, window, padding = case
+    x = (100.0 * torch.rand(shape, generator=torch.Generator().manual_seed(1))).to(dtype)
+    want_t = ho.contract(x, window, padding)
+    got_t = ops.contract(x.to(dev), window, padding)
+    assert got_t.shape == want_t.shape and got_t.dtype == dtype and torch.equal(got_t.cpu(), want_t)
+    want_i = ho.expand(want_t, padding)
+    got_i = ops.expand(got_t, padding)
+    assert got_i.shape == want_i.shape and torch.equal(got_i.cpu(), want_i)
+
+
+GOLD = sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "tiles*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLD, ids=[os.path.basename(p)[:-4] for p in GOLD])
+def test_tiles_golden(dev, path):
+    z = np.load(path)
+    x = torch.from_numpy(z["x"]).to(dev)
+    window, padding = z["window"].tolist(), z["padding"].tolist()
+    tiles = ops.contract(x, window, padding)
+    assert torch.equal(tiles.cpu(), torch.from_numpy(z["tiles"]))
+    assert torch.equal(ops.expand(tiles, padding).cpu(), torch.from_numpy(z["image"]))
+
+
+def test_tile_errors(dev):
+    x = torch.zeros([1, 1, 4, 4], device=dev)
+    with pytest.raises(ValueError, match="non-empty and the same size"):
+        ops.contract(x, [2, 2], [0])
+    with pytest.raises(ValueError, match="Only 2D and 3D window"):
+        ops.contract(x, [2], [0])
+    with pytest.raises(ValueError, match="no greater than the size of the padded image"):
+        ops.contract(x, [5, 2], [0, 0])
+    with pytest.raises(ValueError, match="must have 4 dimensions"):
+        ops.contract(torch.zeros([1, 1, 4, 4, 4], device=dev), [2, 2], [0, 0])
+    with pytest.raises(ValueError, match="contiguous"):
+        ops.contract(x.transpose(2, 3)[:, :, :, ::2], [2, 2], [0, 0])
+    with pytest.raises(ValueError, match="are supported"):
+        ops.contract(x.half(), [2, 2], [0, 0])
+    with pytest.raises(ValueError, match="padding must be non-empty"):
+        ops.expand(torch.zeros([1, 1, 2, 2, 2, 2], device=dev), [])
+    with pytest.raises(ValueError, match="must have 6 dimensions"):
+        ops.expand(x, [0, 0])
+    with pytest.raises(ValueError, match="expanded size of the image must be non-empty"):
+        ops.expand(torch.zeros([1, 1, 1, 1, 2, 2], device=dev), [1, 1])
+
+
+def test_tile_autograd_and_modules(dev):
+    x = torch.randn([2, 3, 8, 8], device=dev, dtype=torch.float64, requires_grad=True)
+    t = Contract([4, 4], padding=2)(x)
+    assert t.shape == (2, 3, 3, 3, 4, 4)
+    u = torch.randn_like(t)
+    (t * u).sum().backward()
+    assert torch.equal(x.grad, expand(u, 2))                    # d<contract(x), u>/dx = expand(u)
+    v = t.detach().clone().requires_grad_(True)
+    img = Expand(padding=2)(v)
+    assert torch.equal(img, x.detach())
+    g = torch.randn_like(img)
+    (img * g).sum().backward()
+    assert torch.equal(v.grad, contract(g, [4, 4], 2))
+    # the segmentation models' use: extra_outputs = [8, 8] tiles expanded back to an image
+    tiles = torch.randn([2, 5, 4, 6, 8, 8], device=dev)
+    assert Expand()(tiles).shape == (2, 5, 32, 48)

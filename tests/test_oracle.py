@@ -259,3 +259,65 @@ def test_fix_then_check_random():
     t2 = 6 * torch.rand([3, 63], generator=g, dtype=torch.float64) - 3
     keep = t2.clone()
     assert not any(ho.fix_thresholds(t2, distinct, w[:3])) and torch.equal(t2, keep)
+
+
+# ---- contract / expand ---------------------------------------------------------------------------------------------
+TILE_FILES = sorted(glob.glob(os.path.join(GOLDEN, "tiles*.npz")))
+
+
+@pytest.mark.parametrize("path", TILE_FILES, ids=[os.path.basename(p)[:-4] for p in TILE_FILES])
+def test_golden_tiles(path):
+    z = np.load(path)
+    x, window, padding = _t(z["x"]), z["window"].tolist(), z["padding"].tolist()
+    tiles = ho.contract(x, window, padding)
+    assert tiles.shape == z["tiles"].shape and torch.equal(tiles, _t(z["tiles"]))
+    image = ho.expand(tiles, padding)
+    assert image.shape == z["image"].shape and torch.equal(image, _t(z["image"]))
+
+
+@pytest.mark.skipif(ho.reference_module() is None, reason="reference build (oracle/_ref) not present")
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64, torch.float32,
+                                   torch.float64])
+def test_tiles_against_reference_build(dtype):
+    ref = ho.reference_module()
+    g = torch.Generator().manual_seed(9)
+    for shape, window, padding in [([2, 3, 8, 12], [2, 3], [0, 0]), ([1, 2, 7, 9], [3, 2], [1, 2]),
+                                   ([2, 1, 5, 6, 7], [2, 3, 2], [1, 0, 1]), ([1, 1, 4, 4], [4, 4], [2, 2]),
+                                   ([1, 2, 9, 9], [4, 5], [3, 1]), ([1, 1, 3, 10, 4], [3, 4, 1], [0, 3, 2])]:
+        x = (100.0 * torch.rand(shape, generator=g)).to(dtype)
+        a, b = ho.contract(x, window, padding), ref.contract(x, window, padding)
+        assert a.shape == b.shape and torch.equal(a, b)
+        c, d = ho.expand(a, padding), ref.expand(b, padding)
+        assert c.shape == d.shape and torch.equal(c, d)
+
+
+def test_tiles_are_a_reshape_when_they_fit():
+    """No padding and sizes that are multiples of the window: contraction is a reshape + permute, expansion undoes it."""
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn([2, 3, 6, 8], generator=g)
+    t = ho.contract(x, [3, 2], [0, 0])
+    assert torch.equal(t, x.reshape(2, 3, 2, 3, 4, 2).permute(0, 1, 2, 4, 3, 5))
+    assert torch.equal(ho.expand(t, [0, 0]), x)
+    v = torch.randn([1, 2, 4, 6, 4], generator=g)
+    t3 = ho.contract(v, [2, 3, 2], [0, 0, 0])
+    assert torch.equal(t3, v.reshape(1, 2, 2, 2, 2, 3, 2, 2).permute(0, 1, 2, 4, 6, 3, 5, 7))
+    assert torch.equal(ho.expand(t3, [0, 0, 0]), v)
+
+
+def test_tiles_padding_reads_zero_and_adjoint():
+    """Padded positions are 0; where the expanded size equals the image size, expand is the adjoint of contract:
+    <contract(x), t> == <x, expand(t)> (the autograd rule of the reference relies on exactly this,
+    _HingeTree.py:46-73)."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn([1, 2, 8, 8], generator=g, dtype=torch.float64)
+    window, padding = [4, 4], [2, 2]
+    t = ho.contract(x, window, padding)
+    assert t.shape == (1, 2, 3, 3, 4, 4)                      # (8 + 4 - 4) // 4 + 1 tiles per dimension
+    assert torch.all(t[:, :, 0, :, :2, :] == 0) and torch.all(t[:, :, :, 0, :, :2] == 0)      # rows / columns -2, -1
+    assert torch.all(t[:, :, 2, :, 2:, :] == 0) and torch.all(t[:, :, :, 2, :, 2:] == 0)      # rows / columns 8, 9
+    assert torch.equal(t[:, :, 1, 1], x[:, :, 2:6, 2:6])
+    u = torch.randn(t.shape, generator=g, dtype=torch.float64)
+    e = ho.expand(u, padding)
+    assert e.shape == x.shape                                 # 3 * 4 - (4 // 4) * 4
+    assert abs(float((t * u).sum() - (x * e).sum())) < 1e-9
+    assert torch.equal(ho.expand(t, padding), x)              # every pixel is covered by exactly one tile
