@@ -10,6 +10,8 @@ from hingetreefortorch_amd.functions import (  # noqa: F401
     HingeFernConv2d,
     HingeFernConv3d,
     LinearBatchNorm,
+    HingeTreeFusedLinear,
+    HingeFernFusedLinear,
     Contract,
     Expand,
     contract,

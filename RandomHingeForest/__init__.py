@@ -10,4 +10,6 @@ from hingetreefortorch_amd.modules import (  # noqa: F401
     HingeFernConv2d,
     HingeFernConv3d,
     LinearHingeForest,
+    RandomHingeForestFusedLinear,
+    RandomHingeFernFusedLinear,
 )

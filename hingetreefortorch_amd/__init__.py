@@ -15,6 +15,8 @@ from .modules import (  # noqa: F401
     HingeTreeConv2d,
     HingeTreeConv3d,
     LinearHingeForest,
+    RandomHingeFernFusedLinear,
+    RandomHingeForestFusedLinear,
     RandomHingeFern,
     RandomHingeForest,
 )

@@ -287,6 +287,20 @@ static int thresholds_common(int64_t T, int64_t depth, int32_t dtype, int32_t ki
   return HT_OK;
 }
 
+int ht_tree_mix_forward(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin,
+                        const float *bias, float *out, void *stream) {
+  if (B < 0 || T < 0 || O < 0 || R < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if (B * O * R > 0 && (!out || (T > 0 && (!f || !lin)))) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return mix_forward(B, T, O, R, f, lin, bias, out, static_cast<hipStream_t>(stream));
+}
+
+int ht_tree_mix_backward(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin, const float *g,
+                         float *h, float *dlin, void *stream) {
+  if (B < 0 || T < 0 || O < 0 || R < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if (B * O * R > 0 && (!g || (h && !lin) || (dlin && !f))) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return mix_backward(B, T, O, R, f, lin, g, h, dlin, static_cast<hipStream_t>(stream));
+}
+
 int ht_contract(const ht_tile_shape *s, const void *image, void *tiles, void *stream) {
   if (s && s->planes > 0 && (!image || !tiles)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
   return tile_contract(s, image, tiles, static_cast<hipStream_t>(stream));

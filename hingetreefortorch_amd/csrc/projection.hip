@@ -85,20 +85,38 @@ __device__ __forceinline__ void stash_tile(float *tile, const Fetch &f) {
   }
 }
 
-// C[i, j] = sum_r A(i, r) * B(j, r), i < n_i, j < n_j, r < n_r; C row-major with leading dimension ldc.
+// C[i, j] = sum_r A(i, r) * B(j, r) (+ bias_i[i] + bias_j[j]), i < n_i, j < n_j, r < n_r; C row-major with leading
+// dimension ldc. A launch covers `batches` such problems whose operands lie stride_a / stride_b / stride_c elements
+// apart: either one result per batch (blockIdx.z), or -- SUM_BATCHES -- one result summed over all of them (the
+// batch index then simply extends the reduction).
 // STATS: also accumulate per column j the sum and the sum of squares of C over i into stats[j], stats[n_j + j] (fp64
 // atomics; the batch statistics of the projection).
-template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS>
-__global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const float *__restrict__ A, long long lda,
-                                                            const float *__restrict__ B, long long ldb,
-                                                            float *__restrict__ C, long long ldc, int n_i, int n_j,
-                                                            int n_r, bool vec_a, bool vec_b, double *stats) {
+struct GemmArgs {
+  const float *A, *B;
+  float *C;
+  long long lda, ldb, ldc, stride_a, stride_b, stride_c;
+  int n_i, n_j, n_r, batches;
+  bool vec_a, vec_b;
+  double *stats;
+  const float *bias_i, *bias_j;
+};
+
+template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS, bool SUM_BATCHES>
+__global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
   __shared__ float As[2][kRed * kPitch];
   __shared__ float Bs[2][kRed * kPitch];
+  const int n_i = g.n_i, n_j = g.n_j, n_r = g.n_r;
   const int i0 = blockIdx.y * kTile, j0 = blockIdx.x * kTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wavefront's 64 x 64 corner
   const int lr = lane & 31, lk = lane >> 5;
+  const float *A = g.A, *B = g.B;
+  float *C = g.C;
+  if (!SUM_BATCHES) {
+    A += (long long)blockIdx.z * g.stride_a;
+    B += (long long)blockIdx.z * g.stride_b;
+    C += (long long)blockIdx.z * g.stride_c;
+  }
 
   Acc16 acc[2][2];
 #pragma unroll
@@ -108,19 +126,24 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const float *__restr
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
+  const int per_batch = (n_r + kRed - 1) / kRed;
+  const int steps = SUM_BATCHES ? per_batch * g.batches : per_batch;
+  auto fetch = [&](Fetch &fa, Fetch &fb, int s) {
+    const int z = SUM_BATCHES ? s / per_batch : 0;
+    const int r0 = (s - z * per_batch) * kRed;
+    fetch_tile<A_RED_CONTIG>(fa, A + (long long)z * g.stride_a, g.lda, i0, n_i, r0, n_r, g.vec_a);
+    fetch_tile<B_RED_CONTIG>(fb, B + (long long)z * g.stride_b, g.ldb, j0, n_j, r0, n_r, g.vec_b);
+  };
   Fetch fa, fb;
-  fetch_tile<A_RED_CONTIG>(fa, A, lda, i0, n_i, 0, n_r, vec_a);
-  fetch_tile<B_RED_CONTIG>(fb, B, ldb, j0, n_j, 0, n_r, vec_b);
-  stash_tile<A_RED_CONTIG>(As[0], fa);
-  stash_tile<B_RED_CONTIG>(Bs[0], fb);
+  if (steps > 0) {
+    fetch(fa, fb, 0);
+    stash_tile<A_RED_CONTIG>(As[0], fa);
+    stash_tile<B_RED_CONTIG>(Bs[0], fb);
+  }
   __syncthreads();
-  const int steps = (n_r + kRed - 1) / kRed;
   for (int s = 0; s < steps; ++s) {
     const int cur = s & 1;
-    if (s + 1 < steps) {
-      fetch_tile<A_RED_CONTIG>(fa, A, lda, i0, n_i, (s + 1) * kRed, n_r, vec_a);
-      fetch_tile<B_RED_CONTIG>(fb, B, ldb, j0, n_j, (s + 1) * kRed, n_r, vec_b);
-    }
+    if (s + 1 < steps) fetch(fa, fb, s + 1);
     const float *as = As[cur], *bs = Bs[cur];
 #pragma unroll
     for (int kk = 0; kk < kRed; kk += 2) {
@@ -142,15 +165,18 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const float *__restr
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
     const int j = j0 + wj + 32 * b + lr;
+    const float bj = (g.bias_j && j < n_j) ? g.bias_j[j] : 0.f;
     double s1 = 0.0, s2 = 0.0;
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int i = i0 + wi + 32 * a + 8 * (e / 4) + 4 * lk + (e % 4);
-        const float v = acc[a][b][e];
         if (i < n_i && j < n_j) {
-          C[(long long)i * ldc + j] = v;
+          float v = acc[a][b][e];
+          if (g.bias_i) v += g.bias_i[i];
+          v += bj;
+          C[(long long)i * g.ldc + j] = v;
           if (STATS) {
             s1 += double(v);
             s2 += double(v) * double(v);
@@ -162,8 +188,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const float *__restr
       s1 += __shfl_xor(s1, 32, 64);
       s2 += __shfl_xor(s2, 32, 64);
       if (lk == 0 && j < n_j) {
-        atomicAdd(stats + j, s1);
-        atomicAdd(stats + n_j + j, s2);
+        atomicAdd(g.stats + j, s1);
+        atomicAdd(g.stats + n_j + j, s2);
       }
     }
   }
@@ -278,19 +304,40 @@ __global__ __launch_bounds__(256) void bn_backward_apply_kernel(float *g, const 
   }
 }
 
-bool aligned16(const void *p, long long ld) { return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0; }
+bool aligned16(const void *p, long long ld, long long stride) {
+  return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0 && stride % 4 == 0;
+}
+
+template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS, bool SUM_BATCHES>
+int launch_gemm_batched(const float *A, long long lda, long long stride_a, const float *B, long long ldb,
+                        long long stride_b, float *C, long long ldc, long long stride_c, long long n_i, long long n_j,
+                        long long n_r, long long batches, double *stats, const float *bias_i, const float *bias_j,
+                        hipStream_t stream) {
+  if (n_i <= 0 || n_j <= 0 || batches <= 0) return HT_OK;
+  const long long gi = (n_i + kTile - 1) / kTile, gj = (n_j + kTile - 1) / kTile;
+  const long long per_batch = (n_r + kRed - 1) / kRed;
+  if (gi > 65535 || gj > 0x7fffffffLL || n_r > 0x7fffffffLL || n_i > 0x7fffffffLL || n_j > 0x7fffffffLL ||
+      batches > 0x7fffffffLL || (!SUM_BATCHES && batches > 65535) || per_batch * batches > 0x7fffffffLL)
+    return fail(HT_ERR_RUNTIME, "Error: matrix product too large for this build.");
+  GemmArgs g;
+  g.A = A, g.B = B, g.C = C;
+  g.lda = lda, g.ldb = ldb, g.ldc = ldc;
+  g.stride_a = stride_a, g.stride_b = stride_b, g.stride_c = stride_c;
+  g.n_i = int(n_i), g.n_j = int(n_j), g.n_r = int(n_r), g.batches = int(batches);
+  g.vec_a = aligned16(A, lda, stride_a), g.vec_b = aligned16(B, ldb, stride_b);
+  g.stats = stats, g.bias_i = bias_i, g.bias_j = bias_j;
+  hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES>),
+                     dim3((unsigned)gj, (unsigned)gi, (unsigned)(SUM_BATCHES ? 1 : batches)), dim3(kGemmThreads), 0,
+                     stream, g);
+  HT_LAUNCH_CHECK("matrix product (matrix cores)");
+  return HT_OK;
+}
 
 template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS>
 int launch_gemm(const float *A, long long lda, const float *B, long long ldb, float *C, long long ldc, long long n_i,
                 long long n_j, long long n_r, double *stats, hipStream_t stream) {
-  if (n_i <= 0 || n_j <= 0) return HT_OK;
-  const long long gi = (n_i + kTile - 1) / kTile, gj = (n_j + kTile - 1) / kTile;
-  if (gi > 65535 || gj > 0x7fffffffLL || n_r > 0x7fffffffLL || n_i > 0x7fffffffLL || n_j > 0x7fffffffLL)
-    return fail(HT_ERR_RUNTIME, "Error: projection too large for this build.");
-  hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS>), dim3((unsigned)gj, (unsigned)gi), dim3(kGemmThreads), 0, stream,
-                     A, lda, B, ldb, C, ldc, int(n_i), int(n_j), int(n_r), aligned16(A, lda), aligned16(B, ldb), stats);
-  HT_LAUNCH_CHECK("projection (matrix cores)");
-  return HT_OK;
+  return launch_gemm_batched<A_RED_CONTIG, B_RED_CONTIG, STATS, false>(A, lda, 0, B, ldb, 0, C, ldc, 0, n_i, n_j, n_r, 1,
+                                                                        stats, nullptr, nullptr, stream);
 }
 
 long long rows_grid(long long B) { return B < 64 ? (B < 1 ? 1 : B) : 64; }
@@ -336,6 +383,45 @@ int projection_backward(long long B, long long K, long long N, const float *x, c
   if (dlin && (rc = launch_gemm<false, false, false>(g, N, x, K, dlin, K, N, K, B, nullptr, stream)) != HT_OK) return rc;
   // dx[b, k] = sum_n g[b, n] * lin[n, k]: g has the reduction index n contiguous, lin the row index k
   if (dx && (rc = launch_gemm<true, false, false>(g, N, lin, K, dx, K, B, K, N, nullptr, stream)) != HT_OK) return rc;
+  return HT_OK;
+}
+
+// Linear mix over the tree axis behind a forest (the reference's "fused linear" operators,
+// hingetree_fused_linear.cpp:75-412): f [B, T, R] are forest outputs (R = inner data positions x outputs per leaf).
+//   forward : out[b, o, r] = bias[o] + sum_t lin[o, t] * f[b, t, r]
+//   backward: h[b, t, r] = sum_o lin[o, t] * g[b, o, r]   (the upstream gradient of the forest)
+//             dlin[o, t] = sum_{b, r} g[b, o, r] * f[b, t, r]
+int mix_forward(long long B, long long T, long long O, long long R, const float *f, const float *lin,
+                const float *bias, float *out, hipStream_t stream) {
+  if (R == 1)  // out [B x O] = f [B x T] * lin [O x T]^T, bias per column
+    return launch_gemm_batched<true, true, false, false>(f, T, 0, lin, T, 0, out, O, 0, B, O, T, 1, nullptr, nullptr, bias,
+                                                         stream);
+  // per sample: out_b [O x R] = lin [O x T] * f_b [T x R], bias per row
+  return launch_gemm_batched<true, false, false, false>(lin, T, 0, f, R, T * R, out, R, O * R, O, R, T, B, nullptr, bias,
+                                                        nullptr, stream);
+}
+
+int mix_backward(long long B, long long T, long long O, long long R, const float *f, const float *lin, const float *g,
+                 float *h, float *dlin, hipStream_t stream) {
+  int rc;
+  if (h) {
+    if (R == 1)  // h [B x T] = g [B x O] * lin [O x T]
+      rc = launch_gemm_batched<true, false, false, false>(g, O, 0, lin, T, 0, h, T, 0, B, T, O, 1, nullptr, nullptr,
+                                                          nullptr, stream);
+    else  // per sample: h_b [T x R] = lin^T [T x O] * g_b [O x R]
+      rc = launch_gemm_batched<false, false, false, false>(lin, T, 0, g, R, O * R, h, R, T * R, T, R, O, B, nullptr,
+                                                           nullptr, nullptr, stream);
+    if (rc != HT_OK) return rc;
+  }
+  if (dlin) {
+    if (R == 1)  // dlin [O x T] = g^T [O x B] * f [B x T]
+      rc = launch_gemm_batched<false, false, false, false>(g, O, 0, f, T, 0, dlin, T, 0, O, T, B, 1, nullptr, nullptr,
+                                                           nullptr, stream);
+    else  // dlin [O x T] = sum_b g_b [O x R] * f_b [T x R]^T
+      rc = launch_gemm_batched<true, true, false, true>(g, R, O * R, f, R, T * R, dlin, T, 0, O, T, R, B, nullptr,
+                                                        nullptr, nullptr, stream);
+    if (rc != HT_OK) return rc;
+  }
   return HT_OK;
 }
 

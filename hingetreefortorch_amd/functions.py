@@ -143,6 +143,53 @@ HingeFernConv2d = _conv_function("HingeFernConv2d", "fern", 2, "fern")
 HingeFernConv3d = _conv_function("HingeFernConv3d", "fern", 3, "fern")
 
 
+class _FusedLinearFunction(torch.autograd.Function):
+    """forward(ctx, inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias) =
+    inLinearBias + inLinearWeights @ forest(inData) over the tree axis (_HingeTree.py:218-258). Unlike the reference,
+    whose GPU forward accumulates with atomics and therefore refuses to run under
+    torch.use_deterministic_algorithms(True), this one is deterministic and selects the deterministic forest backward
+    under that switch."""
+    _prefix = None
+
+    @staticmethod
+    def _forward(cls, ctx, inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias):
+        ctx.save_for_backward(inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias)
+        return getattr(_ops, f"{cls._prefix}_fused_linear_forward")(inData, inThresholds, inOrdinals, inWeights,
+                                                                   inLinearWeights, inLinearBias)
+
+    @staticmethod
+    def _backward(cls, ctx, outDataGrad):
+        inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        name = f"{cls._prefix}_fused_linear_backward" + ("_deterministic" if _is_deterministic() else "")
+        return tuple(getattr(_ops, name)(inData, need[0], inThresholds, need[1], inOrdinals, need[2], inWeights, need[3],
+                                         inLinearWeights, need[4], inLinearBias, need[5], outDataGrad.contiguous()))
+
+
+class HingeTreeFusedLinear(_FusedLinearFunction):
+    _prefix = "tree"
+
+    @staticmethod
+    def forward(ctx, *args):
+        return _FusedLinearFunction._forward(HingeTreeFusedLinear, ctx, *args)
+
+    @staticmethod
+    def backward(ctx, outDataGrad):
+        return _FusedLinearFunction._backward(HingeTreeFusedLinear, ctx, outDataGrad)
+
+
+class HingeFernFusedLinear(_FusedLinearFunction):
+    _prefix = "fern"
+
+    @staticmethod
+    def forward(ctx, *args):
+        return _FusedLinearFunction._forward(HingeFernFusedLinear, ctx, *args)
+
+    @staticmethod
+    def backward(ctx, outDataGrad):
+        return _FusedLinearFunction._backward(HingeFernFusedLinear, ctx, outDataGrad)
+
+
 class LinearBatchNorm(torch.autograd.Function):
     """zhat = BatchNorm1d(affine=False, training)(Linear(bias=False)(x)) as one operator on the HIP library: the dense
     front of the reference's README model (README.md:117-129). forward(ctx, inData, inLinearWeights, eps) returns

@@ -97,6 +97,99 @@ def _validate_ordinals(ordinals, limit):
     _range_ok[key] = (ref, ordinals._version, bound)
 
 
+# ---- forest -> linear ("fused linear") ------------------------------------------------------------------------------
+def _fused_linear_checks(inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias, outDataGrad=None):
+    """Checks and messages of hingetree_fused_linear.cpp:79-109,206-245 (after the dispatcher's dtype / device /
+    contiguity checks)."""
+    reals = [inData, inThresholds, inWeights, inLinearWeights, inLinearBias] + ([] if outDataGrad is None else [outDataGrad])
+    _common_checks(reals, inOrdinals, outDataGrad is not None)
+    if inData.dim() < 2 or inThresholds.dim() != 2 or inOrdinals.dim() != 2 or inWeights.dim() < 2 or \
+            inLinearWeights.dim() != 2 or inLinearBias.dim() != 1 or (outDataGrad is not None and outDataGrad.dim() < 2):
+        _invalid("Error: inData, inWeights must have at least 2 dimensions. inThresholds, inOrdinals, inLinearWeights "
+                 "must have 2 dimensions. inLinearBias must have 1 dimension.")
+    if inThresholds.shape != inOrdinals.shape or inWeights.shape[0] != inThresholds.shape[0] or \
+            inWeights.shape[0] != inLinearWeights.shape[1] or inLinearWeights.shape[0] != inLinearBias.shape[0]:
+        _invalid("Error: inThresholds and inOrdinals must be the same shape. inWeights.shape[0] must be the same as "
+                 "inThresholds.shape[0]. inLinearWeightrs.shape[0] must be the same as inLinearBias.shape[0].")
+    if inData.dtype != torch.float32:
+        _runtime("Error: the forest -> linear operators of this build support torch.float32 only.")
+
+
+def _mix_sizes(inData, inWeights, inLinearWeights):
+    B, T, O = int(inData.shape[0]), int(inWeights.shape[0]), int(inLinearWeights.shape[0])
+    R = _prod(inData.shape[2:]) * _prod(inWeights.shape[2:])
+    return B, T, O, R, [B, O] + list(inData.shape[2:]) + list(inWeights.shape[2:])
+
+
+def _fused_linear_forward(kind, inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias):
+    """out[b, o, ...] = inLinearBias[o] + sum_t inLinearWeights[o, t] * forest(inData)[b, t, ...]
+    (hingetree_fused_linear.cpp:75-198): the forest kernel followed by a matrix-core product over the tree axis."""
+    _fused_linear_checks(inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias)
+    f = _forward(kind, inData, inThresholds, inOrdinals, inWeights)
+    B, T, O, R, out_sizes = _mix_sizes(inData, inWeights, inLinearWeights)
+    with torch.cuda.device(inData.device):
+        out = torch.empty(out_sizes, dtype=inData.dtype, device=inData.device)
+        L.check(L.load().ht_tree_mix_forward(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(inLinearBias), _ptr(out),
+                                             _stream(inData.device)))
+    return out
+
+
+def _fused_linear_backward(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals,
+                           bInOrdinalsGrad, inWeights, bInWeightsGrad, inLinearWeights, bInLinearWeightsGrad,
+                           inLinearBias, bInLinearBiasGrad, outDataGrad):
+    """[dData, dThresholds, None, dWeights, dLinearWeights, dLinearBias] (hingetree_fused_linear.cpp:200-412)."""
+    if bInOrdinalsGrad:
+        _runtime("Error: Gradient on inOrdinals is requested, but inOrdinals never has a gradient.")
+    _fused_linear_checks(inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias, outDataGrad)
+    B, T, O, R, out_sizes = _mix_sizes(inData, inWeights, inLinearWeights)
+    if list(outDataGrad.shape) != out_sizes:
+        _invalid(f"Error: outDataGrad.shape does not match the expected shape ({list(outDataGrad.shape)} != {out_sizes}).")
+    grads = [None] * 6
+    need_forest = bInDataGrad or bInThresholdsGrad or bInWeightsGrad
+    lib = L.load()
+    with torch.cuda.device(inData.device):
+        f = _forward(kind, inData, inThresholds, inOrdinals, inWeights) if bInLinearWeightsGrad else None
+        h = torch.empty([B, T] + list(inData.shape[2:]) + list(inWeights.shape[2:]), dtype=inData.dtype,
+                        device=inData.device) if need_forest else None
+        dlin = torch.empty_like(inLinearWeights) if bInLinearWeightsGrad else None
+        if h is not None or dlin is not None:
+            L.check(lib.ht_tree_mix_backward(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(outDataGrad), _ptr(h),
+                                             _ptr(dlin), _stream(inData.device)))
+        grads[4] = dlin
+        if need_forest:
+            grads[0], grads[1], _, grads[3] = _backward(kind, mode, inData, bInDataGrad, inThresholds,
+                                                        bInThresholdsGrad, inOrdinals, False, inWeights, bInWeightsGrad, h)
+        if bInLinearBiasGrad:  # a plain sum, like the reference's outDataGrad.sum(...) (hingetree_fused_linear.cpp:388)
+            grads[5] = outDataGrad.sum(dim=[0] + list(range(2, outDataGrad.dim())))
+    return grads
+
+
+def tree_fused_linear_forward(*args):
+    return _fused_linear_forward(L.HT_TREE, *args)
+
+
+def fern_fused_linear_forward(*args):
+    return _fused_linear_forward(L.HT_FERN, *args)
+
+
+def tree_fused_linear_backward(*args):
+    return _fused_linear_backward(L.HT_TREE, L.HT_BACKWARD_ATOMIC, *args)
+
+
+def fern_fused_linear_backward(*args):
+    return _fused_linear_backward(L.HT_FERN, L.HT_BACKWARD_ATOMIC, *args)
+
+
+def tree_fused_linear_backward_deterministic(*args):
+    """No counterpart in the reference (its fused-linear operators have no deterministic form on the GPU): the linear
+    mix here uses no atomics, so the deterministic forest backward makes the whole operator reproducible."""
+    return _fused_linear_backward(L.HT_TREE, L.HT_BACKWARD_DETERMINISTIC, *args)
+
+
+def fern_fused_linear_backward_deterministic(*args):
+    return _fused_linear_backward(L.HT_FERN, L.HT_BACKWARD_DETERMINISTIC, *args)
+
+
 # ---- contract / expand ---------------------------------------------------------------------------------------------
 _TILE_DTYPES = (torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64, torch.float32, torch.float64)
 
@@ -627,17 +720,16 @@ fern_conv3d_forward, fern_conv3d_backward = _make_conv(L.HT_FERN, 3)
 # ---- operators of the reference module that lie outside this build's path -------------------------------------------
 def _outside(name):
     def stub(*_args, **_kwargs):
-        raise RuntimeError(f"Error: hingetree_cpp.{name} is not part of this build (forest / fern / convolution "
-                           "forward+backward path only).")
+        raise RuntimeError(f"Error: hingetree_cpp.{name} is not part of this build (forest / fern / convolution / "
+                           "forest -> linear forward+backward path only).")
 
     stub.__name__ = name
     return stub
 
 
 for _name in ["sparse_tree_backward", "sparse_fern_backward", "tree_init_medians", "tree_init_greedy",
-              "fern_init_medians", "trie_forward", "trie_backward", "trie_init_medians", "tree_fused_linear_forward",
-              "tree_fused_linear_backward", "sparse_tree_fused_linear_backward", "fern_fused_linear_forward",
-              "fern_fused_linear_backward", "sparse_fern_fused_linear_backward", "tree_fusion_forward",
+              "fern_init_medians", "trie_forward", "trie_backward", "trie_init_medians",
+              "sparse_tree_fused_linear_backward", "sparse_fern_fused_linear_backward", "tree_fusion_forward",
               "tree_fusion_backward", "fern_fusion_forward", "fern_fusion_backward", "tree_fusion_fused_linear_forward",
               "tree_fusion_fused_linear_backward", "fern_fusion_fused_linear_forward",
               "fern_fusion_fused_linear_backward"]:

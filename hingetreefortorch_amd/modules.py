@@ -194,6 +194,45 @@ class HingeFernConv3d(_ConvBase):
     _function, _nd, _fern = _fn.HingeFernConv3d, 3, True
 
 
+class _FusedLinearMixin:
+    """Adds the linear layer over the tree axis (RandomHingeForest/_RandomHingeForest.py:296-330): `linear_weights`
+    [out_channels, number_of_trees] initialised like nn.Linear, `linear_bias` [out_channels] (zeros and frozen when
+    bias=False)."""
+
+    def _init_linear(self, number_of_trees, out_channels, bias):
+        import math
+        from torch.nn import init
+        self.linear_weights = nn.Parameter(torch.empty([out_channels, number_of_trees]))
+        self.linear_bias = nn.Parameter(torch.zeros([out_channels]), requires_grad=bias)
+        init.kaiming_uniform_(self.linear_weights, a=math.sqrt(5))
+        if bias:
+            fan_in, _ = init._calculate_fan_in_and_fan_out(self.linear_weights)
+            bound = 1 / math.sqrt(fan_in) if fan_in > 0 else 0
+            init.uniform_(self.linear_bias, -bound, bound)
+
+
+class RandomHingeForestFusedLinear(RandomHingeForest, _FusedLinearMixin):
+    def __init__(self, in_channels: int, number_of_trees: int, out_channels: int, depth: int, extra_outputs=None,
+                 init_type: str = "random", bias: bool = True):
+        super().__init__(in_channels, number_of_trees, depth, extra_outputs, init_type)
+        self._init_linear(number_of_trees, out_channels, bias)
+
+    def forward(self, x):
+        return _fn.HingeTreeFusedLinear.apply(x, self.thresholds, self.ordinals, self.weights, self.linear_weights,
+                                              self.linear_bias)
+
+
+class RandomHingeFernFusedLinear(RandomHingeFern, _FusedLinearMixin):
+    def __init__(self, in_channels: int, number_of_trees: int, out_channels: int, depth: int, extra_outputs=None,
+                 init_type: str = "random", bias: bool = True):
+        super().__init__(in_channels, number_of_trees, depth, extra_outputs, init_type)
+        self._init_linear(number_of_trees, out_channels, bias)
+
+    def forward(self, x):
+        return _fn.HingeFernFusedLinear.apply(x, self.thresholds, self.ordinals, self.weights, self.linear_weights,
+                                              self.linear_bias)
+
+
 class LinearHingeForest(nn.Module):
     """Linear(bias=False) -> BatchNorm1d(affine=False) -> RandomHingeForest(init_type="sequential") as one module: the
     model of the reference's README (README.md:117-129; experiments/run_letter_seq.py:45-52), where the linear layer

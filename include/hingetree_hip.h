@@ -136,6 +136,20 @@ int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, cons
                            const float *rstd, float *g, float *dlin, float *dx, void *workspace,
                            size_t workspace_bytes, void *stream);
 
+/* ---- linear mix over the tree axis behind a forest (fp32) ------------------------------------------------------------
+ * The dense half of the reference's fused-linear operators tree_fused_linear_forward / _backward and fern_*
+ * (hingetree_fused_linear.cpp:75-412; GPU: hingetree_fused_linear_gpu.cu, which accumulates the forward with global
+ * atomics). The forest half is ht_forest_forward / ht_forest_backward above; f [B, T, R] is the forest's output with
+ * R = K * M (inner data positions x outputs per leaf).
+ *   forward : out [B, O, R] = bias[o] + sum_t lin[o, t] * f[b, t, r]           (bias may be NULL)
+ *   backward: h [B, T, R]   = sum_o lin[o, t] * g[b, o, r]   -> upstream gradient for ht_forest_backward (may be NULL)
+ *             dlin [O, T]   = sum_{b, r} g[b, o, r] * f[b, t, r]                (may be NULL)
+ * Both run on the matrix cores and are deterministic (no atomics). */
+int ht_tree_mix_forward(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin,
+                        const float *bias, float *out, void *stream);
+int ht_tree_mix_backward(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin, const float *g,
+                         float *h, float *dlin, void *stream);
+
 /* ---- contract / expand -----------------------------------------------------------------------------------------------
  * Replace contract2d/3d and expand2d/3d of the reference (expand.cpp:37-227 on the CPU, expand_gpu.cu:110-172 on the
  * GPU; exported as `contract` / `expand`, hingetree.cpp:2029-2030). Tile j of a dimension covers image positions

@@ -105,6 +105,33 @@ def backward(x, thr, ord_, w, gout, need=(True, True, True), fern=False):
     return dx, dthr, dw
 
 
+def fused_linear_forward(x, thr, ord_, w, lin, bias, fern=False):
+    """bias[o] + sum_t lin[o, t] * forest(x)[b, t, ...] with the reference's order of operations."""
+    _chk(x, thr, ord_, w, lin, bias)
+    B, F, K, T, D, M = _dims(x, thr, w, fern)
+    O = lin.shape[0]
+    out = torch.empty([B, O] + list(x.shape[2:]) + list(w.shape[2:]), dtype=x.dtype)
+    getattr(lib(), "ho_fused_linear_forward" + _sfx(x))(_p(x), _p(thr), _p(ord_), _p(w), _p(lin), _p(bias), _p(out),
+                                                        _i(B), _i(F), _i(K), _i(T), _i(D), _i(M), _i(O),
+                                                        ctypes.c_int(int(fern)))
+    return out
+
+
+def fused_linear_backward(x, thr, ord_, w, lin, gout, need=(True, True, True, True), fern=False):
+    """(dX, dThr, dW, dLin) of fused_linear_forward; the bias gradient is gout summed over everything but o."""
+    _chk(x, thr, ord_, w, lin, gout)
+    B, F, K, T, D, M = _dims(x, thr, w, fern)
+    O = lin.shape[0]
+    dx = torch.zeros_like(x) if need[0] else None
+    dthr = torch.zeros_like(thr) if need[1] else None
+    dw = torch.zeros_like(w) if need[2] else None
+    dlin = torch.zeros_like(lin) if need[3] else None
+    getattr(lib(), "ho_fused_linear_backward" + _sfx(x))(_p(x), _p(thr), _p(ord_), _p(w), _p(lin), _p(gout), _p(dx),
+                                                         _p(dthr), _p(dw), _p(dlin), _i(B), _i(F), _i(K), _i(T), _i(D),
+                                                         _i(M), _i(O), ctypes.c_int(int(fern)))
+    return dx, dthr, dw, dlin
+
+
 def maps(x, thr, ord_, w, fern=False):
     """(leafmap as real, signed margin, selected ordinal int64, reachability counts as real)."""
     _chk(x, thr, ord_, w)

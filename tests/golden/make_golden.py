@@ -3,6 +3,7 @@
 
     python tests/golden/make_golden.py            # everything
     python tests/golden/make_golden.py tiles      # only the contract / expand fixtures
+    python tests/golden/make_golden.py mix        # only the forest -> linear fixtures
 
 Each file holds seeded inputs and the reference's outputs for one small case; tests compare the oracle (CPU) and the
 HIP path (GPU) against them. The fixtures are data only.
@@ -46,6 +47,31 @@ TILE_CASES = {
     "tiles3d_f64_big_pad": ([1, 2, 4, 5, 3], [3, 2, 2], [2, 1, 2], torch.float64),
 }
 
+MIX_CASES = {
+    # name: (B, F, Kd, T, D, Md, O, fern, dtype)
+    "mix_tree_f32": (10, 12, [], 7, 4, [], 5, False, torch.float32),
+    "mix_tree_f32_inner": (3, 6, [2, 3], 4, 3, [3], 6, False, torch.float32),
+    "mix_fern_f32_m2": (8, 9, [], 5, 4, [2], 3, True, torch.float32),
+    "mix_fern_f64_inner": (4, 7, [4], 3, 3, [], 2, True, torch.float64),
+}
+
+
+def write_mix(ref):
+    for name, (B, F, Kd, T, D, Md, O, fern, dtype) in MIX_CASES.items():
+        x, thr, ordn, w, _ = make_forest(B, F, Kd, T, D, Md, fern, dtype, seed=31)
+        g = torch.Generator().manual_seed(32)
+        lin = torch.randn([O, T], generator=g, dtype=dtype) / T ** 0.5
+        bias = torch.randn([O], generator=g, dtype=dtype)
+        pre = "fern_" if fern else "tree_"
+        out = getattr(ref, pre + "fused_linear_forward")(x, thr, ordn, w, lin, bias)
+        gout = torch.randn(out.shape, generator=g, dtype=dtype)
+        dx, dthr, _, dw, dlin, dbias = getattr(ref, pre + "fused_linear_backward")(
+            x, True, thr, True, ordn, False, w, True, lin, True, bias, True, gout)
+        np.savez_compressed(os.path.join(HERE, name + ".npz"), fern=np.int64(fern), x=x.numpy(), thr=thr.numpy(),
+                            ord=ordn.numpy(), w=w.numpy(), lin=lin.numpy(), bias=bias.numpy(), gout=gout.numpy(),
+                            out=out.numpy(), dx=dx.numpy(), dthr=dthr.numpy(), dw=dw.numpy(), dlin=dlin.numpy(),
+                            dbias=dbias.numpy())
+
 
 def write_tiles(ref):
     for name, (shape, window, padding, dtype) in TILE_CASES.items():
@@ -61,9 +87,12 @@ def main():
     ref = ho.reference_module()
     if ref is None:
         raise SystemExit("oracle/_ref/hingetree_cpp.so is missing: run `make -C oracle ref` first")
-    write_tiles(ref)
-    if sys.argv[1:] == ["tiles"]:
-        print("wrote", sorted(f for f in os.listdir(HERE) if f.startswith("tiles")))
+    if sys.argv[1:] != ["mix"]:
+        write_tiles(ref)
+    if sys.argv[1:] != ["tiles"]:
+        write_mix(ref)
+    if sys.argv[1:] in (["tiles"], ["mix"]):
+        print("wrote", sorted(f for f in os.listdir(HERE) if f.startswith(sys.argv[1])))
         return
     for name, (B, F, Kd, T, D, Md, fern, dtype, dist) in FOREST_CASES.items():
         x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype, seed=11, x_dist=dist)

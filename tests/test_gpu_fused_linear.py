@@ -1,0 +1,176 @@
+"""GPU parity of the forest -> linear operators (tree/fern_fused_linear_forward/backward, the HingeTreeFusedLinear /
+HingeFernFusedLinear autograd functions and the RandomHinge*FusedLinear modules) against the CPU oracle and the golden
+vectors written from the reference's own CPU build.
+
+Bar: fp32, every output and gradient within 1e-5 relative to the largest reference entry of the tensor (the sum over
+trees runs on the matrix cores in a different order from the reference's serial loop, so bit equality is not defined
+here; the forest stage underneath is the bit-exact kernel of the plain operators). Where the oracle's own serial fp32
+accumulation (the reference's order) strays from the same computation in fp64 by more than a fraction of that bar -- it
+does by 2e-5 on the largest case, whose threshold gradients sum 10 500 signed terms each -- the HIP result must sit
+within 1e-5 of the fp64 result and within 1e-5 plus the oracle's own fp64 distance of the fp32 oracle.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_forest, rel_err
+from oracle import hinge_oracle as ho
+import hingetree_cpp as ops
+from HingeTree import HingeFernFusedLinear, HingeTreeFusedLinear
+from RandomHingeForest import RandomHingeFernFusedLinear, RandomHingeForestFusedLinear
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+MIX_FILES = sorted(glob.glob(os.path.join(GOLDEN, "mix_*f32*.npz")))
+TOL = 1e-5
+
+CASES = [
+    # B, F, Kd, T, D, Md, O
+    (1, 3, [], 1, 1, [], 1),
+    (9, 11, [], 5, 3, [], 4),
+    (100, 1000, [], 100, 7, [1], 10),       # the reference's CPU-runnable forest, mixed down to 10 classes
+    (300, 40, [], 257, 5, [], 130),         # tiles with ragged edges in every GEMM dimension
+    (2048, 64, [], 130, 6, [], 16),         # large enough for the staged forest backward
+    (33, 13, [], 40, 4, [10], 7),           # extra outputs: the product runs per sample over [T, M]
+    (6, 9, [3, 2], 12, 3, [2, 2], 5),       # inner data dims and inner weight dims
+    (70, 20, [50], 130, 4, [3], 129),       # 150 inner positions: several column tiles per sample
+]
+
+
+def _inputs(case, fern, seed=0):
+    B, F, Kd, T, D, Md, O = case
+    x, thr, ordn, w, _ = make_forest(B, F, Kd, T, D, Md, fern, torch.float32, seed=seed)
+    g = torch.Generator().manual_seed(77 + seed)
+    lin = torch.randn([O, T], generator=g) / T ** 0.5
+    bias = torch.randn([O], generator=g)
+    gout = torch.randn([B, O] + list(Kd) + list(Md), generator=g)
+    return x, thr, ordn, w, lin, bias, gout
+
+
+def _check(dev, fern, x, thr, ordn, w, lin, bias, gout, want=None):
+    pre = "fern_" if fern else "tree_"
+    if want is None:
+        want = dict(out=ho.fused_linear_forward(x, thr, ordn, w, lin, bias, fern))
+        want["dx"], want["dthr"], want["dw"], want["dlin"] = ho.fused_linear_backward(x, thr, ordn, w, lin, gout, fern=fern)
+        want["dbias"] = gout.double().sum(dim=[0] + list(range(2, gout.dim()))).float()
+        x64 = [t.double() if t.is_floating_point() else t for t in (x, thr, ordn, w, lin, gout)]
+        exact = dict(zip(("dx", "dthr", "dw", "dlin"), ho.fused_linear_backward(*x64, fern=fern)))
+    else:
+        exact = {}
+    d = [t.to(dev) for t in (x, thr, ordn, w, lin, bias, gout)]
+    out = getattr(ops, pre + "fused_linear_forward")(*d[:6])
+    assert out.shape == want["out"].shape and out.dtype == torch.float32
+    assert rel_err(out.cpu(), want["out"]) <= TOL
+    for name in ("fused_linear_backward", "fused_linear_backward_deterministic"):
+        dx, dthr, dord, dw, dlin, dbias = getattr(ops, pre + name)(d[0], True, d[1], True, d[2], False, d[3], True,
+                                                                   d[4], True, d[5], True, d[6])
+        assert dord is None
+        for got, key in ((dx, "dx"), (dthr, "dthr"), (dw, "dw"), (dlin, "dlin"), (dbias, "dbias")):
+            assert got.shape == want[key].shape, key
+            slack = 0.0
+            if key in exact:
+                slack = rel_err(want[key].double(), exact[key])
+                assert rel_err(got.cpu().double(), exact[key]) <= TOL, (name, key, "fp64")
+            assert rel_err(got.cpu(), want[key]) <= TOL + slack, (name, key)
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("case", CASES, ids=[f"c{i}" for i in range(len(CASES))])
+def test_against_oracle(dev, case, fern):
+    _check(dev, fern, *_inputs(case, fern))
+
+
+@pytest.mark.parametrize("path", MIX_FILES, ids=[os.path.basename(p)[:-4] for p in MIX_FILES])
+def test_against_golden(dev, path):
+    z = np.load(path)
+    t = {k: torch.from_numpy(np.ascontiguousarray(z[k])) for k in z.files if k != "fern"}
+    _check(dev, bool(z["fern"]), t["x"], t["thr"], t["ord"], t["w"], t["lin"], t["bias"], t["gout"], want=t)
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+def test_selected_gradients_only(dev, fern):
+    x, thr, ordn, w, lin, bias, gout = _inputs(CASES[5], fern, seed=3)
+    rdx, rdthr, rdw, rdlin = ho.fused_linear_backward(x, thr, ordn, w, lin, gout, fern=fern)
+    d = [t.to(dev) for t in (x, thr, ordn, w, lin, bias, gout)]
+    back = getattr(ops, ("fern_" if fern else "tree_") + "fused_linear_backward")
+    only_lin = back(d[0], False, d[1], False, d[2], False, d[3], False, d[4], True, d[5], False, d[6])
+    assert [g is None for g in only_lin] == [True, True, True, True, False, True]
+    assert rel_err(only_lin[4].cpu(), rdlin) <= TOL
+    only_thr = back(d[0], False, d[1], True, d[2], False, d[3], False, d[4], False, d[5], True, d[6])
+    assert [g is None for g in only_thr] == [True, False, True, True, True, False]
+    assert rel_err(only_thr[1].cpu(), rdthr) <= TOL
+    with pytest.raises(RuntimeError):
+        back(d[0], True, d[1], True, d[2], True, d[3], True, d[4], True, d[5], True, d[6])
+
+
+def test_rejects_bad_input(dev):
+    x, thr, ordn, w, lin, bias, gout = (t.to(dev) for t in _inputs(CASES[1], False))
+    with pytest.raises(ValueError):
+        ops.tree_fused_linear_forward(x, thr, ordn, w, lin[:, :-1].contiguous(), bias)       # trees disagree
+    with pytest.raises(ValueError):
+        ops.tree_fused_linear_forward(x, thr, ordn, w, lin, bias[:-1].contiguous())          # out channels disagree
+    with pytest.raises(ValueError):
+        ops.tree_fused_linear_forward(x, thr, ordn, w, lin, bias.view(1, -1))                # bias rank
+    with pytest.raises(ValueError):
+        ops.tree_fused_linear_backward(x, True, thr, True, ordn, False, w, True, lin, True, bias, True,
+                                       gout[:, :-1].contiguous())
+    with pytest.raises(RuntimeError):
+        ops.tree_fused_linear_forward(*(t.double() if t.is_floating_point() else t for t in (x, thr, ordn, w, lin, bias)))
+    with pytest.raises(RuntimeError):
+        ops.tree_fused_linear_forward(x.cpu(), thr.cpu(), ordn.cpu(), w.cpu(), lin.cpu(), bias.cpu())
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+def test_autograd_and_module(dev, fern):
+    """The module's forward / backward through autograd against the oracle on the module's own parameters, and against
+    the unfused composition module(x) == linear(forest(x)) built from the plain forest operator."""
+    torch.manual_seed(4)
+    cls = RandomHingeFernFusedLinear if fern else RandomHingeForestFusedLinear
+    B, F, T, O, depth, M = 50, 30, 24, 6, 4, 3
+    model = cls(F, T, O, depth, extra_outputs=M).to(dev)
+    assert model.linear_weights.shape == (O, T) and model.linear_bias.shape == (O,) and model.linear_bias.requires_grad
+    frozen = cls(F, T, O, depth, bias=False)
+    assert not frozen.linear_bias.requires_grad and float(frozen.linear_bias.abs().max()) == 0.0
+    x = torch.randn([B, F], device=dev, requires_grad=True)
+    out = model(x)
+    assert out.shape == (B, O, M)
+    up = torch.randn(out.shape, device=dev)
+    out.backward(up)
+    p = [t.detach().cpu() for t in (x, model.thresholds, model.ordinals, model.weights, model.linear_weights, model.linear_bias)]
+    assert rel_err(out.detach().cpu(), ho.fused_linear_forward(*p, fern)) <= TOL
+    rdx, rdthr, rdw, rdlin = ho.fused_linear_backward(*p[:5], up.cpu(), fern=fern)
+    assert rel_err(x.grad.cpu(), rdx) <= TOL and rel_err(model.thresholds.grad.cpu(), rdthr) <= TOL
+    assert rel_err(model.weights.grad.cpu(), rdw) <= TOL and rel_err(model.linear_weights.grad.cpu(), rdlin) <= TOL
+    assert rel_err(model.linear_bias.grad.cpu(), up.cpu().sum(dim=(0, 2))) <= TOL
+    assert model.ordinals.grad is None
+    # unfused composition
+    fn = HingeFernFusedLinear if fern else HingeTreeFusedLinear
+    plain = getattr(ops, ("fern_" if fern else "tree_") + "forward")(x.detach(), model.thresholds.detach(),
+                                                                      model.ordinals, model.weights.detach())
+    comp = torch.einsum("ot,btm->bom", model.linear_weights.detach().double(), plain.double()) + \
+        model.linear_bias.detach().double().view(1, -1, 1)
+    again = fn.apply(x.detach(), model.thresholds.detach(), model.ordinals, model.weights.detach(),
+                     model.linear_weights.detach(), model.linear_bias.detach())
+    assert torch.equal(again, out.detach())                    # no atomics in the forward: repeatable bit for bit
+    assert rel_err(out.detach().double().cpu(), comp.cpu()) <= TOL
+
+
+def test_deterministic_switch_is_reproducible(dev):
+    x, thr, ordn, w, lin, bias, gout = (t.to(dev) for t in _inputs(CASES[4], False, seed=2))
+    prev = torch.are_deterministic_algorithms_enabled()
+    torch.use_deterministic_algorithms(True)
+    try:
+        runs = []
+        for _ in range(2):
+            leaves = [t.clone().requires_grad_(True) for t in (x, thr, w, lin, bias)]
+            out = HingeTreeFusedLinear.apply(leaves[0], leaves[1], ordn, leaves[2], leaves[3], leaves[4])
+            out.backward(gout)
+            runs.append([out.detach()] + [t.grad for t in leaves[:4]])
+        for a, b in zip(*runs):
+            assert torch.equal(a, b)
+    finally:
+        torch.use_deterministic_algorithms(prev)

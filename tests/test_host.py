@@ -63,7 +63,19 @@ def test_validation_order_on_cpu_tensors():
     with pytest.raises(RuntimeError, match="no CPU back-end"):
         ops.tree_forward(x, thr, ordn, w)
     with pytest.raises(RuntimeError, match="not part of this build"):
-        ops.tree_fused_linear_forward(x, thr, ordn, w, w, w)
+        ops.tree_fusion_forward(x, x, thr, ordn, w)
+    # forest -> linear: the reference's messages (hingetree_fused_linear.cpp:79-100), then the same refusal to run on the CPU
+    lin, bias = torch.randn(4, 3), torch.randn(4)
+    with pytest.raises(ValueError, match="inLinearBias must have 1 dimension"):
+        ops.tree_fused_linear_forward(x, thr, ordn, w, lin, bias.view(1, 4))
+    with pytest.raises(ValueError, match=r"inLinearWeightrs.shape\[0\] must be the same as inLinearBias.shape\[0\]"):
+        ops.tree_fused_linear_forward(x, thr, ordn, w, lin, bias[:2])
+    with pytest.raises(ValueError, match="same shape"):
+        ops.fern_fused_linear_forward(x, thr, ordn, w, lin[:, :2].contiguous(), bias)
+    with pytest.raises(RuntimeError, match="never has a gradient"):
+        ops.tree_fused_linear_backward(x, True, thr, True, ordn, True, w, True, lin, True, bias, True, torch.randn(8, 4))
+    with pytest.raises(RuntimeError, match="no CPU back-end"):
+        ops.tree_fused_linear_forward(x, thr, ordn, w, lin, bias)
 
 
 def test_conv_validation_on_cpu_tensors():

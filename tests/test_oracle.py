@@ -321,3 +321,65 @@ def test_tiles_padding_reads_zero_and_adjoint():
     assert e.shape == x.shape                                 # 3 * 4 - (4 // 4) * 4
     assert abs(float((t * u).sum() - (x * e).sum())) < 1e-9
     assert torch.equal(ho.expand(t, padding), x)              # every pixel is covered by exactly one tile
+
+
+# ---- forest -> linear -----------------------------------------------------------------------------------------------
+MIX_FILES = sorted(glob.glob(os.path.join(GOLDEN, "mix_*.npz")))
+
+
+def _make_mix(B, F, Kd, T, D, Md, O, fern, dtype, seed):
+    x, thr, ordn, w, _ = make_forest(B, F, Kd, T, D, Md, fern, dtype, seed=seed)
+    g = torch.Generator().manual_seed(400 + seed)
+    lin = torch.randn([O, T], generator=g, dtype=dtype) / T ** 0.5
+    bias = torch.randn([O], generator=g, dtype=dtype)
+    gout = torch.randn([B, O] + list(Kd) + list(Md), generator=g, dtype=dtype)
+    return x, thr, ordn, w, lin, bias, gout
+
+
+@pytest.mark.parametrize("path", MIX_FILES, ids=[os.path.basename(p)[:-4] for p in MIX_FILES])
+def test_golden_mix(path):
+    z = np.load(path)
+    fern = bool(z["fern"])
+    x, thr, ordn, w, lin, bias, gout = (_t(z[k]) for k in ("x", "thr", "ord", "w", "lin", "bias", "gout"))
+    assert torch.equal(ho.fused_linear_forward(x, thr, ordn, w, lin, bias, fern), _t(z["out"]))
+    dx, dthr, dw, dlin = ho.fused_linear_backward(x, thr, ordn, w, lin, gout, fern=fern)
+    assert torch.equal(dx, _t(z["dx"])) and torch.equal(dthr, _t(z["dthr"]))
+    assert torch.equal(dw, _t(z["dw"])) and torch.equal(dlin, _t(z["dlin"]))
+    # the reference's bias gradient is a torch sum over everything but the out-channel axis
+    dbias = gout.sum(dim=[0] + list(range(2, gout.dim())))
+    assert torch.allclose(dbias, _t(z["dbias"]), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.skipif(ho.reference_module() is None, reason="reference build (oracle/_ref) not present")
+@pytest.mark.parametrize("fern,dtype,Kd,Md", list(itertools.product([False, True], [torch.float32, torch.float64],
+                                                                   [[], [3, 2]], [[], [1], [4]])))
+def test_mix_against_reference_build(fern, dtype, Kd, Md):
+    ref = ho.reference_module()
+    x, thr, ordn, w, lin, bias, gout = _make_mix(7, 11, Kd, 6, 4, Md, 5, fern, dtype, seed=len(Kd) + len(Md))
+    pre = "fern_" if fern else "tree_"
+    assert torch.equal(getattr(ref, pre + "fused_linear_forward")(x, thr, ordn, w, lin, bias),
+                       ho.fused_linear_forward(x, thr, ordn, w, lin, bias, fern))
+    r = getattr(ref, pre + "fused_linear_backward")(x, True, thr, True, ordn, False, w, True, lin, True, bias, True, gout)
+    o = ho.fused_linear_backward(x, thr, ordn, w, lin, gout, fern=fern)
+    assert torch.equal(r[0], o[0]) and torch.equal(r[1], o[1]) and torch.equal(r[3], o[2]) and torch.equal(r[4], o[3])
+
+
+@pytest.mark.parametrize("fern", [False, True])
+def test_mix_is_forest_then_linear(fern):
+    """The operator is the forest followed by an affine map over the tree axis: in fp64 the fused oracle must agree
+    with that composition (forward) and with the chain rule through it (backward) to rounding. A transposed weight
+    matrix, a bias added per tree instead of per out channel, or a missing factor fails here."""
+    x, thr, ordn, w, lin, bias, gout = _make_mix(6, 9, [2], 5, 3, [3], 4, fern, torch.float64, seed=9)
+    f = ho.forward(x, thr, ordn, w, fern)                                          # [B, T, 2, 3]
+    want = torch.einsum("ot,btkm->bokm", lin, f) + bias.view(1, -1, 1, 1)
+    got = ho.fused_linear_forward(x, thr, ordn, w, lin, bias, fern)
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
+    h = torch.einsum("ot,bokm->btkm", lin, gout).contiguous()
+    dx, dthr, dw = ho.backward(x, thr, ordn, w, h, fern=fern)
+    gx, gthr, gw, glin = ho.fused_linear_backward(x, thr, ordn, w, lin, gout, fern=fern)
+    assert torch.allclose(gx, dx, rtol=1e-11, atol=1e-12) and torch.allclose(gthr, dthr, rtol=1e-11, atol=1e-12)
+    assert torch.allclose(gw, dw, rtol=1e-11, atol=1e-12)
+    assert torch.allclose(glin, torch.einsum("bokm,btkm->ot", gout, f), rtol=1e-11, atol=1e-12)
+    # with an identity mix and no bias the operator is the forest itself, bit for bit
+    eye = torch.eye(5, dtype=torch.float64)
+    assert torch.equal(ho.fused_linear_forward(x, thr, ordn, w, eye, torch.zeros(5, dtype=torch.float64), fern), f)
