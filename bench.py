@@ -42,7 +42,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the forward kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (KiB per dispatch,
 # scaled by what the same counters read for a plain 1 GiB copy: x2.0 for FETCH_SIZE, x1.0 for WRITE_SIZE); the
 # summaries are under profiles/.
-MEASURED_TRAFFIC = {"c3": None}
+MEASURED_TRAFFIC = {("c3", "train"): 4674308075}   # 1353 MB fetched + 3321 MB written (2621 MB out, 524 MB walk records)
 
 WORKLOADS = {
     # name: (B, F, T, depth, M, kind, x distribution, description)
@@ -334,7 +334,7 @@ def main():
         "config": {"workload": f"{name}: {desc}", "backward_mode": args.mode, "path": args.path, "B": B, "F": F, "T": T, "depth": depth,
                    "extra_outputs": M},
         "roofline": {"bound": "hbm", "kernel": "forward_rows_kernel" if name != "c1" else "forward", "achieved": achieved, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get(name),
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get((name, args.path)),
                      "algorithmic_bytes": fwd_bytes, "ms": fwd_ms, "samples_per_s": B / (fwd_ms * 1e-3)},
         "backward": {"mode": args.mode, "ms": bwd_ms, "samples_per_s": B / (bwd_ms * 1e-3),
                      "algorithmic_bytes": bwd_bytes, "hbm_frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
