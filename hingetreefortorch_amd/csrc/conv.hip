@@ -458,6 +458,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
   const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
   const Real *mine = tile + ty * g.sy * g.IW + tx * g.sx;
   const int tiles = g.tiles_y * g.tiles_x;
+  const int skew = int(threadIdx.x & 63u) % C;
   for (long long it = blockIdx.y; it < items; it += gridDim.y) {
     const long long b = it / tiles;
     const int t = int(it - b * tiles);
@@ -472,9 +473,15 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
       WalkResult<Real> r[kConvIlp];
       const Node<Real> *nd[kConvIlp];
       const Real *px[kConvIlp];
+      int ch[kConvIlp];
 #pragma unroll
       for (int i = 0; i < kConvIlp; ++i) {
-        const int ci = min(c + i, C - 1);
+        // Lane l takes the channels in the order skew(l), skew(l) + 1, ... (mod C): at any moment the lanes of a
+        // wavefront are spread over min(C, 64) trees, so the root-heavy threshold table sees that many times fewer
+        // same-address atomics than with all lanes on one tree.
+        int ci = min(c + i, C - 1) + skew;
+        ci = ci >= C ? ci - C : ci;
+        ch[i] = ci;
         nd[i] = nodes + ci * V;
         px[i] = mine + ci * g.TSZ;
       }
@@ -484,14 +491,14 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
       for (int i = 0; i < kConvIlp; ++i) {
         if (c + i >= C) break;
         const Real a = ht_abs(r[i].margin);
-        const int cell = ((c + i) * L + int(r[i].key)) * M;
+        const int cell = (ch[i] * L + int(r[i].key)) * M;
         Real cs = Real(0);
         for (int m = 0; m < M; ++m) {
           const Real gv = gp[m];
           cs += wl[cell + m] * gv;
           if (dw) atomicAdd(acc_w + cell + m, double(a * gv));
         }
-        if (dthr) atomicAdd(acc_t + (c + i) * V + int(r[i].vertex), -double(ht_sign(r[i].margin) * cs));
+        if (dthr) atomicAdd(acc_t + ch[i] * V + int(r[i].vertex), -double(ht_sign(r[i].margin) * cs));
       }
     }
   }
