@@ -4,6 +4,7 @@
     python tests/golden/make_golden.py            # everything
     python tests/golden/make_golden.py tiles      # only the contract / expand fixtures
     python tests/golden/make_golden.py mix        # only the forest -> linear fixtures
+    python tests/golden/make_golden.py snapshot   # only the trained-snapshot fixture
 
 Each file holds seeded inputs and the reference's outputs for one small case; tests compare the oracle (CPU) and the
 HIP path (GPU) against them. The fixtures are data only.
@@ -72,6 +73,29 @@ def write_mix(ref):
                             out=out.numpy(), dx=dx.numpy(), dthr=dthr.numpy(), dw=dw.numpy(), dlin=dlin.numpy(),
                             dbias=dbias.numpy())
 
+SNAPSHOT = ("/root/reference/rcc/Models/snapshots_unweighted_easyhard_deterministic_hingeforest_depth7_vggblock3_"
+            "randomSplit1/epoch_549.pt")
+SNAPSHOT_TREES = 3
+
+
+def write_snapshot(ref):
+    """Parameters of the first trees of the forest in one of the trained segmentation snapshots the reference ships
+    (data: thresholds, ordinals stored as float32 as old versions of the reference did, leaf weights [.., 8, 8]), and
+    what the reference's CPU build computes from them for a seeded input: forest output, leaf map, and the image the
+    8 x 8 leaf patches expand to. Read with the loader that executes nothing from the file."""
+    sd = torch.load(SNAPSHOT, map_location="cpu", weights_only=True)
+    thr = sd["forest.thresholds"][:SNAPSHOT_TREES].contiguous()
+    ordf = sd["forest.ordinals"][:SNAPSHOT_TREES].contiguous()
+    w = sd["forest.weights"][:SNAPSHOT_TREES].contiguous()
+    assert ordf.dtype == torch.float32 and torch.equal(ordf, ordf.round())
+    x = torch.randn([2, 100, 3, 4], generator=torch.Generator().manual_seed(41))
+    ordn = ordf.long()
+    out = ref.tree_forward(x, thr, ordn, w)
+    leaf = ref.tree_leafmap(x, thr, ordn, w)
+    image = ref.expand(out, [0, 0])
+    np.savez_compressed(os.path.join(HERE, "snapshot_forest_subset.npz"), thr=thr.numpy(), ord_float=ordf.numpy(),
+                        w=w.numpy(), x=x.numpy(), out=out.numpy(), leaf=leaf.numpy(), image=image.numpy())
+
 
 def write_tiles(ref):
     for name, (shape, window, padding, dtype) in TILE_CASES.items():
@@ -87,12 +111,15 @@ def main():
     ref = ho.reference_module()
     if ref is None:
         raise SystemExit("oracle/_ref/hingetree_cpp.so is missing: run `make -C oracle ref` first")
-    if sys.argv[1:] != ["mix"]:
+    only = sys.argv[1] if len(sys.argv) == 2 else None
+    if only in (None, "tiles"):
         write_tiles(ref)
-    if sys.argv[1:] != ["tiles"]:
+    if only in (None, "mix"):
         write_mix(ref)
-    if sys.argv[1:] in (["tiles"], ["mix"]):
-        print("wrote", sorted(f for f in os.listdir(HERE) if f.startswith(sys.argv[1])))
+    if only in (None, "snapshot"):
+        write_snapshot(ref)
+    if only is not None:
+        print("wrote", sorted(f for f in os.listdir(HERE) if f.startswith(only)))
         return
     for name, (B, F, Kd, T, D, Md, fern, dtype, dist) in FOREST_CASES.items():
         x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype, seed=11, x_dist=dist)

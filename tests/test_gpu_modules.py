@@ -130,3 +130,21 @@ def test_segmentation_style_usage(dev):
     ref = ho.forward(x, m.thresholds.data, m.ordinals.data, m.weights.data)
     out = m.to(dev)(x.to(dev))
     assert out.shape == (2, 6, 5, 7, 8, 8) and torch.equal(out.cpu(), ref)
+
+
+def test_trained_snapshot_subset(dev):
+    """Trained parameters from one of the segmentation snapshots the reference ships (first trees; ordinals stored as
+    float32) loaded through load_state_dict and run on the GPU: forest output, leaf map and the image the 8 x 8 leaf
+    patches expand to are those of the reference's CPU build, bit for bit."""
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "snapshot_forest_subset.npz"))
+    t = {k: torch.from_numpy(np.ascontiguousarray(z[k])) for k in z.files}
+    trees = t["thr"].shape[0]
+    forest = RHF.RandomHingeForest(in_channels=100, out_channels=trees, extra_outputs=[8, 8], depth=7)
+    forest.load_state_dict({"thresholds": t["thr"], "ordinals": t["ord_float"], "weights": t["w"]})
+    assert forest.ordinals.dtype == torch.int64
+    forest = forest.to(dev)
+    x = t["x"].to(dev)
+    out = forest(x)
+    assert torch.equal(out.detach().cpu(), t["out"])
+    assert torch.equal(forest.leafmap(x).cpu(), t["leaf"].to(torch.int64))
+    assert torch.equal(HingeTree.Expand(padding=[0, 0])(out).detach().cpu(), t["image"])

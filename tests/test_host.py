@@ -183,3 +183,38 @@ def test_public_names():
                  "fern_backward_deterministic", "tree_conv2d_forward", "tree_conv2d_backward", "tree_leafmap",
                  "tree_marginmap", "tree_reachability", "tree_speedtest", "tree_fix_thresholds", "fern_conv3d_backward"]:
         assert callable(getattr(ops, name))
+
+
+SNAPSHOTS = "/root/reference/rcc/Models"
+
+
+@pytest.mark.skipif(not os.path.isdir(SNAPSHOTS), reason="the reference's trained snapshots are not on this machine")
+def test_reference_snapshots_load_into_the_modules():
+    """Every trained snapshot the reference ships (rcc/Models/*/epoch_*.pt, read with the loader that executes nothing
+    from the file) loads into this build's RandomHingeForest, alone and as a sub-module of a network with the snapshot's
+    layout; float32 ordinals arrive as int64 (_RandomHingeForest.py:138-142, rcc/RCCSeg.py:130-134)."""
+    import glob
+    files = sorted(glob.glob(os.path.join(SNAPSHOTS, "*", "*.pt")))
+    assert files
+    for path in files:
+        sd = torch.load(path, map_location="cpu", weights_only=True)
+        assert sd["forest.ordinals"].dtype == torch.float32
+        forest = RHF.RandomHingeForest(in_channels=100, out_channels=100, extra_outputs=[8, 8], depth=7)
+        forest.load_state_dict({k[len("forest."):]: v for k, v in sd.items() if k.startswith("forest.")})
+        assert forest.ordinals.dtype == torch.int64 and not forest.ordinals.requires_grad
+        assert torch.equal(forest.ordinals.data.float(), sd["forest.ordinals"])
+        assert torch.equal(forest.thresholds.data, sd["forest.thresholds"]) and torch.equal(forest.weights.data, sd["forest.weights"])
+        assert len(forest.check_thresholds()) == 100
+
+    class Net(torch.nn.Module):   # the tail of rcc/Net.py:60-66
+        def __init__(self):
+            super().__init__()
+            self.forestbn1 = torch.nn.BatchNorm2d(100, affine=False)
+            self.features = torch.nn.Conv2d(40, 100, 1, bias=False)
+            self.forest = RHF.RandomHingeForest(in_channels=100, out_channels=100, extra_outputs=[8, 8], depth=7)
+            self.agg = torch.nn.Conv2d(100, 4, 1)
+
+    net = Net()
+    wanted = ("forestbn1.", "features.", "forest.", "agg.")
+    net.load_state_dict({k: v for k, v in sd.items() if k.startswith(wanted)})
+    assert net.forest.ordinals.dtype == torch.int64 and torch.equal(net.forest.ordinals.data.float(), sd["forest.ordinals"])

@@ -383,3 +383,21 @@ def test_mix_is_forest_then_linear(fern):
     # with an identity mix and no bias the operator is the forest itself, bit for bit
     eye = torch.eye(5, dtype=torch.float64)
     assert torch.equal(ho.fused_linear_forward(x, thr, ordn, w, eye, torch.zeros(5, dtype=torch.float64), fern), f)
+
+
+# ---- trained snapshot ----------------------------------------------------------------------------------------------
+def test_golden_snapshot_subset():
+    """Trained parameters (first trees of a segmentation snapshot the reference ships, ordinals stored as float32) and
+    what the reference's CPU build computes from them: the oracle reproduces forest output, leaf map and the expanded
+    image bit for bit; torch's fold of the 8 x 8 patches (channel = tree * 64 + patch cell) gives the same image."""
+    z = np.load(os.path.join(GOLDEN, "snapshot_forest_subset.npz"))
+    x, thr, w = _t(z["x"]), _t(z["thr"]), _t(z["w"])
+    ordn = _t(z["ord_float"]).long()
+    out = ho.forward(x, thr, ordn, w, False)
+    assert torch.equal(out, _t(z["out"]))
+    assert torch.equal(ho.maps(x, thr, ordn, w, False)[0], _t(z["leaf"]))
+    image = ho.expand(out, [0, 0])
+    assert torch.equal(image, _t(z["image"]))
+    B, T, h, wd, p, q = out.shape
+    tmp = out.view(B, T, h * wd, p * q).transpose(2, 3).reshape(B, T * p * q, h * wd)
+    assert torch.equal(Fn.fold(tmp, [h * p, wd * q], [p, q], stride=[p, q]), image)
