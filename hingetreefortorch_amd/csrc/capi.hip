@@ -118,7 +118,7 @@ int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, 
   ForestDims d;
   int rc = make_dims(s, &d);
   if (rc != HT_OK) return rc;
-  if (d.S > 0 && d.T > 0 && (!x || !thr || !ord || !w || !out))
+  if (!is_empty(d) && (!x || !thr || !ord || !w || !out))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool fern = s->kind == HT_FERN;
@@ -142,8 +142,9 @@ int ht_forest_forward_records(const ht_forest_shape *s, const void *x, const voi
   int rc = make_dims(s, &d);
   if (rc != HT_OK) return rc;
   const size_t need = ht_forest_records_bytes(s);
-  if (need == 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: walk records are not offered for this shape.");
-  if (d.S > 0 && d.T > 0 && (!x || !thr || !ord || !w || !out || !records))
+  if (need == 0 && !is_empty(d))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: walk records are not offered for this shape.");
+  if (!is_empty(d) && (!x || !thr || !ord || !w || !out || !records))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
   if (records_bytes < need) return fail(HT_ERR_INVALID_ARGUMENT, "Error: records buffer too small.");
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -173,8 +174,9 @@ int ht_forest_backward_records(const ht_forest_shape *s, const void *w, const vo
   if (mode != HT_BACKWARD_ATOMIC && mode != HT_BACKWARD_DETERMINISTIC)
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: unknown backward mode.");
   const size_t need = ht_forest_records_bytes(s);
-  if (need == 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: walk records are not offered for this shape.");
-  if (d.S > 0 && d.T > 0 && (!w || !gout || !records)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (need == 0 && !is_empty(d))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: walk records are not offered for this shape.");
+  if (!is_empty(d) && (!w || !gout || !records)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
   if (records_bytes < need) return fail(HT_ERR_INVALID_ARGUMENT, "Error: records buffer too small.");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool fern = s->kind == HT_FERN;
@@ -200,7 +202,7 @@ int ht_forest_backward(const ht_forest_shape *s, const void *x, const void *thr,
   if (rc != HT_OK) return rc;
   if (mode != HT_BACKWARD_ATOMIC && mode != HT_BACKWARD_DETERMINISTIC)
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: unknown backward mode.");
-  if (d.S > 0 && d.T > 0 && (!x || !thr || !ord || !w || !gout))
+  if (!is_empty(d) && (!x || !thr || !ord || !w || !gout))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool fern = s->kind == HT_FERN;

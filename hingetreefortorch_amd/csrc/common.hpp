@@ -35,6 +35,9 @@ struct ForestDims {
   int F, K, T, depth, V, L, M;
 };
 
+// No (sample, tree, output) triple exists: outputs are empty and every gradient is zero.
+inline bool is_empty(const ForestDims &d) { return d.S == 0 || d.T == 0 || d.M == 0; }
+
 __host__ __device__ constexpr size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 constexpr int kWave = 64;

@@ -1472,7 +1472,7 @@ int run_route(const ForestDims &d, Route route, bool fern, const Real *x, const 
 template <typename Real>
 int clear_gradients(const ForestDims &d, Route route, Real *dx, Real *dthr, Real *dw, hipStream_t stream, bool *done) {
   int rc;
-  const bool empty = d.S == 0 || d.T == 0;
+  const bool empty = is_empty(d);
   const bool clear_dx = route != Route::kStaged || empty || pick_dx_tile(d.F, sizeof(Real)) == 0;
   if (dx && clear_dx && (rc = zero_fill(dx, size_t(d.S) * d.F * sizeof(Real), stream)) != HT_OK) return rc;
   if (dthr && (rc = zero_fill(dthr, size_t(d.T) * d.V * sizeof(Real), stream)) != HT_OK) return rc;
@@ -1485,6 +1485,7 @@ int clear_gradients(const ForestDims &d, Route route, Real *dx, Real *dthr, Real
 
 template <typename Real>
 size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw) {
+  if (is_empty(d)) return 0;
   const Route r = pick_route<Real>(d, mode, need_dx, need_dw, false);
   return packed_nodes_bytes<Real>(d) + route_bytes<Real>(d, r, need_dthr, need_dw, false);
 }
@@ -1494,7 +1495,7 @@ int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *t
                     const Real *gout, Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes,
                     hipStream_t stream) {
   int rc;
-  const Route route = pick_route<Real>(d, mode, dx != nullptr, dw != nullptr, false);
+  const Route route = is_empty(d) ? Route::kFused : pick_route<Real>(d, mode, dx != nullptr, dw != nullptr, false);
   bool done;
   if ((rc = clear_gradients<Real>(d, route, dx, dthr, dw, stream, &done)) != HT_OK || done) return rc;
   const size_t node_bytes = packed_nodes_bytes<Real>(d);
@@ -1511,12 +1512,14 @@ int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *t
 template <typename Real>
 size_t forest_records_bytes(const ForestDims &d) {
   // offered where the staged kernels can consume them for every combination of requested gradients
+  if (is_empty(d)) return 0;
   if (!staged_ok<Real>(d, true, true, false)) return 0;
   return records_saved_bytes<Real>(d);
 }
 
 template <typename Real>
 size_t forest_backward_records_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw) {
+  if (is_empty(d)) return 0;
   const Route r = pick_route<Real>(d, mode, need_dx, need_dw, true);
   return route_bytes<Real>(d, r, need_dthr, need_dw, true);
 }
@@ -1526,7 +1529,7 @@ int forest_backward_records(const ForestDims &d, bool fern, const Real *w, const
                             Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes,
                             hipStream_t stream) {
   int rc;
-  const Route route = pick_route<Real>(d, mode, dx != nullptr, dw != nullptr, true);
+  const Route route = is_empty(d) ? Route::kFused : pick_route<Real>(d, mode, dx != nullptr, dw != nullptr, true);
   bool done;
   if ((rc = clear_gradients<Real>(d, route, dx, dthr, dw, stream, &done)) != HT_OK || done) return rc;
   const size_t need = route_bytes<Real>(d, route, dthr != nullptr, dw != nullptr, true);

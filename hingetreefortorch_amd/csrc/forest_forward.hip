@@ -619,6 +619,7 @@ static size_t quads_bytes(const ForestDims &d) {
 
 template <typename Real>
 size_t forest_forward_workspace(const ForestDims &d) {
+  if (is_empty(d)) return 0;
   const size_t nodes = packed_nodes_bytes<Real>(d);
   const size_t quads = (quads_ok<Real>(d, false) && rows_ok<Real>(d)) ? quads_bytes<Real>(d) : 0;
   return nodes > quads ? nodes : quads;
@@ -627,7 +628,7 @@ size_t forest_forward_workspace(const ForestDims &d) {
 template <typename Real>
 int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
                    Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream) {
-  if (d.S == 0 || d.T == 0) return HT_OK;
+  if (is_empty(d)) return HT_OK;
   if (ws == nullptr || ws_bytes < forest_forward_workspace<Real>(d))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the forward pass.");
   if (rows_ok<Real>(d)) {

@@ -413,6 +413,7 @@ int mix_backward(long long B, long long T, long long O, long long R, const float
                                                            nullptr, nullptr, stream);
     if (rc != HT_OK) return rc;
   }
+  if (dlin && (B == 0 || R == 0)) return zero_fill(dlin, size_t(O) * size_t(T) * sizeof(float), stream);
   if (dlin) {
     if (R == 1)  // dlin [O x T] = g^T [O x B] * f [B x T]
       rc = launch_gemm_batched<false, false, false, false>(g, O, 0, f, T, 0, dlin, T, 0, O, T, B, 1, nullptr, nullptr,

@@ -274,6 +274,8 @@ def linear_bn_forward(inData, inLinearWeights, eps=1e-5):
         _invalid("Error: inData must be [batch, in_features] and inLinearWeights [out_features, in_features].")
     B, K = inData.shape
     N = inLinearWeights.shape[0]
+    if B == 0:  # torch.nn.BatchNorm1d refuses an empty batch in training mode too
+        _invalid("Error: batch statistics need at least one sample.")
     lib = L.load()
     with torch.cuda.device(inData.device):
         zhat = torch.empty([B, N], dtype=torch.float32, device=inData.device)

@@ -62,3 +62,12 @@ def test_conv_golden(dev, path):
     tol = 1e-5 if x.dtype == torch.float32 else 1e-12
     for got, key in ((dx, "dx"), (dthr, "dthr"), (dw, "dw")):
         assert rel_err(got.cpu(), torch.from_numpy(z[key])) <= tol
+
+
+def test_empty_batch(dev):
+    x, thr, ordn, w = (t.to(dev) for t in make_conv(0, 3, 4, [7, 6], 3, [], [3, 3], False, torch.float32))
+    args = ([3, 3], [1, 1], [1, 1], [1, 1])
+    out = ops.tree_conv2d_forward(x, thr, ordn, w, *args)
+    assert list(out.shape) == [0, 4, 7, 6]
+    dx, dthr, dord, dw = ops.tree_conv2d_backward(x, True, thr, True, ordn, False, w, True, out, *args)
+    assert dx.shape == x.shape and dord is None and not dthr.any() and not dw.any()

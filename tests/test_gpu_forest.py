@@ -13,6 +13,7 @@ import torch
 from conftest import make_forest, rel_err
 from oracle import hinge_oracle as ho
 import hingetree_cpp as ops
+import HingeTree as HingeTreeFn
 
 pytestmark = pytest.mark.gpu
 
@@ -230,3 +231,38 @@ def test_records_path(dev, case, dtype, fern):
     assert only_w[0] is None and only_w[1] is None and rel_err(only_w[3].cpu(), rdw) <= tol
     only_x = bwd(records, False, gx, True, gthr, False, gord, False, gw, False, gg)
     assert only_x[3] is None and rel_err(only_x[0].cpu(), rdx) <= tol
+
+
+EMPTY = {"no samples": (0, 5, [], 3, 2, []), "no inner positions": (4, 5, [0], 3, 2, []),
+         "no outputs per leaf": (4, 5, [], 3, 2, [0]), "no trees": (4, 5, [], 0, 2, [2]),
+         "no samples, staged sizes": (0, 64, [], 300, 6, [10])}
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("name", sorted(EMPTY))
+def test_empty_inputs(dev, name, fern):
+    """Shapes with no (sample, tree, output) triple: the reference's CPU loops run zero times, so outputs are empty
+    tensors of the right shape and every requested gradient is zero (hingetree.cpp:119,233,260,287)."""
+    B, F, Kd, T, D, Md = EMPTY[name]
+    x, thr, ordn, w, gout = _gpu(dev, *make_forest(B, F, Kd, T, D, Md, fern, torch.float32))
+    pre = "fern_" if fern else "tree_"
+    out = getattr(ops, pre + "forward")(x, thr, ordn, w)
+    assert list(out.shape) == [B, T] + Kd + Md and out.numel() == 0
+    for back in ("backward", "backward_deterministic"):
+        dx, dthr, dord, dw = getattr(ops, pre + back)(x, True, thr, True, ordn, False, w, True, gout)
+        assert dx.shape == x.shape and dthr.shape == thr.shape and dw.shape == w.shape and dord is None
+        assert not dx.any() and not dthr.any() and not dw.any()
+    leaf = getattr(ops, pre + "leafmap")(x, thr, ordn, w)
+    assert list(leaf.shape) == [B, T] + Kd
+    reach = getattr(ops, pre + "reachability")(x, thr, ordn, w)
+    assert list(reach.shape) == [T, 2 ** D]
+    if B * T == 0 or 0 in Kd:
+        assert not reach.any()
+    else:
+        assert int(reach.sum()) == B * T        # the walks do not depend on the outputs per leaf
+    # the training path of the autograd function
+    xg, tg, wg = x.clone().requires_grad_(True), thr.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    fn = HingeTreeFn.HingeFern if fern else HingeTreeFn.HingeTree
+    y = fn.apply(xg, tg, ordn, wg)
+    y.backward(gout)
+    assert not xg.grad.any() and not tg.grad.any() and not wg.grad.any()

@@ -174,3 +174,12 @@ def test_deterministic_switch_is_reproducible(dev):
             assert torch.equal(a, b)
     finally:
         torch.use_deterministic_algorithms(prev)
+
+
+def test_empty_batch(dev):
+    x, thr, ordn, w, lin, bias, gout = (t.to(dev) for t in _inputs((0, 5, [], 3, 2, [], 2), False))
+    out = ops.tree_fused_linear_forward(x, thr, ordn, w, lin, bias)
+    assert list(out.shape) == [0, 2]
+    grads = ops.tree_fused_linear_backward(x, True, thr, True, ordn, False, w, True, lin, True, bias, True, gout)
+    assert grads[2] is None and all(g.shape == t.shape and not g.any() for g, t in
+                                    zip(grads[:2] + grads[3:], (x, thr, w, lin, bias)))
