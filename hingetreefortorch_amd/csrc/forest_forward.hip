@@ -288,7 +288,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
                                                                       Real *__restrict__ out,
                                                                       Records<Real, COMPACT> rec,
                                                                       int trees_per_block, FastDiv div_m,
-                                                                      FastDiv div_u_full) {
+                                                                      FastDiv div_u_full, int wpitch) {
   typedef Real Vec __attribute__((ext_vector_type(GW)));
   constexpr int NT = kForestThreads;
   constexpr int kWaves = NT / kWave;
@@ -404,7 +404,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
     if (nt != TPW) div_u = FastDiv(U);
     const int total = n_live * U;
     Real *obase = out + ((long long)s0 * d.T + tb) * d.M;
-    const Real *wbase = w + (long long)tb * d.L * d.M;
+    const Real *wbase = w + (long long)tb * d.L * wpitch;  // wpitch: elements between leaf rows (M, or padded)
     for (int u0 = lane; u0 < total; u0 += kWave * kRowUnroll) {
       Real a[kRowUnroll];
       Vec wv[kRowUnroll];
@@ -417,7 +417,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
         const int tt = div_m.div(e), m = e - tt * d.M;
         const uint32_t key = p_key[jj * LDP + tt];
         a[q] = p_abs[jj * LDP + tt];
-        wv[q] = *reinterpret_cast<const Vec *>(wbase + (uint32_t(tt) * uint32_t(d.L) + key) * uint32_t(d.M) + m);
+        wv[q] = *reinterpret_cast<const Vec *>(wbase + (uint32_t(tt) * uint32_t(d.L) + key) * uint32_t(wpitch) + m);
         off[q] = uint32_t(jj) * TM + uint32_t(e);
       }
 #pragma unroll
@@ -470,8 +470,8 @@ static inline bool quads_ok(const ForestDims &d, bool fern) {
 }
 
 template <typename Real, bool FERN, bool QUAD, int BT, int GW, bool RECORD, bool COMPACT>
-int launch_rows(const ForestDims &d, const Real *x, const void *vertices, const Real *w, Real *out, void *records,
-                hipStream_t stream) {
+int launch_rows(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, Real *out,
+                void *records, hipStream_t stream) {
   constexpr int TPW = kWave / BT * kRowIlp;
   constexpr int TP = kForestThreads / kWave * TPW;
   const size_t lds = rows_lds_bytes<Real>(d.F, BT);
@@ -486,38 +486,39 @@ int launch_rows(const ForestDims &d, const Real *x, const void *vertices, const 
                                    int(lds)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, vertices,
                      int(quads_per_tree(d.depth)), w, out, rec, trees_per_block, FastDiv(d.M),
-                     FastDiv(TPW * d.M / GW));
+                     FastDiv(TPW * d.M / GW), wpitch);
   HT_LAUNCH_CHECK("forest forward (rows)");
   return HT_OK;
 }
 
 template <typename Real, bool FERN, bool QUAD, int BT, int GW>
-int launch_rows_rec(const ForestDims &d, const Real *x, const void *vertices, const Real *w, Real *out, void *records,
-                    hipStream_t stream) {
-  if (!records) return launch_rows<Real, FERN, QUAD, BT, GW, false, true>(d, x, vertices, w, out, records, stream);
-  if (compact_ok(d)) return launch_rows<Real, FERN, QUAD, BT, GW, true, true>(d, x, vertices, w, out, records, stream);
-  return launch_rows<Real, FERN, QUAD, BT, GW, true, false>(d, x, vertices, w, out, records, stream);
+int launch_rows_rec(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, Real *out,
+                    void *records, hipStream_t stream) {
+  if (!records) return launch_rows<Real, FERN, QUAD, BT, GW, false, true>(d, x, vertices, w, wpitch, out, records, stream);
+  if (compact_ok(d))
+    return launch_rows<Real, FERN, QUAD, BT, GW, true, true>(d, x, vertices, w, wpitch, out, records, stream);
+  return launch_rows<Real, FERN, QUAD, BT, GW, true, false>(d, x, vertices, w, wpitch, out, records, stream);
 }
 
 template <typename Real, bool FERN, bool QUAD, int BT>
-int launch_rows_gw(const ForestDims &d, const Real *x, const void *vertices, const Real *w, Real *out, void *records,
-                   hipStream_t stream) {
+int launch_rows_gw(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, Real *out,
+                   void *records, hipStream_t stream) {
   const uintptr_t pw = reinterpret_cast<uintptr_t>(w), po = reinterpret_cast<uintptr_t>(out);
-  if (d.M % 4 == 0 && pw % (4 * sizeof(Real)) == 0 && po % (4 * sizeof(Real)) == 0)
-    return launch_rows_rec<Real, FERN, QUAD, BT, 4>(d, x, vertices, w, out, records, stream);
-  if (d.M % 2 == 0 && pw % (2 * sizeof(Real)) == 0 && po % (2 * sizeof(Real)) == 0)
-    return launch_rows_rec<Real, FERN, QUAD, BT, 2>(d, x, vertices, w, out, records, stream);
-  return launch_rows_rec<Real, FERN, QUAD, BT, 1>(d, x, vertices, w, out, records, stream);
+  if (d.M % 4 == 0 && wpitch % 4 == 0 && pw % (4 * sizeof(Real)) == 0 && po % (4 * sizeof(Real)) == 0)
+    return launch_rows_rec<Real, FERN, QUAD, BT, 4>(d, x, vertices, w, wpitch, out, records, stream);
+  if (d.M % 2 == 0 && wpitch % 2 == 0 && pw % (2 * sizeof(Real)) == 0 && po % (2 * sizeof(Real)) == 0)
+    return launch_rows_rec<Real, FERN, QUAD, BT, 2>(d, x, vertices, w, wpitch, out, records, stream);
+  return launch_rows_rec<Real, FERN, QUAD, BT, 1>(d, x, vertices, w, wpitch, out, records, stream);
 }
 
 template <typename Real, bool FERN, bool QUAD>
-int dispatch_rows(const ForestDims &d, const Real *x, const void *vertices, const Real *w, Real *out, void *records,
-                  hipStream_t stream) {
+int dispatch_rows(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, Real *out,
+                  void *records, hipStream_t stream) {
   switch (pick_rows_tile<Real>(d.F)) {
-    case 64: return launch_rows_gw<Real, FERN, QUAD, 64>(d, x, vertices, w, out, records, stream);
-    case 32: return launch_rows_gw<Real, FERN, QUAD, 32>(d, x, vertices, w, out, records, stream);
-    case 16: return launch_rows_gw<Real, FERN, QUAD, 16>(d, x, vertices, w, out, records, stream);
-    default: return launch_rows_gw<Real, FERN, QUAD, 8>(d, x, vertices, w, out, records, stream);
+    case 64: return launch_rows_gw<Real, FERN, QUAD, 64>(d, x, vertices, w, wpitch, out, records, stream);
+    case 32: return launch_rows_gw<Real, FERN, QUAD, 32>(d, x, vertices, w, wpitch, out, records, stream);
+    case 16: return launch_rows_gw<Real, FERN, QUAD, 16>(d, x, vertices, w, wpitch, out, records, stream);
+    default: return launch_rows_gw<Real, FERN, QUAD, 8>(d, x, vertices, w, wpitch, out, records, stream);
   }
 }
 
@@ -617,12 +618,49 @@ static size_t quads_bytes(const ForestDims &d) {
   return align_up(size_t(d.T) * size_t(quads_per_tree(d.depth)) * sizeof(QuadNode), 256);
 }
 
+// Leaf rows of M values are gathered at random; a row that straddles two 64-byte sectors costs two requests to L2,
+// and the rate of those requests per CU is what bounds the row kernel. So where a row is not already a whole number
+// of sectors (or a power-of-two fraction of one), the forward pass first copies the leaf table to a pitch that is:
+// M = 10 floats -> 16. Worth it only when the gathers outnumber the table rows by far.
 template <typename Real>
-size_t forest_forward_workspace(const ForestDims &d) {
-  if (is_empty(d)) return 0;
+static int weight_pitch(const ForestDims &d) {
+  constexpr int kSector = 64 / int(sizeof(Real));
+  int p = d.M;
+  if (d.M <= kSector) {
+    p = 1;
+    while (p < d.M) p <<= 1;
+  } else {
+    p = (d.M + kSector - 1) / kSector * kSector;
+  }
+  if (p == d.M || !rows_ok<Real>(d)) return d.M;
+  if (d.S < 8ll * d.L || (long long)kWave * kRowIlp * d.L * p >= (1ll << 31)) return d.M;
+  if (size_t(d.T) * d.L * p * sizeof(Real) > (size_t(1) << 30)) return d.M;
+  return p;
+}
+
+template <typename Real>
+static size_t vertex_bytes(const ForestDims &d) {
   const size_t nodes = packed_nodes_bytes<Real>(d);
   const size_t quads = (quads_ok<Real>(d, false) && rows_ok<Real>(d)) ? quads_bytes<Real>(d) : 0;
   return nodes > quads ? nodes : quads;
+}
+
+template <typename Real>
+size_t forest_forward_workspace(const ForestDims &d) {
+  if (is_empty(d)) return 0;
+  const int p = weight_pitch<Real>(d);
+  return vertex_bytes<Real>(d) + (p != d.M ? align_up(size_t(d.T) * d.L * p * sizeof(Real), 256) : 0);
+}
+
+template <typename Real>
+__global__ __launch_bounds__(256) void pad_rows_kernel(const Real *__restrict__ w, Real *__restrict__ dst, long long rows,
+                                                       int M, int P) {
+  const long long n = rows * P;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const long long r = i / P;
+    const int m = int(i - r * P);
+    dst[i] = m < M ? w[r * M + m] : Real(0);
+  }
 }
 
 template <typename Real>
@@ -632,6 +670,16 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
   if (ws == nullptr || ws_bytes < forest_forward_workspace<Real>(d))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the forward pass.");
   if (rows_ok<Real>(d)) {
+    int wpitch = weight_pitch<Real>(d);
+    if (wpitch != d.M) {
+      Real *padded = reinterpret_cast<Real *>(static_cast<unsigned char *>(ws) + vertex_bytes<Real>(d));
+      const long long rows = (long long)d.T * d.L;
+      long long blocks = (rows * wpitch + 255) / 256;
+      if (blocks > 16 * kNumCUs) blocks = 16 * kNumCUs;
+      hipLaunchKernelGGL(pad_rows_kernel<Real>, dim3((unsigned)blocks), dim3(256), 0, stream, w, padded, rows, d.M, wpitch);
+      HT_LAUNCH_CHECK("pad leaf rows");
+      w = padded;
+    }
     if constexpr (std::is_same<Real, float>::value) {
       if (quads_ok<Real>(d, fern)) {
         const int NQ = int(quads_per_tree(d.depth));
@@ -639,13 +687,13 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
         hipLaunchKernelGGL(pack_quads_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, thr, ord,
                            static_cast<QuadNode *>(ws), d.T, d.V, NQ, d.F);
         HT_LAUNCH_CHECK("pack two-level vertices");
-        return dispatch_rows<Real, false, true>(d, x, ws, w, out, records, stream);
+        return dispatch_rows<Real, false, true>(d, x, ws, w, wpitch, out, records, stream);
       }
     }
     int rc = pack_nodes<Real>(d, thr, ord, ws, stream);
     if (rc != HT_OK) return rc;
-    return fern ? dispatch_rows<Real, true, false>(d, x, ws, w, out, records, stream)
-                : dispatch_rows<Real, false, false>(d, x, ws, w, out, records, stream);
+    return fern ? dispatch_rows<Real, true, false>(d, x, ws, w, wpitch, out, records, stream)
+                : dispatch_rows<Real, false, false>(d, x, ws, w, wpitch, out, records, stream);
   }
   int rc = pack_nodes<Real>(d, thr, ord, ws, stream);
   if (rc != HT_OK) return rc;
