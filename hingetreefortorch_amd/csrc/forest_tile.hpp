@@ -20,8 +20,9 @@ static inline int pick_tile(int F, size_t reserve) {
 
 // Cooperative load of the tile starting at sample s0. NT must be a multiple of BT, so a thread always serves the
 // same sample j and only its feature index advances. With K == 1 a sample's features are contiguous: each lane then
-// takes four of them per load (a quarter of the load instructions; the memory pipeline charges an instruction by the
-// lines its lanes touch, and here every lane is on a different row).
+// takes four of them per load, and a wavefront walks along its own span of every row (16-byte chunks
+// wave * CPW ... (wave + 1) * CPW), so the 128-byte lines of a row are requested by consecutive loads of one wavefront
+// and reach L2 as one request each, rather than once from each of four wavefronts.
 template <typename Real, int BT, int NT>
 __device__ __forceinline__ void load_tile(Real *xs, const Real *__restrict__ x, const ForestDims &d, long long s0) {
   typedef Real Vec4 __attribute__((ext_vector_type(4)));
@@ -30,11 +31,18 @@ __device__ __forceinline__ void load_tile(Real *xs, const Real *__restrict__ x, 
   const bool live = s < d.S;
   const long long base = live ? (s / d.K) * d.FK + (s % d.K) : 0;
   if (d.K == 1 && d.F % 4 == 0 && reinterpret_cast<uintptr_t>(x) % sizeof(Vec4) == 0) {
-    for (int f = (threadIdx.x / BT) * 4; f < d.F; f += NT / BT * 4) {
+    constexpr int G = NT / BT;                           // chunk slots of the workgroup per step
+    constexpr int R = BT >= kWave ? 1 : kWave / BT;      // ... of which a wavefront holds R
+    constexpr int W = G / R > 0 ? G / R : 1;             // spans
+    const int slot = threadIdx.x / BT, span = slot / R, r = slot % R;
+    const int chunks = d.F / 4;
+    const int cpw = ((chunks + W - 1) / W + R - 1) / R * R;  // chunks per span, a multiple of R
+    const int c_end = min(chunks, (span + 1) * cpw);
+    for (int c = span * cpw + r; c < c_end; c += R) {
       Vec4 v = {Real(0), Real(0), Real(0), Real(0)};
-      if (live) v = *reinterpret_cast<const Vec4 *>(x + base + f);
+      if (live) v = *reinterpret_cast<const Vec4 *>(x + base + 4 * c);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) xs[(f + i) * BT + j] = v[i];
+      for (int i = 0; i < 4; ++i) xs[(4 * c + i) * BT + j] = v[i];
     }
     return;
   }
