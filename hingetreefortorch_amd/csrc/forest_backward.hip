@@ -127,23 +127,34 @@ __global__ void det_init_kernel(DetHeader *h) {
   }
 }
 
-// max |p[i]| (NaN counts as +inf) folded into *slot.
+// max |p[i]| (NaN counts as +inf) folded into *slot. Four independent 16-byte loads are in flight per thread.
 template <typename Real>
 __global__ __launch_bounds__(256) void absmax_kernel(const Real *__restrict__ p, long long n,
                                                      unsigned long long *slot) {
   constexpr int VEC = 16 / sizeof(Real);
+  constexpr int kInFlight = 4;
   typedef Real Vec __attribute__((ext_vector_type(VEC)));
-  double m = 0.0;
+  Real m = Real(0);
   auto take = [&](Real r) {
-    const double v = fabs(double(r));
-    if (!(v <= m)) m = (v != v) ? double(INFINITY) : v;
+    const Real v = ht_abs(r);
+    if (!(v <= m)) m = (v != v) ? Real(INFINITY) : v;
   };
   const long long tid = (long long)blockIdx.x * 256 + threadIdx.x, nthreads = (long long)gridDim.x * 256;
   long long body = 0;
   if (reinterpret_cast<uintptr_t>(p) % 16 == 0) {
     body = n / VEC;
     const Vec *pv = reinterpret_cast<const Vec *>(p);
-    for (long long i = tid; i < body; i += nthreads) {
+    long long i = tid;
+    for (; i + (kInFlight - 1) * nthreads < body; i += kInFlight * nthreads) {
+      Vec v[kInFlight];
+#pragma unroll
+      for (int q = 0; q < kInFlight; ++q) v[q] = __builtin_nontemporal_load(pv + i + q * nthreads);
+#pragma unroll
+      for (int q = 0; q < kInFlight; ++q)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) take(v[q][e]);
+    }
+    for (; i < body; i += nthreads) {
       const Vec v = __builtin_nontemporal_load(pv + i);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) take(v[e]);
@@ -151,11 +162,12 @@ __global__ __launch_bounds__(256) void absmax_kernel(const Real *__restrict__ p,
     body *= VEC;
   }
   for (long long i = body + tid; i < n; i += nthreads) take(p[i]);
+  double md = double(m);
   for (int off = 32; off > 0; off >>= 1) {
-    const double o = __shfl_xor(m, off, kWave);
-    if (!(o <= m)) m = o;
+    const double o = __shfl_xor(md, off, kWave);
+    if (!(o <= md)) md = o;
   }
-  if ((threadIdx.x & (kWave - 1)) == 0 && m > 0.0) atomicMax(slot, (unsigned long long)__double_as_longlong(m));
+  if ((threadIdx.x & (kWave - 1)) == 0 && md > 0.0) atomicMax(slot, (unsigned long long)__double_as_longlong(md));
 }
 
 __device__ inline void det_pick_scale(double bound, double count, double *scale, double *inv, int *fallback) {
@@ -491,7 +503,8 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
                                                                    unsigned long long *dw_fixed,
                                                                    const DetHeader *hdr, int log2_tb,
                                                                    long long part_size, bool need_c, bool dw_atomic,
-                                                                   int num_groups) {
+                                                                   int num_groups, float *dthr_fold,
+                                                                   uint32_t thr_lds_offset) {
   typedef LeanSplit<M> Split;
   constexpr int P = Split::P, VE = Split::VE, ROUNDS = Split::ROUNDS, SHIFT = Split::SHIFT;
   static_assert(M <= 16, "at most four lanes per pair");
@@ -501,6 +514,9 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
   typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
   extern __shared__ __align__(16) unsigned char smem[];
   Acc *acc = reinterpret_cast<Acc *>(smem);
+  // dthr_fold (atomic mode, where LDS has room behind the leaf accumulators): dThr of the group's trees is reduced
+  // here as well, by selected vertex, and the separate pass over the records and c is not needed.
+  double *acc_thr = reinterpret_cast<double *>(smem + thr_lds_offset);
   double scale = 1.0, inv_scale = 1.0;
   if (FIXED) {
     if (hdr->fallback_w) dw = nullptr;
@@ -515,10 +531,11 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
   const int t0 = group * TB;
   const int nt = min(TB, d.T - t0);
   const uint32_t LM = uint32_t(d.L) * M;
-  if (dw) {
+  if (dw)
     for (uint32_t i = threadIdx.x; i < uint32_t(nt) * LM; i += kForestThreads) acc[i] = Acc(0);
-    __syncthreads();
-  }
+  if (dthr_fold)
+    for (uint32_t i = threadIdx.x; i < uint32_t(nt) * uint32_t(d.V); i += kForestThreads) acc_thr[i] = 0.0;
+  if (dw || dthr_fold) __syncthreads();
   const long long s_begin = (long long)blockIdx.y * part_size;
   const long long s_end = min(d.S, s_begin + part_size);
   const int lane = threadIdx.x & (kWave - 1);
@@ -583,6 +600,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     uint32_t a_r;   // record words of the pair this lane loads (key | vertex << 16, margin)
     float mg_r;
     float mg_own;   // copy of mg_r that survives the reuse of a_r / mg_r for a later block
+    uint32_t v_own;  // ... and the selected vertex of that record
     float mg[P];    // per sub-step: margin of the pair this lane's group serves
     uint32_t rel[P];  // ... and its element offset (tree, leaf, first chunk element) in the group's weights
     Float4U gv[P], wv[P];
@@ -602,6 +620,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
   };
   auto issue_w = [&](Stage &st, const bool (&on)[P]) {
     st.mg_own = st.mg_r;
+    if (dthr_fold) st.v_own = (st.a_r >> rec.vshift) & key_mask;
     static_for<P>([&](auto u_tag) {
       constexpr int u = decltype(u_tag)::value;
       const uint32_t key = uint32_t(group_bcast<P, u>(int(st.a_r))) & key_mask;
@@ -643,7 +662,11 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
         c_mine = (li == u) ? partial : c_mine;
       }
     }
-    if (need_c && (FULL || have)) rec.c[record_index(sblk, have)] = ht_sign(st.mg_own) * c_mine;
+    if (need_c && (FULL || have)) {
+      const float c = ht_sign(st.mg_own) * c_mine;
+      rec.c[record_index(sblk, have)] = c;
+      if (dthr_fold) atomicAdd(acc_thr + uint32_t(rec_t) * uint32_t(d.V) + st.v_own, -double(c));
+    }
   };
 
   // This wavefront's blocks start at first, first + stride, ...; nfull of them are complete (64 existing pairs).
@@ -694,8 +717,19 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     issue_w(st, on);
     compute(st, sblk, have, on, std::false_type{});
   }
+  if (dw || dthr_fold) __syncthreads();
+  if (dthr_fold) {
+    float *dst = dthr_fold + (long long)t0 * d.V;
+    const uint32_t n = uint32_t(nt) * uint32_t(d.V);
+    for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) {
+      if (dw_atomic) {
+        if (acc_thr[i] != 0.0) atomicAdd(dst + i, float(acc_thr[i]));
+      } else {
+        dst[i] = float(acc_thr[i]);
+      }
+    }
+  }
   if (dw) {
-    __syncthreads();
     float *dst = dw + (long long)t0 * LM;
     const uint32_t n = uint32_t(nt) * LM;
     if (FIXED) {
@@ -1169,7 +1203,8 @@ int launch_tree_kernel_u(const ForestDims &d, const TreePlan &p, int P, const Re
 template <typename Real, bool COMPACT, bool FIXED>
 int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, const Real *gout,
                        Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
-                       bool need_c, hipStream_t stream) {
+                       bool need_c, Real *dthr, bool *dthr_done, hipStream_t stream) {
+  *dthr_done = false;
   if constexpr (std::is_same<Real, float>::value && COMPACT) {
     // the specialised kernel: contiguous rows, a power-of-two tree group, 32-bit offsets inside a block and a group
     int log2_tb = 0;
@@ -1177,17 +1212,26 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
     const bool fits = d.K == 1 && (1 << log2_tb) == p.TB && p.TB <= 16 &&
                       (long long)kWave * d.T * d.M < (1ll << 31) && (long long)p.TB * d.L * d.M < (1ll << 31);
     if (fits && (d.M == 10 || d.M == 1)) {
+      // dThr rides along where its fp64 table fits behind the leaf accumulators (atomic mode: the fixed-point scale of
+      // c is only known once every c exists)
+      const size_t thr_off = align_up(p.lds, 16), thr_lds = size_t(p.TB) * d.V * sizeof(double);
+      const bool fold = !FIXED && dthr != nullptr && need_c && thr_off + thr_lds <= size_t(kLdsBytes);
+      const size_t lds = fold ? thr_off + thr_lds : p.lds;
+      float *dthr_fold = fold ? dthr : nullptr;
+      *dthr_done = fold;
       HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(d.M == 10 ? (const void *)tree_lean_kernel<10, FIXED>
                                                                                 : (const void *)tree_lean_kernel<1, FIXED>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(p.lds)));
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
       const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
       const dim3 grid((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts);
       if (d.M == 10)
-        hipLaunchKernelGGL((tree_lean_kernel<10, FIXED>), grid, dim3(kForestThreads), p.lds, stream, d, w, gout, rec, dw,
-                           dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups);
+        hipLaunchKernelGGL((tree_lean_kernel<10, FIXED>), grid, dim3(kForestThreads), lds, stream, d, w, gout, rec, dw,
+                           dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
+                           uint32_t(thr_off));
       else
-        hipLaunchKernelGGL((tree_lean_kernel<1, FIXED>), grid, dim3(kForestThreads), p.lds, stream, d, w, gout, rec, dw,
-                           dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups);
+        hipLaunchKernelGGL((tree_lean_kernel<1, FIXED>), grid, dim3(kForestThreads), lds, stream, d, w, gout, rec, dw,
+                           dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
+                           uint32_t(thr_off));
       HT_LAUNCH_CHECK("forest backward (trees)");
       return HT_OK;
     }
@@ -1307,7 +1351,8 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
     if (dthr && dthr_gy > 1 && (rc = zero_fill(dthr_fixed, size_t(d.T) * d.V * 8, stream)) != HT_OK) return rc;
   }
 
-  rc = launch_tree_kernel<Real, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
+  bool dthr_done = false;
+  rc = launch_tree_kernel<Real, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, dthr, &dthr_done, stream);
   if (rc != HT_OK) return rc;
 
   if (FIXED) {
@@ -1340,7 +1385,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
     }
   }
 
-  if (dthr) {
+  if (dthr && !dthr_done) {
     hipLaunchKernelGGL((dthr_kernel<Real, COMPACT, FIXED>), dim3((unsigned)d.T, (unsigned)dthr_gy), dim3(256),
                        size_t(d.V) * sizeof(double), stream, d, rec, dthr, dthr_fixed, hdr, dthr_part, dthr_gy > 1);
     HT_LAUNCH_CHECK("forest backward (dThr)");
