@@ -167,7 +167,15 @@ __global__ __launch_bounds__(256) void absmax_kernel(const Real *__restrict__ p,
     const double o = __shfl_xor(md, off, kWave);
     if (!(o <= md)) md = o;
   }
-  if ((threadIdx.x & (kWave - 1)) == 0 && md > 0.0) atomicMax(slot, (unsigned long long)__double_as_longlong(md));
+  // one atomic per workgroup: thousands of atomics on the one slot would serialise in L2 for longer than the pass reads
+  __shared__ double part[256 / kWave];
+  if ((threadIdx.x & (kWave - 1)) == 0) part[threadIdx.x / kWave] = md;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int i = 1; i < 256 / kWave; ++i)
+      if (!(part[i] <= md)) md = part[i];
+    if (md > 0.0) atomicMax(slot, (unsigned long long)__double_as_longlong(md));
+  }
 }
 
 __device__ inline void det_pick_scale(double bound, double count, double *scale, double *inv, int *fallback) {
