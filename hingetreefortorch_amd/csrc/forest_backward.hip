@@ -780,6 +780,13 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
   const long long s_begin = (long long)blockIdx.y * part_size;
   const long long s_end = min(d.S, s_begin + part_size);
   constexpr int kBatch = 8;  // loads in flight per thread
+  // The root and its children are selected far more often than any other vertex; as LDS atomics those hits would
+  // serialise on one address, so every lane sums them in registers instead (integer sums in deterministic mode, so
+  // the result stays independent of the order).
+  constexpr int kTop = 3;
+  Acc top[kTop];
+#pragma unroll
+  for (int k = 0; k < kTop; ++k) top[k] = Acc(0);
   for (long long s0 = s_begin + threadIdx.x; s0 < s_end; s0 += 256 * kBatch) {
     uint32_t v[kBatch];
     Real cv[kBatch];
@@ -793,11 +800,25 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
 #pragma unroll
     for (int i = 0; i < kBatch; ++i) {
       if (s0 + i * 256 >= s_end) break;
-      if (FIXED)
-        atomicAdd(reinterpret_cast<unsigned long long *>(acc) + v[i], to_fixed(-double(cv[i]), scale));
+      Acc val;
+      if constexpr (FIXED)
+        val = to_fixed(-double(cv[i]), scale);
       else
-        atomicAdd(reinterpret_cast<double *>(acc) + v[i], -double(cv[i]));
+        val = -double(cv[i]);
+      if (v[i] < uint32_t(kTop)) {
+#pragma unroll
+        for (int k = 0; k < kTop; ++k) top[k] += v[i] == uint32_t(k) ? val : Acc(0);
+      } else {
+        atomicAdd(acc + v[i], val);
+      }
     }
+  }
+  // the lanes' sums for the top vertices: reduced over the wavefront, then one atomic each
+#pragma unroll
+  for (int k = 0; k < kTop; ++k) {
+    Acc sum = top[k];
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0 && k < d.V) atomicAdd(acc + k, sum);
   }
   __syncthreads();
   Real *dst = dthr + (long long)t * d.V;
