@@ -504,7 +504,7 @@ __device__ __forceinline__ int group_bcast(int v) {
   }
 }
 
-template <int M, bool FIXED>
+template <int M, bool FIXED, bool WLDS>
 __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d, const float *__restrict__ w,
                                                                    const float *__restrict__ gout,
                                                                    Records<float, true> rec, float *dw,
@@ -512,7 +512,8 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
                                                                    const DetHeader *hdr, int log2_tb,
                                                                    long long part_size, bool need_c, bool dw_atomic,
                                                                    int num_groups, float *dthr_fold,
-                                                                   uint32_t thr_lds_offset) {
+                                                                   uint32_t thr_lds_offset, uint32_t w_lds_offset) {
+  static_assert(!WLDS || M == 1, "leaf weights are staged in LDS for single-output leaves only");
   typedef LeanSplit<M> Split;
   constexpr int P = Split::P, VE = Split::VE, ROUNDS = Split::ROUNDS, SHIFT = Split::SHIFT;
   static_assert(M <= 16, "at most four lanes per pair");
@@ -525,6 +526,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
   // dthr_fold (atomic mode, where LDS has room behind the leaf accumulators): dThr of the group's trees is reduced
   // here as well, by selected vertex, and the separate pass over the records and c is not needed.
   double *acc_thr = reinterpret_cast<double *>(smem + thr_lds_offset);
+  float *w_lds = reinterpret_cast<float *>(smem + w_lds_offset);  // WLDS: the group's leaf weights
   double scale = 1.0, inv_scale = 1.0;
   if (FIXED) {
     if (hdr->fallback_w) dw = nullptr;
@@ -543,7 +545,9 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     for (uint32_t i = threadIdx.x; i < uint32_t(nt) * LM; i += kForestThreads) acc[i] = Acc(0);
   if (dthr_fold)
     for (uint32_t i = threadIdx.x; i < uint32_t(nt) * uint32_t(d.V); i += kForestThreads) acc_thr[i] = 0.0;
-  if (dw || dthr_fold) __syncthreads();
+  if (WLDS && need_c)
+    for (uint32_t i = threadIdx.x; i < uint32_t(nt) * LM; i += kForestThreads) w_lds[i] = w[(long long)t0 * LM + i];
+  if (dw || dthr_fold || WLDS) __syncthreads();
   const long long s_begin = (long long)blockIdx.y * part_size;
   const long long s_end = min(d.S, s_begin + part_size);
   const int lane = threadIdx.x & (kWave - 1);
@@ -634,7 +638,13 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
       const uint32_t key = uint32_t(group_bcast<P, u>(int(st.a_r))) & key_mask;
       st.mg[u] = __int_as_float(group_bcast<P, u>(__float_as_int(st.mg_r)));
       st.rel[u] = woff + key * M;
-      if (need_c) st.wv[u] = load_chunk(wbase + (on[u] ? st.rel[u] : uint32_t(e0)), false);
+      if (need_c) {
+        if constexpr (WLDS) {
+          st.wv[u] = Float4U{w_lds[on[u] ? st.rel[u] : 0u], 0.f, 0.f, 0.f};
+        } else {
+          st.wv[u] = load_chunk(wbase + (on[u] ? st.rel[u] : uint32_t(e0)), false);
+        }
+      }
     });
   };
   auto compute = [&](Stage &st, long long sblk, bool have, const bool (&on)[P], auto full_tag) {
@@ -1179,22 +1189,48 @@ struct TreePlan {
   size_t lds;
 };
 
-static bool plan_trees(const ForestDims &d, bool need_dw, TreePlan *p) {
+// Single-output leaf tables (M == 1, 4 bytes per leaf) are small enough to sit in LDS next to the accumulators of the
+// lean tree kernel; its leaf-weight gathers then never leave the CU.
+static inline size_t staged_weights_per_tree(const ForestDims &d, bool lean) {
+  return lean && d.M == 1 ? size_t(d.L) * sizeof(float) : 0;
+}
+
+static bool plan_trees(const ForestDims &d, bool need_dw, bool lean, TreePlan *p) {
   const size_t per_tree = size_t(d.L) * d.M * sizeof(double);
+  const size_t w_tree = staged_weights_per_tree(d, lean);
   int tb = 4;
   if (need_dw) {
     if (per_tree > size_t(kLdsBytes)) return false;
     tb = int(size_t(kLdsBytes) / per_tree);
   }
+  if (w_tree != 0) {
+    // room for the staged weights and the vertex table of the group as well; the lean kernel wants a power of two
+    const size_t all = (need_dw ? per_tree : 0) + w_tree + size_t(d.V) * sizeof(double);
+    int fit = int(size_t(kLdsBytes - 64) / all);
+    if (fit < 1) fit = 1;
+    if (tb > fit) tb = fit;
+    while (tb & (tb - 1)) tb &= tb - 1;
+  }
   if (tb > kMaxGroupTrees) tb = kMaxGroupTrees;
   if (tb > d.T) tb = d.T;
-  // keep at least ~one workgroup per CU by shrinking the groups before splitting the samples
-  while (tb > 4 && (d.T + tb - 1) / tb < kNumCUs) tb = (tb + 1) / 2;
+  // Keep at least ~one workgroup per CU by shrinking the groups before splitting the samples -- except for
+  // single-output leaves, where a group reads only 4 * TB bytes of every 128-byte line of upstream gradients it
+  // requests: there wide groups matter more, and the samples are split instead.
+  const bool keep = w_tree != 0;
+  while (!keep && tb > 4 && (d.T + tb - 1) / tb < kNumCUs) tb = (tb + 1) / 2;
   p->TB = tb;
   p->groups = (d.T + tb - 1) / tb;
   long long parts = 1;
   if (p->groups < kNumCUs) parts = (kNumCUs + p->groups - 1) / p->groups;
   const long long max_parts = (d.S + 4 * kForestThreads - 1) / (4 * kForestThreads);  // >= 4 samples per thread
+  if (keep && p->groups < kNumCUs) {  // the split that leaves the fewest CUs idle in the last round
+    double best = -1.0;
+    for (long long c = 1; c <= 16 && c <= max_parts; ++c) {
+      const long long wgs = c * p->groups, rounds = (wgs + kNumCUs - 1) / kNumCUs;
+      const double eff = double(wgs) / double(rounds * kNumCUs);
+      if (eff > best + 0.02) best = eff, parts = c;
+    }
+  }
   if (parts > max_parts) parts = max_parts;
   if (parts < 1) parts = 1;
   if (parts > 65535) parts = 65535;
@@ -1243,24 +1279,35 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
     if (fits && (d.M == 10 || d.M == 1)) {
       // dThr rides along where its fp64 table fits behind the leaf accumulators (atomic mode: the fixed-point scale of
       // c is only known once every c exists)
-      const size_t thr_off = align_up(p.lds, 16), thr_lds = size_t(p.TB) * d.V * sizeof(double);
-      const bool fold = !FIXED && dthr != nullptr && need_c && thr_off + thr_lds <= size_t(kLdsBytes);
-      const size_t lds = fold ? thr_off + thr_lds : p.lds;
+      const size_t acc_lds = dw ? size_t(p.TB) * d.L * d.M * sizeof(double) : 0;
+      const size_t thr_off = align_up(acc_lds, 16), thr_lds = size_t(p.TB) * d.V * sizeof(double);
+      const size_t w_lds = size_t(p.TB) * staged_weights_per_tree(d, true);
+      const bool stage_w = w_lds != 0 && need_c && thr_off + thr_lds + w_lds <= size_t(kLdsBytes);
+      const bool fold = !FIXED && dthr != nullptr && need_c &&
+                        thr_off + thr_lds + (stage_w ? w_lds : 0) <= size_t(kLdsBytes);
+      const size_t w_off = fold ? thr_off + thr_lds : thr_off;
+      size_t lds = stage_w ? w_off + w_lds : (fold ? thr_off + thr_lds : acc_lds);
+      if (lds < p.lds) lds = p.lds;
       float *dthr_fold = fold ? dthr : nullptr;
       *dthr_done = fold;
-      HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(d.M == 10 ? (const void *)tree_lean_kernel<10, FIXED>
-                                                                                : (const void *)tree_lean_kernel<1, FIXED>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
+      const void *fn = d.M == 10 ? (const void *)tree_lean_kernel<10, FIXED, false>
+                                 : (stage_w ? (const void *)tree_lean_kernel<1, FIXED, true>
+                                            : (const void *)tree_lean_kernel<1, FIXED, false>);
+      HT_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
       const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
       const dim3 grid((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts);
       if (d.M == 10)
-        hipLaunchKernelGGL((tree_lean_kernel<10, FIXED>), grid, dim3(kForestThreads), lds, stream, d, w, gout, rec, dw,
-                           dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
-                           uint32_t(thr_off));
+        hipLaunchKernelGGL((tree_lean_kernel<10, FIXED, false>), grid, dim3(kForestThreads), lds, stream, d, w, gout,
+                           rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
+                           uint32_t(thr_off), uint32_t(w_off));
+      else if (stage_w)
+        hipLaunchKernelGGL((tree_lean_kernel<1, FIXED, true>), grid, dim3(kForestThreads), lds, stream, d, w, gout,
+                           rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
+                           uint32_t(thr_off), uint32_t(w_off));
       else
-        hipLaunchKernelGGL((tree_lean_kernel<1, FIXED>), grid, dim3(kForestThreads), lds, stream, d, w, gout, rec, dw,
-                           dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
-                           uint32_t(thr_off));
+        hipLaunchKernelGGL((tree_lean_kernel<1, FIXED, false>), grid, dim3(kForestThreads), lds, stream, d, w, gout,
+                           rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
+                           uint32_t(thr_off), uint32_t(w_off));
       HT_LAUNCH_CHECK("forest backward (trees)");
       return HT_OK;
     }
@@ -1317,13 +1364,13 @@ static bool prefer_fused(const ForestDims &d) { return double(d.S) * double(d.T)
 struct FixedLayout {
   size_t header, dw, dthr, total;
 };
-static FixedLayout fixed_layout(const ForestDims &d, bool need_dthr, bool need_dw) {
+static FixedLayout fixed_layout(const ForestDims &d, bool need_dthr, bool need_dw, bool lean) {
   FixedLayout l{};
   TreePlan plan;
   l.header = 0;
   size_t at = kDetHeaderBytes;
   l.dw = at;
-  if (need_dw && plan_trees(d, true, &plan) && plan.parts > 1) at += align_up(size_t(d.T) * d.L * d.M * 8, 256);
+  if (need_dw && plan_trees(d, true, lean, &plan) && plan.parts > 1) at += align_up(size_t(d.T) * d.L * d.M * 8, 256);
   l.dthr = at;
   long long part_size;
   int gy;
@@ -1355,7 +1402,8 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
   const bool need_c = dx || dthr;
   const long long pairs = (long long)d.T * d.S;
   TreePlan plan;
-  if (!plan_trees(d, dw != nullptr, &plan)) return fail(HT_ERR_RUNTIME, "Error: leaf table too large.");
+  constexpr bool kLean = std::is_same<Real, float>::value && COMPACT;
+  if (!plan_trees(d, dw != nullptr, kLean && d.K == 1, &plan)) return fail(HT_ERR_RUNTIME, "Error: leaf table too large.");
   long long dthr_part;
   int dthr_gy;
   plan_dthr(d, &dthr_part, &dthr_gy);
@@ -1363,7 +1411,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
   DetHeader *hdr = nullptr;
   unsigned long long *dw_fixed = nullptr, *dthr_fixed = nullptr;
   if (FIXED) {
-    const FixedLayout lay = fixed_layout(d, dthr != nullptr, dw != nullptr);
+    const FixedLayout lay = fixed_layout(d, dthr != nullptr, dw != nullptr, kLean && d.K == 1);
     unsigned char *base = static_cast<unsigned char *>(fixed_ws);
     hdr = reinterpret_cast<DetHeader *>(base + lay.header);
     dw_fixed = reinterpret_cast<unsigned long long *>(base + lay.dw);
@@ -1507,7 +1555,8 @@ template <typename Real>
 size_t route_bytes(const ForestDims &d, Route r, bool need_dthr, bool need_dw, bool have_records) {
   if (r == Route::kFused) return 0;
   size_t bytes = (have_records ? 0 : records_saved_bytes<Real>(d)) + records_scratch_bytes<Real>(d);
-  if (r == Route::kFixed) bytes += fixed_layout(d, need_dthr, need_dw).total;
+  if (r == Route::kFixed)
+    bytes += fixed_layout(d, need_dthr, need_dw, std::is_same<Real, float>::value && compact_ok(d) && d.K == 1).total;
   return bytes;
 }
 
