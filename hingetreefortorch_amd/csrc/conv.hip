@@ -237,9 +237,9 @@ static bool make_tile(const ConvGeom &g, ConvTile *t) {
 
 // Cooperative load of the input region of tile (tyi, txi) of image b, all channels: a thread owns one or two cells of
 // the region and copies them channel by channel (the coordinate arithmetic is done once per cell, not per element).
-template <typename Real>
+template <typename Real, bool CHECK = false>
 __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restrict__ x, const ConvTile &g, int C,
-                                               long long b, int tyi, int txi) {
+                                               long long b, int tyi, int txi, int *special) {
   const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
   const long long chan = (long long)g.H * g.W;
   const Real *img = x + b * C * chan;
@@ -249,8 +249,14 @@ __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restric
     Real *q = tile + e;
     if (gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) {
       const Real *p = img + (long long)gy * g.W + gx;
+      bool plain = true;
 #pragma unroll 4
-      for (int c = 0; c < C; ++c) q[c * g.TSZ] = p[c * chan];
+      for (int c = 0; c < C; ++c) {
+        const Real v = p[c * chan];
+        if (CHECK) plain = plain && plain_feature(v);
+        q[c * g.TSZ] = v;
+      }
+      if (CHECK && !plain) *special = 1;  // see walk_paths_plain; never reset, every writer stores the same value
     } else {
       for (int c = 0; c < C; ++c) q[c * g.TSZ] = Real(0);
     }
@@ -258,10 +264,10 @@ __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restric
 }
 
 // Trees (and optionally leaf weights) of out channel j into LDS.
-template <typename Real>
+template <typename Real, bool CHECK = false>
 __device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, const ConvTile &g, int C, int V, int LM,
                                                  int j, const Real *__restrict__ thr, const int64_t *__restrict__ ord,
-                                                 const Real *__restrict__ w) {
+                                                 const Real *__restrict__ w, int *special) {
   const long long first = (long long)j * C * V;
   for (int i = threadIdx.x; i < C * V; i += kConvThreads) {
     const int tap = clamp_ordinal(ord[first + i], g.taps);
@@ -270,6 +276,7 @@ __device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, co
     n.thr = thr[first + i];
     n.ord = ky * g.dy * g.IW + kx * g.dx;
     nodes[i] = n;
+    if (CHECK && !plain_threshold(n.thr)) *special = 1;
   }
   if (wl) {
     const long long wfirst = (long long)j * C * LM;
@@ -278,7 +285,7 @@ __device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, co
 }
 
 struct ConvLds {
-  size_t tile, acc_x, nodes, wl, acc_w, acc_t, total;
+  size_t tile, acc_x, nodes, wl, acc_w, acc_t, flag, total;
 };
 
 template <typename Real>
@@ -297,8 +304,28 @@ static ConvLds conv_lds_layout(const ConvTile &t, int C, int V, int LM, bool dx_
   if (tree_acc) at += align_up(size_t(C) * LM * sizeof(double), 16);
   l.acc_t = at;
   if (tree_acc) at += align_up(size_t(C) * V * sizeof(double), 16);
+  l.flag = at;  // one word: set once the tile or the staged trees hold a value that rules out walk_paths_plain
+  at += 16;
   l.total = at;
   return l;
+}
+
+// kConvIlp walks of one output position through the staged trees nd[] over the tile planes px[]: the short form where
+// the workgroup's data allow it (see walk_paths_plain), else the general one.
+template <typename Real, bool FERN, bool TRACK>
+__device__ __forceinline__ void conv_walks(bool plain, int depth, const Node<Real> *const (&nd)[kConvIlp],
+                                           const Real *const (&px)[kConvIlp], WalkResult<Real> (&r)[kConvIlp]) {
+  // (the backward kernels are bound by LDS traffic, and the short form reads the selected vertex a second time:
+  // measured slower there, so they keep the general walk)
+  if constexpr (std::is_same<Real, float>::value && !TRACK) {
+    if (plain) {
+      walk_paths_plain<FERN, TRACK, kConvIlp>(
+          depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
+      return;
+    }
+  }
+  walk_paths<Real, FERN, TRACK, kConvIlp>(
+      depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
 }
 
 // MREG = outputs per leaf kept in registers per pass over the channels (1, 4 or 16: the smallest that holds M, so the
@@ -317,7 +344,10 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_forward_kernel(ConvTi
   Real *wl = reinterpret_cast<Real *>(smem + lay.wl);
   const int tyi = blockIdx.x / g.tiles_x, txi = blockIdx.x - tyi * g.tiles_x;
   const long long b = blockIdx.z;
-  load_conv_tile<Real>(tile, x, g, C, b, tyi, txi);
+  int *special = reinterpret_cast<int *>(smem + lay.flag);
+  if (threadIdx.x == 0) *special = 0;
+  __syncthreads();
+  load_conv_tile<Real, true>(tile, x, g, C, b, tyi, txi, special);
   const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
   const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
   const bool live = oy < g.OH && ox < g.OW;
@@ -326,9 +356,10 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_forward_kernel(ConvTi
   const int j_begin = blockIdx.y * j_per, j_end = min(Cout, j_begin + j_per);
   for (int j = j_begin; j < j_end; ++j) {
     __syncthreads();  // the tile is complete / the previous out channel's trees are no longer read
-    stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w);
+    stage_conv_trees<Real, true>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
     __syncthreads();
     if (!live) continue;
+    const bool plain = *special == 0;
     Real *o = out + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
     for (int m0 = 0; m0 < M; m0 += MREG) {
       const int mc = min(MREG, M - m0);
@@ -346,8 +377,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_forward_kernel(ConvTi
           nd[i] = nodes + ci * V;
           px[i] = mine + ci * g.TSZ;
         }
-        walk_paths<Real, FERN, false, kConvIlp>(
-            depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
+        conv_walks<Real, FERN, false>(plain, depth, nd, px, r);
 #pragma unroll
         for (int i = 0; i < kConvIlp; ++i) {
           if (c + i >= C) break;
@@ -383,7 +413,10 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_dx_kernel(ConvTile g,
   Real *wl = reinterpret_cast<Real *>(smem + lay.wl);
   const int tyi = blockIdx.x / g.tiles_x, txi = blockIdx.x - tyi * g.tiles_x;
   const long long b = blockIdx.z;
-  load_conv_tile<Real>(tile, x, g, C, b, tyi, txi);
+  int *special = reinterpret_cast<int *>(smem + lay.flag);
+  if (threadIdx.x == 0) *special = 0;
+  __syncthreads();
+  load_conv_tile<Real>(tile, x, g, C, b, tyi, txi, special);
   for (int i = threadIdx.x; i < C * g.TSZ; i += kConvThreads) acc[i] = 0.0;
   const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
   const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
@@ -394,9 +427,10 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_dx_kernel(ConvTile g,
   const int j_begin = blockIdx.y * j_per, j_end = min(Cout, j_begin + j_per);
   for (int j = j_begin; j < j_end; ++j) {
     __syncthreads();
-    stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w);
+    stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
     __syncthreads();
     if (!live) continue;
+    const bool plain = *special == 0;
     const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
     for (int c = 0; c < C; c += kConvIlp) {
       WalkResult<Real> r[kConvIlp];
@@ -408,8 +442,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_dx_kernel(ConvTile g,
         nd[i] = nodes + ci * V;
         px[i] = mine + ci * g.TSZ;
       }
-      walk_paths<Real, FERN, true, kConvIlp>(
-          depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
+      conv_walks<Real, FERN, true>(plain, depth, nd, px, r);
 #pragma unroll
       for (int i = 0; i < kConvIlp; ++i) {
         if (c + i >= C) break;
@@ -452,7 +485,10 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
   double *acc_t = reinterpret_cast<double *>(smem + lay.acc_t);
   const int j = blockIdx.x;
   const int LM = L * M;
-  stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w);
+  int *special = reinterpret_cast<int *>(smem + lay.flag);
+  if (threadIdx.x == 0) *special = 0;
+  __syncthreads();
+  stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
   for (int i = threadIdx.x; i < C * LM; i += kConvThreads) acc_w[i] = 0.0;
   for (int i = threadIdx.x; i < C * V; i += kConvThreads) acc_t[i] = 0.0;
   const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
@@ -464,8 +500,9 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
     const int t = int(it - b * tiles);
     const int tyi = t / g.tiles_x, txi = t - tyi * g.tiles_x;
     __syncthreads();  // the previous tile is no longer read (first pass: the staged trees are complete)
-    load_conv_tile<Real>(tile, x, g, C, b, tyi, txi);
+    load_conv_tile<Real>(tile, x, g, C, b, tyi, txi, special);
     __syncthreads();
+    const bool plain = *special == 0;
     const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
     if (oy >= g.OH || ox >= g.OW) continue;
     const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
@@ -485,8 +522,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
         nd[i] = nodes + ci * V;
         px[i] = mine + ci * g.TSZ;
       }
-      walk_paths<Real, FERN, true, kConvIlp>(
-          depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
+      conv_walks<Real, FERN, true>(plain, depth, nd, px, r);
 #pragma unroll
       for (int i = 0; i < kConvIlp; ++i) {
         if (c + i >= C) break;

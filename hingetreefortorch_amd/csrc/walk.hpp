@@ -144,6 +144,72 @@ __device__ __forceinline__ void walk_paths(int depth, NodeFn node, FeatureFn fea
   }
 }
 
+// walk_paths for float data known to be "plain": every feature and threshold finite and no threshold equal to -0.0.
+// Then t = thr - x carries everything the walk needs -- |t| is |margin| and the sign bit of t is the decision
+// (x > thr  <=>  t < 0; t is +0.0 whenever x == thr, and never NaN) -- so a level costs one subtraction, one funnel
+// shift that appends the sign bit to the path, and the minimum tracking. With TRACK only the level of the smallest
+// |margin| is carried through the loop (first level wins ties, as in the reference); its vertex is rebuilt from the
+// finished path and read once more for the signed margin and the ordinal.
+template <bool FERN, bool TRACK, int N, typename NodeFn, typename FeatureFn>
+__device__ __forceinline__ void walk_paths_plain(int depth, NodeFn node, FeatureFn feature, WalkResult<float> (&r)[N]) {
+  uint32_t path[N];
+  float best_abs[N];
+  uint32_t best_lvl[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const Node<float> n = node(i, 0u);
+    const float t = n.thr - feature(i, int(n.ord));
+    path[i] = __float_as_uint(t) >> 31;
+    best_abs[i] = ht_abs(t);
+    best_lvl[i] = 0;
+  }
+  for (int lvl = 1; lvl < depth; ++lvl) {
+    const uint32_t first = FERN ? uint32_t(lvl) : (1u << lvl) - 1u;  // wave uniform
+    Node<float> n[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) n[i] = node(i, FERN ? first : first + path[i]);
+    float t[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) t[i] = n[i].thr - feature(i, int(n[i].ord));
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const float a = ht_abs(t[i]);
+      if (TRACK) {
+        const bool closer = a < best_abs[i];
+        best_abs[i] = closer ? a : best_abs[i];
+        best_lvl[i] = closer ? uint32_t(lvl) : best_lvl[i];
+      } else {
+        best_abs[i] = __builtin_fminf(best_abs[i], a);
+      }
+      path[i] = __builtin_amdgcn_alignbit(path[i], __float_as_uint(t[i]), 31);  // (path << 1) | sign(t)
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    r[i].key = __brev(path[i]) >> (32 - depth);
+    if (TRACK) {
+      const uint32_t lvl = best_lvl[i];
+      const uint32_t vertex = FERN ? lvl : ((1u << lvl) - 1u) + (path[i] >> (uint32_t(depth) - lvl));
+      const Node<float> n = node(i, vertex);
+      r[i].vertex = vertex;
+      r[i].ord = uint32_t(n.ord);
+      r[i].margin = feature(i, int(n.ord)) - n.thr;
+    } else {
+      r[i].vertex = 0;
+      r[i].ord = 0;
+      r[i].margin = best_abs[i];
+    }
+  }
+}
+
+// Whether a value keeps a walk "plain" in the sense of walk_paths_plain.
+__device__ __forceinline__ bool plain_feature(float v) { return ht_abs(v) < __builtin_inff(); }
+__device__ __forceinline__ bool plain_threshold(float v) {
+  return ht_abs(v) < __builtin_inff() && __float_as_uint(v) != 0x80000000u;
+}
+__device__ __forceinline__ bool plain_feature(double) { return false; }
+__device__ __forceinline__ bool plain_threshold(double) { return false; }
+
 // Single walk over separate threshold / ordinal arrays (used where the vertices are not packed).
 // `node(i)` returns (threshold, ordinal) of decision i; `feature(f)` returns this sample's value of feature f.
 template <typename Real, bool FERN, typename NodeFn, typename FeatureFn>

@@ -71,3 +71,47 @@ def test_empty_batch(dev):
     assert list(out.shape) == [0, 4, 7, 6]
     dx, dthr, dord, dw = ops.tree_conv2d_backward(x, True, thr, True, ordn, False, w, True, out, *args)
     assert dx.shape == x.shape and dord is None and not dthr.any() and not dw.any()
+
+
+def _same_bits(a, b):
+    """Equal values, NaN in the same places."""
+    return torch.equal(a.isnan(), b.isnan()) and torch.equal(a.nan_to_num(0.0, 1.0, -1.0), b.nan_to_num(0.0, 1.0, -1.0))
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("special", ["ties and zeros", "negative zero thresholds", "nan", "inf", "plain"])
+def test_conv_special_values(dev, special, fern):
+    """The tiled kernels walk by the sign of thr - x where every value of a workgroup is finite and no threshold is
+    -0.0, and by the reference's comparisons otherwise: both must agree with the oracle bit for bit, in particular on
+    exact ties (x == thr goes left with a zero margin), on the zeros read from the padding against thresholds of either
+    zero, and on non-finite values (a NaN margin goes left and is never the minimum after the root)."""
+    B, C, Cout, size, D, ker, pad = 2, 3, 5, [19, 37], 4, [3, 3], [1, 1]
+    x, thr, ordn, w = make_conv(B, C, Cout, size, D, [], ker, fern, torch.float32, seed=8)
+    g = torch.Generator().manual_seed(12)
+    if special == "ties and zeros":
+        x = torch.round(x * 2) / 2                     # many exact zeros and repeated values
+        thr = torch.round(thr * 2) / 2                 # ... that thresholds hit exactly
+    elif special == "negative zero thresholds":
+        x = torch.round(x)
+        thr = torch.where(torch.rand(thr.shape, generator=g) < 0.5, torch.zeros_like(thr), torch.round(thr))
+        thr = torch.where(thr == 0, torch.full_like(thr, -0.0), thr)
+        assert (thr == 0).any() and torch.signbit(thr[thr == 0]).all()
+    elif special == "nan":
+        x.view(-1)[::97] = float("nan")
+        thr.view(-1)[::31] = float("nan")
+    elif special == "inf":
+        x.view(-1)[::89] = float("inf")
+        x.view(-1)[5::131] = float("-inf")
+        thr.view(-1)[::29] = float("inf")
+    args = (ker, [1, 1], pad, [1, 1])
+    ref = ho.conv_forward(x, thr, ordn, w, *args, fern)
+    pre = ("fern_" if fern else "tree_") + "conv2d_"
+    d = [t.to(dev) for t in (x, thr, ordn, w)]
+    out = getattr(ops, pre + "forward")(*d, *args)
+    assert _same_bits(out.cpu(), ref)
+    if special in ("nan", "inf"):
+        return                                          # gradients of non-finite inputs are not compared
+    gout = torch.randn(ref.shape, generator=g)
+    rdx, rdthr, rdw = ho.conv_backward(x, thr, ordn, w, gout, *args, fern=fern)
+    dx, dthr, _, dw = getattr(ops, pre + "backward")(d[0], True, d[1], True, d[2], False, d[3], True, gout.to(dev), *args)
+    assert rel_err(dx.cpu(), rdx) <= 1e-5 and rel_err(dthr.cpu(), rdthr) <= 1e-5 and rel_err(dw.cpu(), rdw) <= 1e-5
