@@ -266,3 +266,48 @@ def test_empty_inputs(dev, name, fern):
     y = fn.apply(xg, tg, ordn, wg)
     y.backward(gout)
     assert not xg.grad.any() and not tg.grad.any() and not wg.grad.any()
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("special", ["ties and zeros", "negative zero thresholds", "nan", "inf"])
+def test_special_values(dev, special, fern):
+    """Exact ties (x == thr goes left with a zero margin), zeros of either sign on both sides of the comparison, and
+    non-finite values (a NaN margin goes left and never replaces a smaller one after the root): outputs and what the
+    training path records must be the oracle's bit for bit, whichever form of the walk a kernel picks for its data."""
+    B, F, T, D, M = 300, 24, 70, 6, 2
+    x, thr, ordn, w, gout = make_forest(B, F, [], T, D, [M], fern, torch.float32, seed=21)
+    g = torch.Generator().manual_seed(22)
+    if special == "ties and zeros":
+        x, thr = torch.round(x * 2) / 2, torch.round(thr * 2) / 2
+    elif special == "negative zero thresholds":
+        x = torch.round(x)
+        thr = torch.where(torch.rand(thr.shape, generator=g) < 0.5, torch.zeros_like(thr), torch.round(thr))
+        thr = torch.where(thr == 0, torch.full_like(thr, -0.0), thr)
+        x = torch.where((x == 0) & (torch.rand(x.shape, generator=g) < 0.5), torch.full_like(x, -0.0), x)
+    elif special == "nan":
+        x.view(-1)[::97] = float("nan")
+        thr.view(-1)[::31] = float("nan")
+    else:
+        x.view(-1)[::89] = float("inf")
+        x.view(-1)[5::131] = float("-inf")
+        thr.view(-1)[::29] = float("inf")
+    pre = "fern_" if fern else "tree_"
+    d = _gpu(dev, x, thr, ordn, w, gout)
+
+    def same(a, b):
+        return torch.equal(a.isnan(), b.isnan()) and torch.equal(a.nan_to_num(0.0, 1.0, -1.0), b.nan_to_num(0.0, 1.0, -1.0))
+
+    ref = ho.forward(x, thr, ordn, w, fern)
+    assert same(getattr(ops, pre + "forward")(*d[:4]).cpu(), ref)
+    out, records = getattr(ops, pre + "forward_records")(*d[:4])
+    assert same(out.cpu(), ref)
+    leaf, margin, sel, _ = ho.maps(x, thr, ordn, w, fern)
+    assert torch.equal(getattr(ops, pre + "leafmap")(*d[:4]).cpu(), leaf.to(torch.int64))
+    gm, gs = getattr(ops, pre + "marginmap")(*d[:4])
+    assert same(gm.cpu(), margin) and torch.equal(gs.cpu(), sel)
+    if special in ("nan", "inf"):
+        return
+    rdx, rdthr, rdw = ho.backward(x, thr, ordn, w, gout, fern=fern)
+    dx, dthr, _, dw = getattr(ops, pre + "backward_records")(records, False, d[0], True, d[1], True, d[2], False, d[3],
+                                                             True, d[4])
+    assert rel_err(dx.cpu(), rdx) <= 1e-5 and rel_err(dthr.cpu(), rdthr) <= 1e-5 and rel_err(dw.cpu(), rdw) <= 1e-5
