@@ -125,8 +125,33 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
           }
         }
       }
+    } else if (d.K >= BT) {
+      // Inner data dimensions: for a fixed tree the rows of consecutive inner positions follow each other,
+      // out[b, t, k .. k + BT, 0 .. M) -- one contiguous run per tree unless the tile crosses into the next batch
+      // row, which moves the rest of the run by (T - 1) * K * M elements. Lanes run along (position, m) in vectors
+      // of VW elements; the tree is uniform per pass of the loop, so its part of every address is scalar.
+      const long long b0 = s0 / d.K;
+      const int k0 = int(s0 - b0 * d.K);
+      const long long wrap = (long long)(d.T - 1) * d.K * d.M;
+      const int vecs = BT * d.M / VW;  // per tree
+      for (int t2 = 0; t2 < nt; ++t2) {
+        Real *obase = out + ((b0 * d.T + tb + t2) * d.K + k0) * d.M;
+        const Real *wbase = w + (long long)(tb + t2) * d.L * d.M;
+        for (int v = threadIdx.x; v < vecs; v += NT) {
+          const int r = v * VW;
+          const int jj = div_m.div(r), m = r - jj * d.M;
+          if (s0 + jj >= d.S) continue;
+          const uint32_t key = r_key[jj * LDR + t2];
+          const Real a = r_abs[jj * LDR + t2];
+          const Vec wv = *reinterpret_cast<const Vec *>(wbase + (long long)key * d.M + m);
+          Vec o;
+#pragma unroll
+          for (int i = 0; i < VW; ++i) o[i] = a * wv[i];
+          *reinterpret_cast<Vec *>(obase + r + (k0 + jj >= d.K ? wrap : 0ll)) = o;
+        }
+      }
     } else {
-      // out[b, t, k .. , 0 .. M) is contiguous for a fixed tree
+      // inner dimensions shorter than the tile: generic addressing
       const int row = BT * d.M, total = nt * row;
       for (int idx = threadIdx.x; idx < total; idx += NT) {
         const int t2 = idx / row, r = idx - t2 * row;
@@ -560,11 +585,12 @@ int launch_forward_rec(const ForestDims &d, const Real *x, const Node<Real> *nod
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT>
 int launch_forward_as(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
                       void *records, hipStream_t stream) {
-  // widest output vector that M and the pointers allow (K > 1 keeps scalar outputs)
+  // widest output vector that M and the pointers allow (inner dimensions shorter than the tile keep scalar outputs)
   const uintptr_t pw = reinterpret_cast<uintptr_t>(w), po = reinterpret_cast<uintptr_t>(out);
-  if (d.K == 1 && d.M % 4 == 0 && pw % (4 * sizeof(Real)) == 0 && po % (4 * sizeof(Real)) == 0)
+  const bool runs = d.K == 1 || d.K >= BT;  // the branches of the kernel that store whole vectors
+  if (runs && d.M % 4 == 0 && pw % (4 * sizeof(Real)) == 0 && po % (4 * sizeof(Real)) == 0)
     return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 4>(d, x, nodes, w, out, records, stream);
-  if (d.K == 1 && d.M % 2 == 0 && pw % (2 * sizeof(Real)) == 0 && po % (2 * sizeof(Real)) == 0)
+  if (runs && d.M % 2 == 0 && pw % (2 * sizeof(Real)) == 0 && po % (2 * sizeof(Real)) == 0)
     return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 2>(d, x, nodes, w, out, records, stream);
   return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 1>(d, x, nodes, w, out, records, stream);
 }
