@@ -63,3 +63,31 @@ def test_full_size_properties(dev, name):
     for a, b, ref in ((d1[0], d2[0], dx), (d1[1], d2[1], dthr), (d1[3], d2[3], dw)):
         assert torch.equal(a, b)
         assert rel_err(a, ref) <= 1e-5
+
+
+def test_offsets_beyond_32_bits(dev):
+    """2.2e9 output elements (8.8 GB): every flat offset into out / gout / records must be 64-bit. Rows from the start,
+    the middle and the end of the batch against the oracle (forward bit-exact, dX within tolerance), the leaf-weight
+    gradient of the last tree against a histogram of |margin| * g built from leafmap and marginmap."""
+    B, F, T, D, M = 220000, 64, 1000, 6, 10
+    assert B * T * M > 2 ** 31
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.randn([B, F], generator=g, device=dev)
+    thr = 6 * torch.rand([T, 2 ** D - 1], generator=g, device=dev) - 3
+    ordn = torch.randint(0, F, [T, 2 ** D - 1], generator=g, device=dev)
+    w = torch.randn([T, 2 ** D, M], generator=g, device=dev)
+    out, rec = ops.tree_forward_records(x, thr, ordn, w)
+    idx = torch.cat([torch.arange(0, 24), torch.arange(B // 2 - 12, B // 2 + 12), torch.arange(B - 24, B)]).to(dev)
+    host = [t.cpu() for t in (thr, ordn, w)]
+    assert torch.equal(out[idx].cpu(), ho.forward(x[idx].cpu(), *host, False))
+    gout = torch.randn(out.shape, generator=g, device=dev)
+    dx, dthr, _, dw = ops.tree_backward_records(rec, False, x, True, thr, True, ordn, False, w, True, gout)
+    rdx, _, _ = ho.backward(x[idx].cpu(), *host, gout[idx].cpu())
+    assert rel_err(dx[idx].cpu(), rdx) <= 1e-5
+    total = float(dx.double().abs().sum())
+    assert abs(float(dx.double().sum()) + float(dthr.double().sum())) <= 1e-5 * total
+    leaf = ops.tree_leafmap(x, thr, ordn, w)
+    margins, _ = ops.tree_marginmap(x, thr, ordn, w)
+    want = torch.zeros([2 ** D, M], dtype=torch.float64, device=dev)
+    want.index_add_(0, leaf[:, T - 1], margins[:, T - 1].abs().double()[:, None] * gout[:, T - 1, :].double())
+    assert rel_err(dw[T - 1].double().cpu(), want.cpu()) <= 1e-5
