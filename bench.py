@@ -25,8 +25,9 @@ Prints ONE JSON line. `value` is samples/s over the timed steps (wall clock betw
 `roofline` prices the dominant kernel (the forward kernel: tree_forward launches it plus a ~7 us vertex-packing
 pre-pass) against the 8 TB/s HBM peak using its algorithmic bytes (every input read once, every output written once)
 and its duration measured with events on the launch stream; `backward` and `step_hbm_frac` give the same fraction for
-the backward pass (five kernels) and for the whole step; `cpu_baseline` is the single-threaded CPU oracle timed on a
-bounded slice of the same workload on this host.
+the backward pass (five kernels) and for the whole step; `cpu_baseline` is the reference's single-threaded CPU path (its own sources
+compiled into oracle/_ref, else the oracle's restatement of them) timed on a bounded slice of the same workload on this
+host.
 """
 import argparse
 import json
@@ -85,23 +86,49 @@ def make_inputs(torch, name, dev):
 
 
 def cpu_baseline(torch, name, x, thr, ordn, w, gout, budget_rows):
-    """Single-threaded CPU oracle (a port of the reference's CPU loops) on the first rows of the same batch."""
+    """The reference's CPU path on the first rows of the same batch, one thread: its own sources as compiled into
+    oracle/_ref where that build is present (kind "reference"), else the oracle's restatement of them (kind "port");
+    with the reference build present the port is timed on half the slice as well, to show the two agree."""
     from oracle import hinge_oracle as ho
     B, F, T, depth, M, kind, _, _ = WORKLOADS[name]
     rows = min(B, budget_rows)
     xs, gs = x[:rows].cpu().contiguous(), gout[:rows].cpu().contiguous()
     tc, oc, wc = thr.cpu(), ordn.cpu(), w.cpu()
     fern = kind == "fern"
+    pre = "fern_" if fern else "tree_"
     ho.lib()
-    t0 = time.perf_counter()
-    ho.forward(xs, tc, oc, wc, fern)
-    t1 = time.perf_counter()
-    ho.backward(xs, tc, oc, wc, gs, fern=fern)
-    t2 = time.perf_counter()
-    return {"value": rows / (t2 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+    try:
+        ref = ho.reference_module()
+    except Exception:  # a build for another torch: fall back to the port
+        ref = None
+
+    def port(n):
+        t0 = time.perf_counter()
+        ho.forward(xs[:n], tc, oc, wc, fern)
+        t1 = time.perf_counter()
+        ho.backward(xs[:n], tc, oc, wc, gs[:n], fern=fern)
+        return t1 - t0, time.perf_counter() - t0
+
+    if ref is None:
+        fwd_s, all_s = port(rows)
+        extra = {}
+    else:
+        threads = torch.get_num_threads()
+        torch.set_num_threads(1)
+        try:
+            t0 = time.perf_counter()
+            getattr(ref, pre + "forward")(xs, tc, oc, wc)
+            t1 = time.perf_counter()
+            getattr(ref, pre + "backward")(xs, True, tc, True, oc, False, wc, True, gs)
+            fwd_s, all_s = t1 - t0, time.perf_counter() - t0
+        finally:
+            torch.set_num_threads(threads)
+        half = max(1, rows // 2)
+        extra = {"port_value": half / port(half)[1], "port_sample": f"the oracle's restatement on the first {half} rows"}
+    return {"value": rows / all_s, "unit": "samples/s", "cores": 1, "kind": "port" if ref is None else "reference",
             "sample": f"first {rows} of {B} rows of the same batch, all {T} trees; 1 forward + 1 backward "
-                      f"(3 gradients) = {t2 - t0:.2f} s (forward {t1 - t0:.2f} s), single thread",
-            "host_cores": os.cpu_count()}
+                      f"(3 gradients) = {all_s:.2f} s (forward {fwd_s:.2f} s), single thread",
+            "host_cores": os.cpu_count(), **extra}
 
 
 def bench_conv(torch, ops, dev, args):
