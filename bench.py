@@ -259,6 +259,8 @@ def main():
                     help="timed steps of the path not selected by --path (-1: a quarter of --steps, 0: skip)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run three 1 GiB device-to-device copies (what the HBM counters are scaled against)")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time the step replayed from a HIP graph (always done for the launch-bound c1)")
     ap.add_argument("--cpu-rows", type=int, default=32768, help="rows of the batch timed on the CPU (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -336,6 +338,30 @@ def main():
         return ((t1 - t0) * 1e3 / steps, sum(e[0].elapsed_time(e[1]) for e in ev) / steps,
                 sum(e[1].elapsed_time(e[2]) for e in ev) / steps)
 
+    def run_graph(path, steps):
+        """The same step captured once into a HIP graph and replayed: what a launch-bound shape costs without the
+        per-launch host work (the library allocates nothing and clears memory with kernels, so it can be captured)."""
+        fwd, bwd = make_step(path)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                bwd(fwd())
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            held = bwd(fwd())
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        del held
+        return (time.perf_counter() - t0) * 1e3 / steps
+
     other = "stateless" if args.path == "train" else "train"
     other_steps = max(3, args.steps // 4) if args.other_steps < 0 else args.other_steps
     o_ms = o_fwd = o_bwd = None
@@ -367,6 +393,10 @@ def main():
                      "algorithmic_bytes": bwd_bytes, "hbm_frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
         "step_hbm_frac": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
     }
+    if args.graph or name == "c1":
+        g_ms = run_graph(args.path, max(args.steps, 50))
+        result["hip_graph"] = {"ms_per_step": g_ms, "samples_per_s": B / (g_ms * 1e-3),
+                               "note": "the same step captured once with torch.cuda.CUDAGraph and replayed"}
     if o_ms is not None:
         result["other_path"] = {"path": other, "ms_per_step": o_ms, "forward_ms": o_fwd, "backward_ms": o_bwd,
                                 "samples_per_s": B / (o_ms * 1e-3)}
