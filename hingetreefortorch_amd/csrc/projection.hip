@@ -31,10 +31,21 @@ struct Fetch {
   Vec4 v[2];
 };
 
+// `full` (uniform over the workgroup): the whole 128 x 16 tile lies inside the operand and may be read as float4s, so
+// no thread needs a bounds check -- the common case, and the one whose instruction count matters.
 template <bool RED_CONTIG>
 __device__ __forceinline__ void fetch_tile(Fetch &f, const float *__restrict__ p, long long ld, int i0, int n_i,
-                                           int r0, int n_r, bool vec_ok) {
+                                           int r0, int n_r, bool vec_ok, bool full) {
   const int t = threadIdx.x;
+  if (full) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float *src = RED_CONTIG ? p + (long long)(i0 + t / 4 + 64 * h) * ld + r0 + (t % 4) * 4
+                                    : p + (long long)(r0 + t / 32 + 8 * h) * ld + i0 + (t % 32) * 4;
+      f.v[h] = *reinterpret_cast<const Vec4 *>(src);
+    }
+    return;
+  }
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     Vec4 v = {0.f, 0.f, 0.f, 0.f};
@@ -128,25 +139,21 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 
   const int per_batch = (n_r + kRed - 1) / kRed;
   const int steps = SUM_BATCHES ? per_batch * g.batches : per_batch;
+  const bool rows_a_full = g.vec_a && i0 + kTile <= n_i, rows_b_full = g.vec_b && j0 + kTile <= n_j;
   auto fetch = [&](Fetch &fa, Fetch &fb, int s) {
     const int z = SUM_BATCHES ? s / per_batch : 0;
     const int r0 = (s - z * per_batch) * kRed;
-    fetch_tile<A_RED_CONTIG>(fa, A + (long long)z * g.stride_a, g.lda, i0, n_i, r0, n_r, g.vec_a);
-    fetch_tile<B_RED_CONTIG>(fb, B + (long long)z * g.stride_b, g.ldb, j0, n_j, r0, n_r, g.vec_b);
+    const bool red_full = r0 + kRed <= n_r;
+    fetch_tile<A_RED_CONTIG>(fa, A + (long long)z * g.stride_a, g.lda, i0, n_i, r0, n_r, g.vec_a, rows_a_full && red_full);
+    fetch_tile<B_RED_CONTIG>(fb, B + (long long)z * g.stride_b, g.ldb, j0, n_j, r0, n_r, g.vec_b, rows_b_full && red_full);
   };
-  Fetch fa, fb;
-  if (steps > 0) {
-    fetch(fa, fb, 0);
-    stash_tile<A_RED_CONTIG>(As[0], fa);
-    stash_tile<B_RED_CONTIG>(Bs[0], fb);
-  }
-  __syncthreads();
-  for (int s = 0; s < steps; ++s) {
-    const int cur = s & 1;
-    if (s + 1 < steps) fetch(fa, fb, s + 1);
-    const float *as = As[cur], *bs = Bs[cur];
+  // Pipeline: while step s is multiplied out of LDS buffer s & 1, the operands of step s + 1 (fetched during step
+  // s - 1) are written to the other buffer in the middle of the multiply, and the global loads of step s + 2 are in
+  // flight. A wavefront therefore issues its LDS writes and address arithmetic in the shadow of its own MFMAs, and one
+  // barrier per step remains.
+  auto multiply = [&](const float *as, const float *bs, int kk_begin, int kk_end) {
 #pragma unroll
-    for (int kk = 0; kk < kRed; kk += 2) {
+    for (int kk = kk_begin; kk < kk_end; kk += 2) {
       const float a0 = as[(kk + lk) * kPitch + wi + lr], a1 = as[(kk + lk) * kPitch + wi + 32 + lr];
       const float b0 = bs[(kk + lk) * kPitch + wj + lr], b1 = bs[(kk + lk) * kPitch + wj + 32 + lr];
       acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
@@ -154,12 +161,33 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
       acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
       acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
     }
-    if (s + 1 < steps) {
-      stash_tile<A_RED_CONTIG>(As[cur ^ 1], fa);
-      stash_tile<B_RED_CONTIG>(Bs[cur ^ 1], fb);
-    }
-    __syncthreads();
+  };
+  Fetch fa0, fb0, fa1, fb1;
+  if (steps > 0) {
+    fetch(fa0, fb0, 0);
+    stash_tile<A_RED_CONTIG>(As[0], fa0);
+    stash_tile<B_RED_CONTIG>(Bs[0], fb0);
+    if (steps > 1) fetch(fa0, fb0, 1);
   }
+  __syncthreads();
+  // one step: `held` carries the operands of step s + 1, `next` receives those of step s + 2
+  auto step = [&](int s, Fetch &held_a, Fetch &held_b, Fetch &next_a, Fetch &next_b) {
+    const int cur = s & 1;
+    if (s + 2 < steps) fetch(next_a, next_b, s + 2);
+    multiply(As[cur], Bs[cur], 0, kRed / 2);
+    if (s + 1 < steps) {
+      stash_tile<A_RED_CONTIG>(As[cur ^ 1], held_a);
+      stash_tile<B_RED_CONTIG>(Bs[cur ^ 1], held_b);
+    }
+    multiply(As[cur], Bs[cur], kRed / 2, kRed);
+    __syncthreads();
+  };
+  int s = 0;
+  for (; s + 1 < steps; s += 2) {
+    step(s, fa0, fb0, fa1, fb1);
+    step(s + 1, fa1, fb1, fa0, fb0);
+  }
+  if (s < steps) step(s, fa0, fb0, fa1, fb1);
 
   // accumulator element e of lane l is C(row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32) of its 32 x 32 tile
 #pragma unroll
