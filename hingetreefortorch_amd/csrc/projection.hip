@@ -107,6 +107,7 @@ struct GemmArgs {
   float *C;
   long long lda, ldb, ldc, stride_a, stride_b, stride_c;
   int n_i, n_j, n_r, batches;
+  int tiles_i, tiles_j, rows_per_xcd;  // result tiles, and how many tile rows each of the 8 L2 domains takes
   bool vec_a, vec_b;
   double *stats;
   const float *bias_i, *bias_j;
@@ -117,7 +118,29 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
   __shared__ float As[2][kRed * kPitch];
   __shared__ float Bs[2][kRed * kPitch];
   const int n_i = g.n_i, n_j = g.n_j, n_r = g.n_r;
-  const int i0 = blockIdx.y * kTile, j0 = blockIdx.x * kTile;
+  // Workgroup -> result tile. Workgroups are dealt to the 8 XCDs (each with its own L2) round robin by index, so
+  // index % 8 names the L2 a workgroup will use. Every XCD takes a contiguous band of tile rows and walks it in panels
+  // of 8 tile columns, row by row inside a panel: the ~100 workgroups an XCD runs at a time then cover about 12 x 8
+  // tiles and share their 12 + 8 operand tiles through that L2, instead of each fetching its own pair.
+  int tile_i, tile_j;
+  {
+    const int xcd = blockIdx.x % kNumXCDs, slot = blockIdx.x / kNumXCDs;
+    const int row0 = xcd * g.rows_per_xcd;
+    const int rows = min(g.rows_per_xcd, g.tiles_i - row0);
+    if (rows <= 0 || slot >= rows * g.tiles_j) return;
+    constexpr int kPanel = 8;
+    const int full = g.tiles_j / kPanel;              // panels of the full width
+    int panel = slot / (rows * kPanel), rem = slot - panel * (rows * kPanel), width = kPanel;
+    if (panel >= full) {
+      panel = full;
+      rem = slot - full * (rows * kPanel);
+      width = g.tiles_j - full * kPanel;
+    }
+    const int r = rem / width;
+    tile_i = row0 + r;
+    tile_j = panel * kPanel + (rem - r * width);
+  }
+  const int i0 = tile_i * kTile, j0 = tile_j * kTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wavefront's 64 x 64 corner
   const int lr = lane & 31, lk = lane >> 5;
@@ -344,7 +367,7 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
   if (n_i <= 0 || n_j <= 0 || batches <= 0) return HT_OK;
   const long long gi = (n_i + kTile - 1) / kTile, gj = (n_j + kTile - 1) / kTile;
   const long long per_batch = (n_r + kRed - 1) / kRed;
-  if (gi > 65535 || gj > 0x7fffffffLL || n_r > 0x7fffffffLL || n_i > 0x7fffffffLL || n_j > 0x7fffffffLL ||
+  if (gi > 0x7fffffffLL || gj > 0x7fffffffLL || n_r > 0x7fffffffLL || n_i > 0x7fffffffLL || n_j > 0x7fffffffLL ||
       batches > 0x7fffffffLL || (!SUM_BATCHES && batches > 65535) || per_batch * batches > 0x7fffffffLL)
     return fail(HT_ERR_RUNTIME, "Error: matrix product too large for this build.");
   GemmArgs g;
@@ -352,11 +375,13 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
   g.lda = lda, g.ldb = ldb, g.ldc = ldc;
   g.stride_a = stride_a, g.stride_b = stride_b, g.stride_c = stride_c;
   g.n_i = int(n_i), g.n_j = int(n_j), g.n_r = int(n_r), g.batches = int(batches);
+  g.tiles_i = int(gi), g.tiles_j = int(gj), g.rows_per_xcd = int((gi + kNumXCDs - 1) / kNumXCDs);
+  const long long slots = (long long)g.rows_per_xcd * gj * kNumXCDs;
+  if (slots > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: matrix product too large for this build.");
   g.vec_a = aligned16(A, lda, stride_a), g.vec_b = aligned16(B, ldb, stride_b);
   g.stats = stats, g.bias_i = bias_i, g.bias_j = bias_j;
   hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES>),
-                     dim3((unsigned)gj, (unsigned)gi, (unsigned)(SUM_BATCHES ? 1 : batches)), dim3(kGemmThreads), 0,
-                     stream, g);
+                     dim3((unsigned)slots, 1, (unsigned)(SUM_BATCHES ? 1 : batches)), dim3(kGemmThreads), 0, stream, g);
   HT_LAUNCH_CHECK("matrix product (matrix cores)");
   return HT_OK;
 }
