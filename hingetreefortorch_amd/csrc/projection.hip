@@ -10,6 +10,8 @@
 // both operand tiles are staged in LDS reduction-major (tile[r][i], pitch 132), so the MFMA operand of lane l
 // (row l % 32, reduction index l / 32) is one conflict-free ds_read_b32, and the next step's global loads are in
 // flight while the current step is multiplied (register double buffering).
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace ht {
@@ -163,13 +165,6 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
   const int per_batch = (n_r + kRed - 1) / kRed;
   const int steps = SUM_BATCHES ? per_batch * g.batches : per_batch;
   const bool rows_a_full = g.vec_a && i0 + kTile <= n_i, rows_b_full = g.vec_b && j0 + kTile <= n_j;
-  auto fetch = [&](Fetch &fa, Fetch &fb, int s) {
-    const int z = SUM_BATCHES ? s / per_batch : 0;
-    const int r0 = (s - z * per_batch) * kRed;
-    const bool red_full = r0 + kRed <= n_r;
-    fetch_tile<A_RED_CONTIG>(fa, A + (long long)z * g.stride_a, g.lda, i0, n_i, r0, n_r, g.vec_a, rows_a_full && red_full);
-    fetch_tile<B_RED_CONTIG>(fb, B + (long long)z * g.stride_b, g.ldb, j0, n_j, r0, n_r, g.vec_b, rows_b_full && red_full);
-  };
   // Pipeline: while step s is multiplied out of LDS buffer s & 1, the operands of step s + 1 (fetched during step
   // s - 1) are written to the other buffer in the middle of the multiply, and the global loads of step s + 2 are in
   // flight. A wavefront therefore issues its LDS writes and address arithmetic in the shadow of its own MFMAs, and one
@@ -185,32 +180,58 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
       acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
     }
   };
-  Fetch fa0, fb0, fa1, fb1;
-  if (steps > 0) {
-    fetch(fa0, fb0, 0);
-    stash_tile<A_RED_CONTIG>(As[0], fa0);
-    stash_tile<B_RED_CONTIG>(Bs[0], fb0);
-    if (steps > 1) fetch(fa0, fb0, 1);
-  }
-  __syncthreads();
-  // one step: `held` carries the operands of step s + 1, `next` receives those of step s + 2
-  auto step = [&](int s, Fetch &held_a, Fetch &held_b, Fetch &next_a, Fetch &next_b) {
-    const int cur = s & 1;
-    if (s + 2 < steps) fetch(next_a, next_b, s + 2);
-    multiply(As[cur], Bs[cur], 0, kRed / 2);
-    if (s + 1 < steps) {
-      stash_tile<A_RED_CONTIG>(As[cur ^ 1], held_a);
-      stash_tile<B_RED_CONTIG>(Bs[cur ^ 1], held_b);
+  // The loop exists twice: for workgroups whose operand tiles all lie inside the matrices (FULL: exactly four
+  // unconditional float4 loads per fetch, so the wait in front of the LDS writes can leave the newest four in flight)
+  // and for the edge tiles (bounds checks, a data-dependent number of loads, hence full waits).
+  auto run = [&](auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
+    auto fetch = [&](Fetch &fa, Fetch &fb, int s) {
+      const int z = SUM_BATCHES ? s / per_batch : 0;
+      const int r0 = (s - z * per_batch) * kRed;
+      fetch_tile<A_RED_CONTIG>(fa, A + (long long)z * g.stride_a, g.lda, i0, n_i, r0, n_r, g.vec_a, FULL);
+      fetch_tile<B_RED_CONTIG>(fb, B + (long long)z * g.stride_b, g.ldb, j0, n_j, r0, n_r, g.vec_b, FULL);
+    };
+    Fetch fa0, fb0, fa1, fb1;
+    if (steps > 0) {
+      fetch(fa0, fb0, 0);
+      stash_tile<A_RED_CONTIG>(As[0], fa0);
+      stash_tile<B_RED_CONTIG>(Bs[0], fb0);
+      if (steps > 1) fetch(fa0, fb0, 1);
     }
-    multiply(As[cur], Bs[cur], kRed / 2, kRed);
     __syncthreads();
+    // one step: `held` carries the operands of step s + 1, `next` receives those of step s + 2. PREFETCH is a
+    // compile-time property of the call site: the steady-state loop always fetches (so the wait in front of the LDS
+    // writes may leave exactly those newest loads in flight), the last two steps never do.
+    auto step = [&](int s, Fetch &held_a, Fetch &held_b, Fetch &next_a, Fetch &next_b, auto prefetch_tag) {
+      constexpr bool PREFETCH = decltype(prefetch_tag)::value;
+      const int cur = s & 1;
+      if (PREFETCH) fetch(next_a, next_b, s + 2);
+      multiply(As[cur], Bs[cur], 0, kRed / 2);
+      if (PREFETCH || s + 1 < steps) {
+        stash_tile<A_RED_CONTIG>(As[cur ^ 1], held_a);
+        stash_tile<B_RED_CONTIG>(Bs[cur ^ 1], held_b);
+      }
+      multiply(As[cur], Bs[cur], kRed / 2, kRed);
+      __syncthreads();
+    };
+    int s = 0;
+    for (; s + 3 < steps; s += 2) {  // both steps have a step s + 2 to fetch
+      step(s, fa0, fb0, fa1, fb1, std::true_type{});
+      step(s + 1, fa1, fb1, fa0, fb0, std::true_type{});
+    }
+    if (s + 2 < steps) {             // one more step that fetches; the operand registers swap roles once more
+      step(s, fa0, fb0, fa1, fb1, std::true_type{});
+      step(s + 1, fa1, fb1, fa0, fb0, std::false_type{});
+      step(s + 2, fa0, fb0, fa1, fb1, std::false_type{});
+    } else {
+      if (s < steps) step(s, fa0, fb0, fa1, fb1, std::false_type{});
+      if (s + 1 < steps) step(s + 1, fa1, fb1, fa0, fb0, std::false_type{});
+    }
   };
-  int s = 0;
-  for (; s + 1 < steps; s += 2) {
-    step(s, fa0, fb0, fa1, fb1);
-    step(s + 1, fa1, fb1, fa0, fb0);
-  }
-  if (s < steps) step(s, fa0, fb0, fa1, fb1);
+  if (rows_a_full && rows_b_full && n_r % kRed == 0)
+    run(std::true_type{});
+  else
+    run(std::false_type{});
 
   // accumulator element e of lane l is C(row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32) of its 32 x 32 tile
 #pragma unroll
