@@ -247,12 +247,100 @@ def bench_projection(torch, ops, dev, args):
     }
 
 
+def _timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def bench_mix(torch, ops, dev, args):
+    """The forest -> linear operators (tree_fused_linear_forward / backward) at the headline forest shape with a
+    10-class linear head: 65536 x 1024 inputs, 1000 trees of depth 10 with one output per leaf, mixed down to 10
+    channels."""
+    B, F, T, depth, O = 65536, 1024, 1000, 10, 10
+    V, L = 2 ** depth - 1, 2 ** depth
+    g = torch.Generator().manual_seed(6112)
+    thr = 6.0 * torch.rand([T, V], generator=g) - 3.0
+    ordn = torch.randint(0, F, [T, V], generator=g, dtype=torch.int64)
+    w = torch.randn([T, L], generator=g)
+    ops.tree_fix_thresholds(thr, ordn, w)
+    lin = (torch.randn([O, T], generator=g) / T ** 0.5).to(dev)
+    bias = torch.randn([O], generator=g).to(dev)
+    thr, ordn, w = thr.to(dev), ordn.to(dev), w.to(dev)
+    gg = torch.Generator(device=dev).manual_seed(6113)
+    x = torch.randn([B, F], generator=gg, device=dev)
+    gout = torch.randn([B, O], generator=gg, device=dev)
+    # the training path of the autograd function: the forward keeps the forest output and the walk records
+    fwd_ms = _timed(torch, lambda: ops.tree_fused_linear_forward_records(x, thr, ordn, w, lin, bias), args.steps,
+                    args.warmup)
+    _, f, records = ops.tree_fused_linear_forward_records(x, thr, ordn, w, lin, bias)
+    bwd_ms = _timed(torch, lambda: ops.tree_fused_linear_backward_records((f, records), False, x, True, thr, True, ordn,
+                                                                           False, w, True, lin, True, bias, True, gout),
+                    args.steps, args.warmup)
+    # ... and the reference's stateless operator pair, whose backward computes the forest again
+    s_fwd = _timed(torch, lambda: ops.tree_fused_linear_forward(x, thr, ordn, w, lin, bias), args.steps, args.warmup)
+    s_bwd = _timed(torch, lambda: ops.tree_fused_linear_backward(x, True, thr, True, ordn, False, w, True, lin, True,
+                                                                  bias, True, gout), args.steps, args.warmup)
+    plain_fwd = _timed(torch, lambda: ops.tree_forward(x, thr, ordn, w), args.steps, args.warmup)
+    ms = fwd_ms + bwd_ms
+    # every input read once, every output written once (the forest's [B, T] intermediate is not part of the interface)
+    fwd_bytes = 4 * (B * F + T * V + T * L + O * T + O + B * O) + 8 * T * V
+    bwd_bytes = fwd_bytes + 4 * (B * F + T * V + T * L + O * T + O)
+    return {
+        "metric": "fwd+bwd samples/s (forest -> linear: B=65536,F=1024,T=1000,D=10 -> 10 channels)",
+        "value": B / (ms * 1e-3), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "f1: forest -> linear forward + backward (all five gradients) as HingeTreeFusedLinear runs them, "
+                               "x~N(0,1) [65536,1024], 1000 trees of depth 10, one output per leaf, linear head "
+                               "[10,1000] with bias", "B": B, "F": F, "T": T, "depth": depth, "out_channels": O},
+        "forward": {"ms": fwd_ms, "of_which_forest_ms": plain_fwd}, "backward": {"ms": bwd_ms},
+        "other_path": {"path": "stateless", "forward_ms": s_fwd, "backward_ms": s_bwd},
+        "roofline": {"bound": "hbm", "kernel": "forward_rows_kernel + gemm_kernel (forest, then the mix over trees)",
+                     "achieved": fwd_bytes / (fwd_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "algorithmic_bytes": fwd_bytes,
+                     "note": "interface bytes only; the operator also writes and re-reads the 262 MB forest output"},
+        "backward_hbm_frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+    }
+
+
+def bench_tiles(torch, ops, dev, args):
+    """contract / expand on the segmentation shape: leaf patches [8,100,64,64,8,8] <-> images [8,100,512,512]."""
+    B, C, H, W, P = 8, 100, 512, 512, 8
+    gg = torch.Generator(device=dev).manual_seed(6113)
+    image = torch.randn([B, C, H, W], generator=gg, device=dev)
+    tiles = ops.contract(image, [P, P], [0, 0])
+    c_ms = _timed(torch, lambda: ops.contract(image, [P, P], [0, 0]), args.steps, args.warmup)
+    e_ms = _timed(torch, lambda: ops.expand(tiles, [0, 0]), args.steps, args.warmup)
+    nbytes = 2 * image.numel() * 4   # read once, written once
+    ms = c_ms + e_ms
+    return {
+        "metric": "contract + expand GB/s (tiles [8,100,64,64,8,8] <-> images [8,100,512,512])",
+        "value": 2 * nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "f3: one contract and one expand of an 839 MB float32 image batch, window 8 x 8, no padding"},
+        "contract": {"ms": c_ms, "gbps": nbytes / (c_ms * 1e-3) / 1e9}, "expand": {"ms": e_ms, "gbps": nbytes / (e_ms * 1e-3) / 1e9},
+        "roofline": {"bound": "hbm", "kernel": "tile_permute_kernel", "achieved": 2 * nbytes / (ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": 2 * nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": None, "algorithmic_bytes": nbytes},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "c5"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "c5", "f1", "f3"])
     ap.add_argument("--mode", default="atomic", choices=["atomic", "deterministic"])
     ap.add_argument("--path", default="train", choices=["train", "stateless"])
     ap.add_argument("--other-steps", type=int, default=-1,
@@ -288,6 +376,12 @@ def main():
         return
     if name == "c5":
         print(json.dumps(bench_projection(torch, ops, dev, args)), flush=True)
+        return
+    if name == "f1":
+        print(json.dumps(bench_mix(torch, ops, dev, args)), flush=True)
+        return
+    if name == "f3":
+        print(json.dumps(bench_tiles(torch, ops, dev, args)), flush=True)
         return
     B, F, T, depth, M, kind, _, desc = WORKLOADS[name]
     x, thr, ordn, w, gout = make_inputs(torch, name, dev)

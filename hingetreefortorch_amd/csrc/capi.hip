@@ -297,10 +297,10 @@ int ht_tree_mix_forward(int64_t B, int64_t T, int64_t O, int64_t R, const float 
 }
 
 int ht_tree_mix_backward(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin, const float *g,
-                         float *h, float *dlin, void *stream) {
+                         float *h, float *dlin, int deterministic, void *stream) {
   if (B < 0 || T < 0 || O < 0 || R < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
   if (B * O * R > 0 && (!g || (h && !lin) || (dlin && !f))) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
-  return mix_backward(B, T, O, R, f, lin, g, h, dlin, static_cast<hipStream_t>(stream));
+  return mix_backward(B, T, O, R, f, lin, g, h, dlin, deterministic != 0, static_cast<hipStream_t>(stream));
 }
 
 int ht_contract(const ht_tile_shape *s, const void *image, void *tiles, void *stream) {

@@ -117,7 +117,7 @@ int conv_output_size(const ht_conv_shape &s, int64_t *out_size);
 int mix_forward(long long B, long long T, long long O, long long R, const float *f, const float *lin,
                 const float *bias, float *out, hipStream_t stream);
 int mix_backward(long long B, long long T, long long O, long long R, const float *f, const float *lin, const float *g,
-                 float *h, float *dlin, hipStream_t stream);
+                 float *h, float *dlin, bool deterministic, hipStream_t stream);
 
 // Tile <-> image permutation (expand.hip).
 int tile_contract(const ht_tile_shape *s, const void *in, void *out, hipStream_t stream);

@@ -110,6 +110,7 @@ struct GemmArgs {
   long long lda, ldb, ldc, stride_a, stride_b, stride_c;
   int n_i, n_j, n_r, batches;
   int tiles_i, tiles_j, rows_per_xcd;  // result tiles, and how many tile rows each of the 8 L2 domains takes
+  int splits;                          // > 1: blockIdx.y takes a share of the reduction and adds into a zeroed C
   bool vec_a, vec_b;
   double *stats;
   const float *bias_i, *bias_j;
@@ -163,7 +164,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
       for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
   const int per_batch = (n_r + kRed - 1) / kRed;
-  const int steps = SUM_BATCHES ? per_batch * g.batches : per_batch;
+  // this workgroup's share of the reduction steps (all of them unless the launch splits the reduction)
+  const int all_steps = SUM_BATCHES ? per_batch * g.batches : per_batch;
+  const int chunk = (all_steps + g.splits - 1) / g.splits;
+  const int step0 = blockIdx.y * chunk;
+  const int steps = max(0, min(chunk, all_steps - step0));
+  if (g.splits > 1 && steps == 0) return;
   const bool rows_a_full = g.vec_a && i0 + kTile <= n_i, rows_b_full = g.vec_b && j0 + kTile <= n_j;
   // Pipeline: while step s is multiplied out of LDS buffer s & 1, the operands of step s + 1 (fetched during step
   // s - 1) are written to the other buffer in the middle of the multiply, and the global loads of step s + 2 are in
@@ -186,8 +192,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
   auto run = [&](auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
     auto fetch = [&](Fetch &fa, Fetch &fb, int s) {
-      const int z = SUM_BATCHES ? s / per_batch : 0;
-      const int r0 = (s - z * per_batch) * kRed;
+      const int gs = s + step0;
+      const int z = SUM_BATCHES ? gs / per_batch : 0;
+      const int r0 = (gs - z * per_batch) * kRed;
       fetch_tile<A_RED_CONTIG>(fa, A + (long long)z * g.stride_a, g.lda, i0, n_i, r0, n_r, g.vec_a, FULL);
       fetch_tile<B_RED_CONTIG>(fb, B + (long long)z * g.stride_b, g.ldb, j0, n_j, r0, n_r, g.vec_b, FULL);
     };
@@ -237,7 +244,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
     const int j = j0 + wj + 32 * b + lr;
-    const float bj = (g.bias_j && j < n_j) ? g.bias_j[j] : 0.f;
+    const bool first = blockIdx.y == 0;  // the biases belong to one share of a split reduction only
+    const float bj = (g.bias_j && first && j < n_j) ? g.bias_j[j] : 0.f;
     double s1 = 0.0, s2 = 0.0;
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
@@ -246,9 +254,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         const int i = i0 + wi + 32 * a + 8 * (e / 4) + 4 * lk + (e % 4);
         if (i < n_i && j < n_j) {
           float v = acc[a][b][e];
-          if (g.bias_i) v += g.bias_i[i];
+          if (g.bias_i && first) v += g.bias_i[i];
           v += bj;
-          C[(long long)i * g.ldc + j] = v;
+          if (g.splits > 1)
+            atomicAdd(C + (long long)i * g.ldc + j, v);
+          else
+            C[(long long)i * g.ldc + j] = v;
           if (STATS) {
             s1 += double(v);
             s2 += double(v) * double(v);
@@ -384,7 +395,7 @@ template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS, bool SUM_BATCHES>
 int launch_gemm_batched(const float *A, long long lda, long long stride_a, const float *B, long long ldb,
                         long long stride_b, float *C, long long ldc, long long stride_c, long long n_i, long long n_j,
                         long long n_r, long long batches, double *stats, const float *bias_i, const float *bias_j,
-                        hipStream_t stream) {
+                        hipStream_t stream, bool allow_split = false) {
   if (n_i <= 0 || n_j <= 0 || batches <= 0) return HT_OK;
   const long long gi = (n_i + kTile - 1) / kTile, gj = (n_j + kTile - 1) / kTile;
   const long long per_batch = (n_r + kRed - 1) / kRed;
@@ -401,8 +412,24 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
   if (slots > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: matrix product too large for this build.");
   g.vec_a = aligned16(A, lda, stride_a), g.vec_b = aligned16(B, ldb, stride_b);
   g.stats = stats, g.bias_i = bias_i, g.bias_j = bias_j;
+  // A product with few result tiles and a long reduction (dLin of a narrow linear head: 10 x 1000 from 65536 rows)
+  // would leave most of the device idle: the reduction is then split over blockIdx.y and the shares are added into
+  // the zeroed result with float atomics (a few thousand elements times the number of shares).
+  g.splits = 1;
+  const long long all_steps = SUM_BATCHES ? per_batch * batches : per_batch;
+  if (allow_split && !STATS && ldc == n_j && (SUM_BATCHES || batches == 1) && gi * gj < kNumCUs && all_steps >= 64) {
+    long long want = (2 * kNumCUs + gi * gj - 1) / (gi * gj);
+    if (want > all_steps / 16) want = all_steps / 16;
+    if (want > 65535) want = 65535;
+    if (want > 1) {
+      g.splits = int(want);
+      int rc = zero_fill(C, size_t(n_i) * size_t(n_j) * sizeof(float), stream);
+      if (rc != HT_OK) return rc;
+    }
+  }
   hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES>),
-                     dim3((unsigned)slots, 1, (unsigned)(SUM_BATCHES ? 1 : batches)), dim3(kGemmThreads), 0, stream, g);
+                     dim3((unsigned)slots, (unsigned)g.splits, (unsigned)(SUM_BATCHES ? 1 : batches)), dim3(kGemmThreads),
+                     0, stream, g);
   HT_LAUNCH_CHECK("matrix product (matrix cores)");
   return HT_OK;
 }
@@ -476,7 +503,7 @@ int mix_forward(long long B, long long T, long long O, long long R, const float 
 }
 
 int mix_backward(long long B, long long T, long long O, long long R, const float *f, const float *lin, const float *g,
-                 float *h, float *dlin, hipStream_t stream) {
+                 float *h, float *dlin, bool deterministic, hipStream_t stream) {
   int rc;
   if (h) {
     if (R == 1)  // h [B x T] = g [B x O] * lin [O x T]
@@ -491,10 +518,10 @@ int mix_backward(long long B, long long T, long long O, long long R, const float
   if (dlin) {
     if (R == 1)  // dlin [O x T] = g^T [O x B] * f [B x T]
       rc = launch_gemm_batched<false, false, false, false>(g, O, 0, f, T, 0, dlin, T, 0, O, T, B, 1, nullptr, nullptr,
-                                                           nullptr, stream);
+                                                           nullptr, stream, !deterministic);
     else  // dlin [O x T] = sum_b g_b [O x R] * f_b [T x R]^T
       rc = launch_gemm_batched<true, true, false, true>(g, R, O * R, f, R, T * R, dlin, T, 0, O, T, R, B, nullptr,
-                                                        nullptr, nullptr, stream);
+                                                        nullptr, nullptr, stream, !deterministic);
     if (rc != HT_OK) return rc;
   }
   return HT_OK;

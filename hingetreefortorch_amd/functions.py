@@ -153,17 +153,29 @@ class _FusedLinearFunction(torch.autograd.Function):
 
     @staticmethod
     def _forward(cls, ctx, inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias):
-        ctx.save_for_backward(inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias)
-        return getattr(_ops, f"{cls._prefix}_fused_linear_forward")(inData, inThresholds, inOrdinals, inWeights,
-                                                                   inLinearWeights, inLinearBias)
+        args = (inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias)
+        # when a backward pass will follow, the forest's output and walk records are kept for it (the reference's
+        # backward computes the forest again, hingetree_fused_linear.cpp:200-412; same gradients)
+        ctx.kept = 0
+        if any(ctx.needs_input_grad) and inData.is_cuda:
+            out, f, records = getattr(_ops, f"{cls._prefix}_fused_linear_forward_records")(*args)
+            ctx.kept = 1 if records is None else 2
+            ctx.save_for_backward(*args, f, *([] if records is None else [records]))
+            return out
+        ctx.save_for_backward(*args)
+        return getattr(_ops, f"{cls._prefix}_fused_linear_forward")(*args)
 
     @staticmethod
     def _backward(cls, ctx, outDataGrad):
-        inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias = ctx.saved_tensors
+        inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias = ctx.saved_tensors[:6]
         need = ctx.needs_input_grad
+        args = (inData, need[0], inThresholds, need[1], inOrdinals, need[2], inWeights, need[3], inLinearWeights,
+                need[4], inLinearBias, need[5], outDataGrad.contiguous())
+        if ctx.kept:
+            state = (ctx.saved_tensors[6], ctx.saved_tensors[7] if ctx.kept == 2 else None)
+            return tuple(getattr(_ops, f"{cls._prefix}_fused_linear_backward_records")(state, _is_deterministic(), *args))
         name = f"{cls._prefix}_fused_linear_backward" + ("_deterministic" if _is_deterministic() else "")
-        return tuple(getattr(_ops, name)(inData, need[0], inThresholds, need[1], inOrdinals, need[2], inWeights, need[3],
-                                         inLinearWeights, need[4], inLinearBias, need[5], outDataGrad.contiguous()))
+        return tuple(getattr(_ops, name)(*args))
 
 
 class HingeTreeFusedLinear(_FusedLinearFunction):

@@ -121,23 +121,31 @@ def _mix_sizes(inData, inWeights, inLinearWeights):
     return B, T, O, R, [B, O] + list(inData.shape[2:]) + list(inWeights.shape[2:])
 
 
-def _fused_linear_forward(kind, inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias):
+def _fused_linear_forward(kind, inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias,
+                          keep=False):
     """out[b, o, ...] = inLinearBias[o] + sum_t inLinearWeights[o, t] * forest(inData)[b, t, ...]
-    (hingetree_fused_linear.cpp:75-198): the forest kernel followed by a matrix-core product over the tree axis."""
+    (hingetree_fused_linear.cpp:75-198): the forest kernel followed by a matrix-core product over the tree axis.
+    keep: also return (forest output, walk records or None) for `_fused_linear_backward(..., state=...)`."""
     _fused_linear_checks(inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias)
-    f = _forward(kind, inData, inThresholds, inOrdinals, inWeights)
+    records = None
+    if keep:
+        f, records = _forward_records(kind, inData, inThresholds, inOrdinals, inWeights)
+    else:
+        f = _forward(kind, inData, inThresholds, inOrdinals, inWeights)
     B, T, O, R, out_sizes = _mix_sizes(inData, inWeights, inLinearWeights)
     with torch.cuda.device(inData.device):
         out = torch.empty(out_sizes, dtype=inData.dtype, device=inData.device)
         L.check(L.load().ht_tree_mix_forward(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(inLinearBias), _ptr(out),
                                              _stream(inData.device)))
-    return out
+    return (out, f, records) if keep else out
 
 
 def _fused_linear_backward(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals,
                            bInOrdinalsGrad, inWeights, bInWeightsGrad, inLinearWeights, bInLinearWeightsGrad,
-                           inLinearBias, bInLinearBiasGrad, outDataGrad):
-    """[dData, dThresholds, None, dWeights, dLinearWeights, dLinearBias] (hingetree_fused_linear.cpp:200-412)."""
+                           inLinearBias, bInLinearBiasGrad, outDataGrad, state=None):
+    """[dData, dThresholds, None, dWeights, dLinearWeights, dLinearBias] (hingetree_fused_linear.cpp:200-412).
+    state: (forest output, walk records or None) kept by `_fused_linear_forward(..., keep=True)`; without it the forest
+    output is computed again and the forest backward walks again, like the reference's operator."""
     if bInOrdinalsGrad:
         _runtime("Error: Gradient on inOrdinals is requested, but inOrdinals never has a gradient.")
     _fused_linear_checks(inData, inThresholds, inOrdinals, inWeights, inLinearWeights, inLinearBias, outDataGrad)
@@ -148,15 +156,23 @@ def _fused_linear_backward(kind, mode, inData, bInDataGrad, inThresholds, bInThr
     need_forest = bInDataGrad or bInThresholdsGrad or bInWeightsGrad
     lib = L.load()
     with torch.cuda.device(inData.device):
-        f = _forward(kind, inData, inThresholds, inOrdinals, inWeights) if bInLinearWeightsGrad else None
+        if state is not None:
+            f = state[0]
+        else:
+            f = _forward(kind, inData, inThresholds, inOrdinals, inWeights) if bInLinearWeightsGrad else None
         h = torch.empty([B, T] + list(inData.shape[2:]) + list(inWeights.shape[2:]), dtype=inData.dtype,
                         device=inData.device) if need_forest else None
         dlin = torch.empty_like(inLinearWeights) if bInLinearWeightsGrad else None
         if h is not None or dlin is not None:
             L.check(lib.ht_tree_mix_backward(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(outDataGrad), _ptr(h),
-                                             _ptr(dlin), _stream(inData.device)))
+                                             _ptr(dlin), int(mode == L.HT_BACKWARD_DETERMINISTIC),
+                                             _stream(inData.device)))
         grads[4] = dlin
-        if need_forest:
+        if need_forest and state is not None and state[1] is not None:
+            grads[0], grads[1], _, grads[3] = _backward_records(kind, mode, state[1], inData, bInDataGrad, inThresholds,
+                                                                bInThresholdsGrad, inOrdinals, False, inWeights,
+                                                                bInWeightsGrad, h)
+        elif need_forest:
             grads[0], grads[1], _, grads[3] = _backward(kind, mode, inData, bInDataGrad, inThresholds,
                                                         bInThresholdsGrad, inOrdinals, False, inWeights, bInWeightsGrad, h)
         if bInLinearBiasGrad:  # a plain sum, like the reference's outDataGrad.sum(...) (hingetree_fused_linear.cpp:388)
@@ -180,9 +196,29 @@ def fern_fused_linear_backward(*args):
     return _fused_linear_backward(L.HT_FERN, L.HT_BACKWARD_ATOMIC, *args)
 
 
+def tree_fused_linear_forward_records(*args):
+    """(out, forest output, walk records or None): the forward of the training path; not part of the reference."""
+    return _fused_linear_forward(L.HT_TREE, *args, keep=True)
+
+
+def fern_fused_linear_forward_records(*args):
+    return _fused_linear_forward(L.HT_FERN, *args, keep=True)
+
+
+def tree_fused_linear_backward_records(state, deterministic, *args):
+    mode = L.HT_BACKWARD_DETERMINISTIC if deterministic else L.HT_BACKWARD_ATOMIC
+    return _fused_linear_backward(L.HT_TREE, mode, *args, state=state)
+
+
+def fern_fused_linear_backward_records(state, deterministic, *args):
+    mode = L.HT_BACKWARD_DETERMINISTIC if deterministic else L.HT_BACKWARD_ATOMIC
+    return _fused_linear_backward(L.HT_FERN, mode, *args, state=state)
+
+
 def tree_fused_linear_backward_deterministic(*args):
-    """No counterpart in the reference (its fused-linear operators have no deterministic form on the GPU): the linear
-    mix here uses no atomics, so the deterministic forest backward makes the whole operator reproducible."""
+    """No counterpart in the reference (its fused-linear operators have no deterministic form on the GPU): the forest
+    part uses the deterministic forest backward and the linear mix runs without atomics (dLinearWeights of a narrow
+    head then takes its unsplit, slower product), so the whole operator is reproducible."""
     return _fused_linear_backward(L.HT_TREE, L.HT_BACKWARD_DETERMINISTIC, *args)
 
 

@@ -144,11 +144,13 @@ int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, cons
  *   forward : out [B, O, R] = bias[o] + sum_t lin[o, t] * f[b, t, r]           (bias may be NULL)
  *   backward: h [B, T, R]   = sum_o lin[o, t] * g[b, o, r]   -> upstream gradient for ht_forest_backward (may be NULL)
  *             dlin [O, T]   = sum_{b, r} g[b, o, r] * f[b, t, r]                (may be NULL)
- * Both run on the matrix cores and are deterministic (no atomics). */
+ * Both run on the matrix cores. The forward and h use no atomics. dlin of a narrow head has few result tiles and a
+ * long reduction: unless `deterministic` is set its reduction is split over workgroups whose shares meet in float
+ * atomics (an order of magnitude faster, not bit-reproducible run to run). */
 int ht_tree_mix_forward(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin,
                         const float *bias, float *out, void *stream);
 int ht_tree_mix_backward(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin, const float *g,
-                         float *h, float *dlin, void *stream);
+                         float *h, float *dlin, int deterministic, void *stream);
 
 /* ---- contract / expand -----------------------------------------------------------------------------------------------
  * Replace contract2d/3d and expand2d/3d of the reference (expand.cpp:37-227 on the CPU, expand_gpu.cu:110-172 on the

@@ -76,6 +76,15 @@ def _check(dev, fern, x, thr, ordn, w, lin, bias, gout, want=None):
                 slack = rel_err(want[key].double(), exact[key])
                 assert rel_err(got.cpu().double(), exact[key]) <= TOL, (name, key, "fp64")
             assert rel_err(got.cpu(), want[key]) <= TOL + slack, (name, key)
+    # the training path: forest output and walk records kept by the forward pass
+    out2, f, records = getattr(ops, pre + "fused_linear_forward_records")(*d[:6])
+    assert torch.equal(out2, out)
+    for det in (False, True):
+        grads = getattr(ops, pre + "fused_linear_backward_records")((f, records), det, d[0], True, d[1], True, d[2], False,
+                                                                    d[3], True, d[4], True, d[5], True, d[6])
+        for got, key in zip(grads[:2] + grads[3:], ("dx", "dthr", "dw", "dlin", "dbias")):
+            slack = rel_err(want[key].double(), exact[key]) if key in exact else 0.0
+            assert rel_err(got.cpu(), want[key]) <= TOL + slack, ("records", det, key)
 
 
 @pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
