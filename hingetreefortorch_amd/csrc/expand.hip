@@ -17,6 +17,13 @@ struct TileGeom {
   int size[3], tiles[3], win[3], pad[3];
 };
 
+// 16 opaque bytes: where the innermost window extent, padding and image extent are all whole multiples of 16 bytes, a
+// run of that many consecutive innermost elements is consecutive in both layouts and lies wholly inside or wholly
+// outside, so the permutation can move such runs as single elements of a geometry with the innermost extents divided.
+struct alignas(16) Word16 {
+  uint32_t w[4];
+};
+
 template <typename Word, bool EXPAND>
 __global__ __launch_bounds__(256) void tile_permute_kernel(TileGeom g, const Word *__restrict__ in,
                                                            Word *__restrict__ out, long long total) {
@@ -24,7 +31,7 @@ __global__ __launch_bounds__(256) void tile_permute_kernel(TileGeom g, const Wor
   const long long wsz = (long long)g.win[0] * g.win[1] * g.win[2];
   const long long tiled = (long long)g.tiles[0] * g.tiles[1] * g.tiles[2] * wsz;
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
-    Word v = Word(0);
+    Word v = Word{};
     if (EXPAND) {
       const long long plane = i / image;
       long long r = i - plane * image;
@@ -74,8 +81,23 @@ template <bool EXPAND>
 int launch_permute(const TileGeom &g, int elem_size, const void *in, void *out, hipStream_t stream) {
   const long long image = (long long)g.size[0] * g.size[1] * g.size[2];
   const long long tiled = (long long)g.tiles[0] * g.tiles[1] * g.tiles[2] * g.win[0] * g.win[1] * g.win[2];
-  const long long total = g.planes * (EXPAND ? image : tiled);
+  long long total = g.planes * (EXPAND ? image : tiled);
   if (total <= 0) return HT_OK;
+  const int per16 = 16 / elem_size;  // elements in 16 bytes
+  if (per16 > 1 && g.size[2] % per16 == 0 && g.win[2] % per16 == 0 && g.pad[2] % per16 == 0 &&
+      reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    TileGeom wide = g;
+    wide.size[2] /= per16;
+    wide.win[2] /= per16;
+    wide.pad[2] /= per16;
+    total /= per16;
+    long long blocks = (total + 255) / 256;
+    if (blocks > 64 * kNumCUs) blocks = 64 * kNumCUs;
+    hipLaunchKernelGGL((tile_permute_kernel<Word16, EXPAND>), dim3((unsigned)blocks), dim3(256), 0, stream, wide,
+                       static_cast<const Word16 *>(in), static_cast<Word16 *>(out), total);
+    HT_LAUNCH_CHECK((EXPAND ? "expand (16-byte runs)" : "contract (16-byte runs)"));
+    return HT_OK;
+  }
   long long blocks = (total + 255) / 256;
   if (blocks > 64 * kNumCUs) blocks = 64 * kNumCUs;
 #define HT_PERMUTE(Word)                                                                                        \

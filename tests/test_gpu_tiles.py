@@ -16,7 +16,9 @@ pytestmark = pytest.mark.gpu
 
 CASES = [([2, 3, 8, 12], [2, 3], [0, 0]), ([1, 2, 7, 9], [3, 2], [1, 2]), ([2, 1, 5, 6, 7], [2, 3, 2], [1, 0, 1]),
          ([1, 1, 4, 4], [4, 4], [2, 2]), ([1, 2, 9, 9], [4, 5], [3, 1]), ([1, 1, 3, 10, 4], [3, 4, 1], [0, 3, 2]),
-         ([3, 5, 64, 48], [8, 8], [0, 0])]
+         ([3, 5, 64, 48], [8, 8], [0, 0]),
+         # innermost window, padding and image extent whole multiples of 16 bytes: moved as 16-byte runs
+         ([2, 2, 16, 32], [4, 16], [2, 16]), ([1, 2, 6, 8, 16], [2, 4, 8], [1, 0, 4]), ([2, 1, 9, 24], [3, 8], [1, 8])]
 DTYPES = [torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64, torch.float32, torch.float64]
 
 
@@ -31,6 +33,20 @@ def test_contract_expand_bit_exact(dev, case, dtype):
     want_i = ho.expand(want_t, padding)
     got_i = ops.expand(got_t, padding)
     assert got_i.shape == want_i.shape and torch.equal(got_i.cpu(), want_i)
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.float32], ids=["uint8", "int16", "float32"])
+def test_tiles_of_an_offset_view(dev, dtype):
+    """A contiguous view that starts in the middle of an allocation is not aligned to 16 bytes: the run-wise path must
+    not be taken for it (or must cope), whatever the geometry allows."""
+    base = (100.0 * torch.rand([3 * 16 * 32 + 3], generator=torch.Generator().manual_seed(2))).to(dtype).to(dev)
+    for off in (0, 1, 3):
+        x = base[off:off + 3 * 16 * 32].view(1, 3, 16, 32)
+        tiles = ops.contract(x, [4, 16], [0, 16])
+        assert torch.equal(tiles.cpu(), ho.contract(x.cpu(), [4, 16], [0, 16]))
+        room = torch.empty([tiles.numel() + off], dtype=dtype, device=dev)
+        t2 = room[off:].view(tiles.shape).copy_(tiles)          # the same tiles, stored off elements into a buffer
+        assert torch.equal(ops.expand(t2, [0, 16]).cpu(), ho.expand(t2.cpu(), [0, 16]))
 
 
 GOLD = sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "tiles*.npz")))
