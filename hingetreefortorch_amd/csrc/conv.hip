@@ -195,13 +195,13 @@ __global__ __launch_bounds__(kConvThreads) void conv_backward_kernel(ConvGeom g,
 struct ConvTile {
   int H, W, OH, OW;
   int kh, kw, sy, sx, py, px, dy, dx;
-  int TY, TX, log2_tx;  // output tile, TY * TX == kConvThreads
+  int TY, TX, log2_tx;  // output tile, TY * TX == threads of the workgroup
   int IH, IW, TSZ;      // input region of a tile, TSZ = IH * IW
   int tiles_y, tiles_x;
   int taps;
 };
 
-static bool make_tile(const ConvGeom &g, ConvTile *t) {
+static bool make_tile(const ConvGeom &g, ConvTile *t, int threads = kConvThreads) {
   if (g.nd > 2) return false;
   const int a = g.nd == 2 ? 0 : -1;  // index of the row dimension, none for 1-d
   t->H = a < 0 ? 1 : g.size[0];
@@ -217,11 +217,11 @@ static bool make_tile(const ConvGeom &g, ConvTile *t) {
   t->sx = g.str[c];
   t->px = g.pad[c];
   t->dx = g.dil[c];
-  int tx = kConvThreads;  // widest power-of-two tile row that the output needs
+  int tx = threads;  // widest power-of-two tile row that the output needs
   while (tx > 32 && tx / 2 >= t->OW) tx /= 2;
   if (t->OH > 1 && tx > 32) tx = 32;
   t->TX = tx;
-  t->TY = kConvThreads / tx;
+  t->TY = threads / tx;
   t->log2_tx = 0;
   while ((1 << t->log2_tx) < tx) ++t->log2_tx;
   t->IH = (t->TY - 1) * t->sy + (t->kh - 1) * t->dy + 1;
@@ -243,7 +243,7 @@ __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restric
   const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
   const long long chan = (long long)g.H * g.W;
   const Real *img = x + b * C * chan;
-  for (int e = threadIdx.x; e < g.TSZ; e += kConvThreads) {
+  for (int e = threadIdx.x; e < g.TSZ; e += int(blockDim.x)) {
     const int iy = e / g.IW, ix = e - iy * g.IW;
     const int gy = iy0 + iy, gx = ix0 + ix;
     Real *q = tile + e;
@@ -269,7 +269,7 @@ __device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, co
                                                  int j, const Real *__restrict__ thr, const int64_t *__restrict__ ord,
                                                  const Real *__restrict__ w, int *special) {
   const long long first = (long long)j * C * V;
-  for (int i = threadIdx.x; i < C * V; i += kConvThreads) {
+  for (int i = threadIdx.x; i < C * V; i += int(blockDim.x)) {
     const int tap = clamp_ordinal(ord[first + i], g.taps);
     const int ky = tap / g.kw, kx = tap - ky * g.kw;
     Node<Real> n;
@@ -280,7 +280,7 @@ __device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, co
   }
   if (wl) {
     const long long wfirst = (long long)j * C * LM;
-    for (int i = threadIdx.x; i < C * LM; i += kConvThreads) wl[i] = w[wfirst + i];
+    for (int i = threadIdx.x; i < C * LM; i += int(blockDim.x)) wl[i] = w[wfirst + i];
   }
 }
 
@@ -547,6 +547,128 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
       if (acc_t[i] != 0.0) atomicAdd(dthr + (long long)j * C * V + i, Real(acc_t[i]));
 }
 
+// All three gradients from ONE walk per (position, out channel, channel), for callers that want dX together with dThr
+// or dW: tile-stationary like the dX kernel, with the fp64 tables of the current out channel's C trees beside the dX
+// image. The tree tables are flushed to memory with atomics after each out channel (C * (V + L * M) cells per NT
+// positions x C walks), which is what the second walk of the two-kernel form is traded for; workgroups start at
+// different out channels so that those atomics spread over all trees' addresses. NT = 512: the larger tile halves the
+// flushes and the tree staging per walk, and one workgroup fills a CU's wavefront slots the way two smaller ones do.
+template <typename Real, bool FERN, int NT>
+__global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, ConvLds lay, int C, int Cout, int depth,
+                                                                 int V, int L, int M, int j_per,
+                                                                 const Real *__restrict__ x,
+                                                                 const Real *__restrict__ thr,
+                                                                 const int64_t *__restrict__ ord,
+                                                                 const Real *__restrict__ w,
+                                                                 const Real *__restrict__ gout, Real *dx, Real *dthr,
+                                                                 Real *dw) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *tile = reinterpret_cast<Real *>(smem + lay.tile);
+  double *acc = reinterpret_cast<double *>(smem + lay.acc_x);
+  Node<Real> *nodes = reinterpret_cast<Node<Real> *>(smem + lay.nodes);
+  Real *wl = reinterpret_cast<Real *>(smem + lay.wl);
+  double *acc_w = reinterpret_cast<double *>(smem + lay.acc_w);
+  double *acc_t = reinterpret_cast<double *>(smem + lay.acc_t);
+  const int tyi = blockIdx.x / g.tiles_x, txi = blockIdx.x - tyi * g.tiles_x;
+  const long long b = blockIdx.z;
+  int *special = reinterpret_cast<int *>(smem + lay.flag);
+  const int LM = L * M;
+  load_conv_tile<Real>(tile, x, g, C, b, tyi, txi, special);
+  for (int i = threadIdx.x; i < C * g.TSZ; i += NT) acc[i] = 0.0;
+  for (int i = threadIdx.x; i < C * LM; i += NT) acc_w[i] = 0.0;
+  for (int i = threadIdx.x; i < C * V; i += NT) acc_t[i] = 0.0;
+  const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
+  const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
+  const bool live = oy < g.OH && ox < g.OW;
+  const int base = ty * g.sy * g.IW + tx * g.sx;
+  const Real *mine = tile + base;
+  // Lane l takes the channels in the order skew(l), skew(l) + 1, ... (mod C): the lanes of a wavefront are spread over
+  // min(C, 64) trees' tables and dX planes, so the atomics of one instruction rarely meet on one address.
+  const int lane = int(threadIdx.x & 63u);
+  const int skew = ((lane & 31) + (lane >> 5) * (C >> 1)) % C;
+  const int j_begin = blockIdx.y * j_per, j_count = min(Cout, j_begin + j_per) - j_begin;
+  const int rot = int((blockIdx.x * 7u + blockIdx.z * 13u) % unsigned(j_count));
+  for (int jj = 0; jj < j_count; ++jj) {
+    const int j = j_begin + (jj + rot >= j_count ? jj + rot - j_count : jj + rot);
+    __syncthreads();  // the tile and the zeroed tables are complete / the previous out channel's walks are done
+    if (jj > 0) {
+      // flush the previous out channel's tables (its trees are still known by index only: jp)
+      const int jp = j_begin + (jj - 1 + rot >= j_count ? jj - 1 + rot - j_count : jj - 1 + rot);
+      if (dw)
+        for (int i = threadIdx.x; i < C * LM; i += NT) {
+          const double v = acc_w[i];
+          if (v != 0.0) {
+            atomicAdd(dw + (long long)jp * C * LM + i, Real(v));
+            acc_w[i] = 0.0;
+          }
+        }
+      if (dthr)
+        for (int i = threadIdx.x; i < C * V; i += NT) {
+          const double v = acc_t[i];
+          if (v != 0.0) {
+            atomicAdd(dthr + (long long)jp * C * V + i, Real(v));
+            acc_t[i] = 0.0;
+          }
+        }
+    }
+    stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
+    __syncthreads();
+    if (!live) continue;
+    const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+    for (int c = 0; c < C; c += kConvIlp) {
+      WalkResult<Real> r[kConvIlp];
+      const Node<Real> *nd[kConvIlp];
+      const Real *px[kConvIlp];
+      int ch[kConvIlp];
+#pragma unroll
+      for (int i = 0; i < kConvIlp; ++i) {
+        int ci = min(c + i, C - 1) + skew;
+        ci = ci >= C ? ci - C : ci;
+        ch[i] = ci;
+        nd[i] = nodes + ci * V;
+        px[i] = mine + ci * g.TSZ;
+      }
+      conv_walks<Real, FERN, true>(false, depth, nd, px, r);
+#pragma unroll
+      for (int i = 0; i < kConvIlp; ++i) {
+        if (c + i >= C) break;
+        const Real a = ht_abs(r[i].margin);
+        const int cell = (ch[i] * L + int(r[i].key)) * M;
+        Real cs = Real(0);
+        for (int m = 0; m < M; ++m) {
+          const Real gv = gp[m];
+          cs += wl[cell + m] * gv;
+          if (dw) atomicAdd(acc_w + cell + m, double(a * gv));
+        }
+        cs = ht_sign(r[i].margin) * cs;
+        if (dthr) atomicAdd(acc_t + ch[i] * V + int(r[i].vertex), -double(cs));
+        atomicAdd(acc + ch[i] * g.TSZ + base + int(r[i].ord), double(cs));  // r.ord is the tap's tile offset
+      }
+    }
+  }
+  __syncthreads();
+  {
+    const int jp = j_begin + (j_count - 1 + rot >= j_count ? rot - 1 : j_count - 1 + rot);
+    if (dw)
+      for (int i = threadIdx.x; i < C * LM; i += NT)
+        if (acc_w[i] != 0.0) atomicAdd(dw + (long long)jp * C * LM + i, Real(acc_w[i]));
+    if (dthr)
+      for (int i = threadIdx.x; i < C * V; i += NT)
+        if (acc_t[i] != 0.0) atomicAdd(dthr + (long long)jp * C * V + i, Real(acc_t[i]));
+  }
+  const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
+  for (int i = threadIdx.x; i < C * g.TSZ; i += NT) {
+    const double v = acc[i];
+    if (v == 0.0) continue;
+    const int c = i / g.TSZ, r = i - c * g.TSZ;
+    const int iy = r / g.IW, ix = r - iy * g.IW;
+    const int gy = iy0 + iy, gx = ix0 + ix;
+    if (gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) atomicAdd(dx + ((b * C + c) * g.H + gy) * (long long)g.W + gx, Real(v));
+  }
+}
+
+constexpr int kConvWideThreads = 512;  // workgroup of the one-walk backward kernel
+
 constexpr size_t kConvTiledLdsMax = 160 * 1024;  // LDS of a CU
 
 // Out channels per workgroup of the tile-stationary kernels: all of them unless that leaves the device underfilled.
@@ -671,6 +793,28 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
   if (dw && (rc = zero_fill(dw, size_t(s.Cout) * s.C * L * s.M * sizeof(Real), stream)) != HT_OK) return rc;
   if (s.B == 0 || s.Cout == 0 || s.C == 0 || g.rows == 0 || (!dx && !dthr && !dw)) return HT_OK;
   ConvTile t;
+  // dX together with a tree gradient: one walk serves all of them where the tables fit beside the dX image, with the
+  // wide workgroup first and the ordinary one for shapes whose wide tile is too large for LDS.
+  for (int threads : {kConvWideThreads, kConvThreads}) {
+    if (!(dx && (dthr || dw)) || !make_tile(g, &t, threads)) continue;
+    const int LM = L * int(s.M);
+    const ConvLds lay = conv_lds_layout<Real>(t, int(s.C), V, LM, true, true, true);
+    const long long tiles = (long long)t.tiles_y * t.tiles_x;
+    if (lay.total > kConvTiledLdsMax || tiles > 0x7fffffffLL) continue;
+    const int j_per = conv_j_per(tiles * s.B, int(s.Cout));
+    const dim3 grid((unsigned)tiles, (unsigned)((s.Cout + j_per - 1) / j_per), (unsigned)s.B);
+    auto kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvWideThreads>
+                       : conv_tiled_backward_kernel<Real, false, kConvWideThreads>;
+    if (threads == kConvThreads)
+      kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvThreads>
+                    : conv_tiled_backward_kernel<Real, false, kConvThreads>;
+    HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(lay.total)));
+    hipLaunchKernelGGL(kernel, grid, dim3(threads), lay.total, stream, t, lay, int(s.C), int(s.Cout), int(s.depth), V,
+                       L, int(s.M), j_per, x, thr, ord, w, gout, dx, dthr, dw);
+    HT_LAUNCH_CHECK("conv backward (one walk, tiled)");
+    return HT_OK;
+  }
   if (make_tile(g, &t)) {
     const int LM = L * int(s.M);
     const ConvLds lay_x = conv_lds_layout<Real>(t, int(s.C), V, LM, true, false, true);

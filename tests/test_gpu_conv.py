@@ -22,6 +22,8 @@ CASES = [
     (2, 2, 2, [6, 5, 7], 3, [2], [2, 2, 3], [1, 2, 1], [0, 1, 1], [1, 1, 1]),
     (1, 2, 2, [40, 9], 3, [20], [3, 3], [1, 1], [0, 0], [1, 1]),       # more than 16 outputs per leaf
     (1, 1, 2, [30, 30], 12, [], [5, 5], [1, 1], [2, 2], [1, 1]),       # deep trees: accumulators leave LDS
+    (1, 24, 3, [21, 40], 3, [], [3, 3], [1, 1], [1, 1], [1, 1]),       # many channels: the one-walk backward's narrow tile
+    (2, 40, 2, [9, 33], 2, [], [3, 3], [1, 1], [1, 1], [1, 1]),        # more channels than any tile holds in LDS
 ]
 
 
@@ -44,6 +46,8 @@ def test_conv_parity(dev, case, dtype, fern):
     assert rel_err(dx.cpu(), rdx) <= tol and rel_err(dthr.cpu(), rdthr) <= tol and rel_err(dw.cpu(), rdw) <= tol
     only = getattr(ops, pre + "backward")(gx, False, gthr, True, gord, False, gw, False, gg, ker, st, pad, dil)
     assert only[0] is None and only[3] is None and rel_err(only[1].cpu(), rdthr) <= tol
+    only = getattr(ops, pre + "backward")(gx, True, gthr, False, gord, False, gw, False, gg, ker, st, pad, dil)
+    assert only[1] is None and only[3] is None and rel_err(only[0].cpu(), rdx) <= tol
 
 
 GOLD = sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "conv*.npz")))
