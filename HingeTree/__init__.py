@@ -12,6 +12,8 @@ from hingetreefortorch_amd.functions import (  # noqa: F401
     LinearBatchNorm,
     HingeTreeFusedLinear,
     HingeFernFusedLinear,
+    HingeTreeExpanded,
+    HingeFernExpanded,
     Contract,
     Expand,
     contract,

@@ -12,4 +12,6 @@ from hingetreefortorch_amd.modules import (  # noqa: F401
     LinearHingeForest,
     RandomHingeForestFusedLinear,
     RandomHingeFernFusedLinear,
+    RandomHingeForestExpanded,
+    RandomHingeFernExpanded,
 )

@@ -322,6 +322,17 @@ def bench_tiles(torch, ops, dev, args):
     e_ms = _timed(torch, lambda: ops.expand(tiles, [0, 0]), args.steps, args.warmup)
     nbytes = 2 * image.numel() * 4   # read once, written once
     ms = c_ms + e_ms
+    # the head of the segmentation model: forest with 8 x 8 outputs per leaf on [8, 100, 64, 64], then expand
+    F, T, D = 100, 100, 6
+    cg = torch.Generator().manual_seed(6114)
+    x = torch.randn([B, F, H // P, W // P], generator=cg).to(dev)
+    thr = (6 * torch.rand([T, 2 ** D - 1], generator=cg) - 3).to(dev)
+    ordn = torch.randint(0, F, [T, 2 ** D - 1], generator=cg, dtype=torch.int64).to(dev)
+    wts = torch.randn([T, 2 ** D, P, P], generator=cg).to(dev)
+    assert torch.equal(ops.tree_forward_expanded(x, thr, ordn, wts, [0, 0]),
+                       ops.expand(ops.tree_forward(x, thr, ordn, wts), [0, 0]))
+    two_ms = _timed(torch, lambda: ops.expand(ops.tree_forward(x, thr, ordn, wts), [0, 0]), args.steps, args.warmup)
+    one_ms = _timed(torch, lambda: ops.tree_forward_expanded(x, thr, ordn, wts, [0, 0]), args.steps, args.warmup)
     return {
         "metric": "contract + expand GB/s (tiles [8,100,64,64,8,8] <-> images [8,100,512,512])",
         "value": 2 * nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -329,6 +340,9 @@ def bench_tiles(torch, ops, dev, args):
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "f3: one contract and one expand of an 839 MB float32 image batch, window 8 x 8, no padding"},
         "contract": {"ms": c_ms, "gbps": nbytes / (c_ms * 1e-3) / 1e9}, "expand": {"ms": e_ms, "gbps": nbytes / (e_ms * 1e-3) / 1e9},
+        "forest_then_expand": {"ms": two_ms, "what": "tree_forward [8,100,64,64] x 100 trees of depth 6 x [8,8] outputs, then expand"},
+        "forest_expanded": {"ms": one_ms, "what": "the same image from one pass (tree_forward_expanded)",
+                            "gbps": (nbytes // 2 + x.numel() * 4) / (one_ms * 1e-3) / 1e9},
         "roofline": {"bound": "hbm", "kernel": "tile_permute_kernel", "achieved": 2 * nbytes / (ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": 2 * nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": None, "algorithmic_bytes": nbytes},

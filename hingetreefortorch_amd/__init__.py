@@ -17,6 +17,8 @@ from .modules import (  # noqa: F401
     LinearHingeForest,
     RandomHingeFernFusedLinear,
     RandomHingeForestFusedLinear,
+    RandomHingeFernExpanded,
+    RandomHingeForestExpanded,
     RandomHingeFern,
     RandomHingeForest,
 )

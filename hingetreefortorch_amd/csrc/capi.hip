@@ -44,6 +44,48 @@ int make_dims(const ht_forest_shape *s, ForestDims *d) {
   return HT_OK;
 }
 
+int make_image_store(const ht_tile_shape *g, const ForestDims &d, long long B, ImageStore *img, bool *clear) {
+  if (!g) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null shape.");
+  if (g->nd != 2 && g->nd != 3)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: Only 2D and 3D window sizes are supported.");
+  const int shift = 3 - g->nd;  // a 2-d geometry is a 3-d one with a leading dimension of extent 1
+  for (int dd = 0; dd < 3; ++dd) {
+    img->tiles[dd] = img->win[dd] = img->size[dd] = 1;
+    img->pad[dd] = 0;
+  }
+  long long positions = 1, outputs = 1, plane = 1;
+  *clear = false;
+  for (int dd = 0; dd < g->nd; ++dd) {
+    if (g->size[dd] < 1 || g->tiles[dd] < 1 || g->window[dd] < 1 || g->padding[dd] < 0 || g->size[dd] > 0x3fffffff ||
+        g->tiles[dd] > 0x3fffffff || g->window[dd] > 0x3fffffff || g->padding[dd] > 0x3fffffff)
+      return fail(HT_ERR_INVALID_ARGUMENT, "Error: invalid tile geometry.");
+    img->size[dd + shift] = int(g->size[dd]);
+    img->tiles[dd + shift] = int(g->tiles[dd]);
+    img->win[dd + shift] = int(g->window[dd]);
+    img->pad[dd + shift] = int(g->padding[dd]);
+    positions *= g->tiles[dd];
+    outputs *= g->window[dd];
+    plane *= g->size[dd];
+    if (g->size[dd] > g->tiles[dd] * g->window[dd] - g->padding[dd]) *clear = true;  // positions behind the last tile
+  }
+  if (positions != d.K || outputs != d.M || g->planes != B * d.T)
+    return fail(HT_ERR_INVALID_ARGUMENT,
+                "Error: the tile geometry does not match the forest (tiles = inner data positions, window = outputs "
+                "per leaf, planes = samples x trees).");
+  if (plane > (1ll << 40)) return fail(HT_ERR_RUNTIME, "Error: image too large for this build.");
+  // the in-kernel divisions are exact for dividend x divisor < 2^32
+  for (int dd = 1; dd < 3; ++dd)
+    if ((long long)d.K * img->tiles[dd] >= (1ll << 32) || (long long)d.M * img->win[dd] >= (1ll << 32))
+      return fail(HT_ERR_RUNTIME, "Error: tile geometry too large for the image store of this build.");
+  for (int dd = 0; dd < 3; ++dd) {
+    img->by_tiles[dd] = FastDiv(img->tiles[dd]);
+    img->by_win[dd] = FastDiv(img->win[dd]);
+  }
+  img->plane = plane;
+  img->nd = g->nd;
+  return HT_OK;
+}
+
 // ---- threshold consistency (host memory) -----------------------------------------------------------------------
 // A vertex that re-tests a feature already tested by an ancestor must keep its threshold on the side of the ancestor's
 // threshold that its path came from (HingeTreeCommon.h:211-287).
@@ -127,6 +169,33 @@ int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, 
                                  nullptr, workspace, workspace_bytes, st);
   return forest_forward<double>(d, fern, (const double *)x, (const double *)thr, ord, (const double *)w, (double *)out,
                                 nullptr, workspace, workspace_bytes, st);
+}
+
+int ht_forest_forward_image(const ht_forest_shape *s, const ht_tile_shape *g, const void *x, const void *thr,
+                            const int64_t *ord, const void *w, void *image, void *workspace, size_t workspace_bytes,
+                            void *stream) {
+  ForestDims d;
+  int rc = make_dims(s, &d);
+  if (rc != HT_OK) return rc;
+  ImageStore img{};
+  bool clear = false;
+  if ((rc = make_image_store(g, d, s->B, &img, &clear)) != HT_OK) return rc;
+  if (g->elem_size != (s->dtype == HT_F32 ? 4 : 8))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: the element size of the tile geometry must be that of the forest's data type.");
+  if (d.K == 1)
+    return fail(HT_ERR_INVALID_ARGUMENT,
+                "Error: an image result needs inner data positions (inData of 3 or more dimensions).");
+  if (is_empty(d)) return HT_OK;
+  if (!x || !thr || !ord || !w || !image) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (clear && (rc = zero_fill(image, size_t(g->planes) * size_t(img.plane) * size_t(g->elem_size), st)) != HT_OK)
+    return rc;
+  const bool fern = s->kind == HT_FERN;
+  if (s->dtype == HT_F32)
+    return forest_forward<float>(d, fern, (const float *)x, (const float *)thr, ord, (const float *)w, (float *)image,
+                                 nullptr, workspace, workspace_bytes, st, &img);
+  return forest_forward<double>(d, fern, (const double *)x, (const double *)thr, ord, (const double *)w,
+                                (double *)image, nullptr, workspace, workspace_bytes, st, &img);
 }
 
 size_t ht_forest_records_bytes(const ht_forest_shape *s) {

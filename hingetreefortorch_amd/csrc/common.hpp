@@ -55,6 +55,30 @@ struct FastDiv {
   __device__ __forceinline__ int div(int n) const { return d <= 1 ? n : int(__umulhi(uint32_t(n), inv)); }
 };
 
+// Where a forest with inner data positions [tiles...] and outputs per leaf [window...] stores its result when the caller
+// wants the image that the expand permutation would make of it: element (position k, output m) of a (sample, tree)
+// plane goes to image coordinate tile * window + within - padding of every dimension, and is dropped outside the image.
+// Dimensions are right-aligned in the arrays (a 2-d geometry has a leading dimension of extent 1). nd == 0: off.
+struct ImageStore {
+  int nd;
+  int tiles[3], win[3], pad[3], size[3];
+  FastDiv by_tiles[3], by_win[3];
+  long long plane;  // elements of one (sample, tree) image
+  __device__ __forceinline__ long long offset(int k, int m) const {
+    int q = by_tiles[2].div(k);
+    const int j2 = k - q * tiles[2];
+    const int j0 = by_tiles[1].div(q), j1 = q - j0 * tiles[1];
+    q = by_win[2].div(m);
+    const int w2 = m - q * win[2];
+    const int w0 = by_win[1].div(q), w1 = q - w0 * win[1];
+    const int p0 = j0 * win[0] + w0 - pad[0], p1 = j1 * win[1] + w1 - pad[1], p2 = j2 * win[2] + w2 - pad[2];
+    if (p0 < 0 || p0 >= size[0] || p1 < 0 || p1 >= size[1] || p2 < 0 || p2 >= size[2]) return -1;
+    return ((long long)p0 * size[1] + p1) * size[2] + p2;
+  }
+};
+// Validates the geometry against the forest's shape; *clear is set when the image has positions no tile covers.
+int make_image_store(const ht_tile_shape *g, const ForestDims &d, long long B, ImageStore *img, bool *clear);
+
 // How a tile kernel spreads the trees over blockIdx.y: with few sample tiles the trees are split so that at least
 // ~2 workgroups per CU exist; `group` is the number of trees a workgroup handles per pass.
 static inline void split_trees(long long tiles, int T, int group, int *trees_per_block, int *grid_y) {
@@ -78,9 +102,11 @@ int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *d
 template <typename Real>
 size_t forest_forward_workspace(const ForestDims &d);
 // `records` (optional): forest_records_bytes() bytes that receive the walk records for forest_backward_records().
+// `image` (optional): store the result as that image instead of [B, T, K, M]; needs K > 1.
 template <typename Real>
 int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                   Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream);
+                   Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream,
+                   const ImageStore *image = nullptr);
 
 template <typename Real>
 size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw);

@@ -42,7 +42,7 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
                                                      const Node<Real> *__restrict__ nodes,
                                                      const Real *__restrict__ w, Real *__restrict__ out,
                                                      Records<Real, COMPACT> rec, int trees_per_block,
-                                                     FastDiv div_m) {
+                                                     FastDiv div_m, ImageStore img) {
   typedef Real Vec __attribute__((ext_vector_type(VW)));
   constexpr int TC = NT / BT;        // tree slots per walk round
   constexpr int kIlp = ILP;
@@ -141,13 +141,21 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
           const int r = v * VW;
           const int jj = div_m.div(r), m = r - jj * d.M;
           if (s0 + jj >= d.S) continue;
+          Real *dst = obase + r + (k0 + jj >= d.K ? wrap : 0ll);
+          if (img.nd) {
+            // the vector's VW outputs are consecutive along the innermost window dimension, hence in the image
+            const bool next = k0 + jj >= d.K;
+            const long long at = img.offset(k0 + jj - (next ? d.K : 0), m);
+            if (at < 0) continue;
+            dst = out + ((b0 + (next ? 1 : 0)) * d.T + tb + t2) * img.plane + at;
+          }
           const uint32_t key = r_key[jj * LDR + t2];
           const Real a = r_abs[jj * LDR + t2];
           const Vec wv = *reinterpret_cast<const Vec *>(wbase + (long long)key * d.M + m);
           Vec o;
 #pragma unroll
           for (int i = 0; i < VW; ++i) o[i] = a * wv[i];
-          *reinterpret_cast<Vec *>(obase + r + (k0 + jj >= d.K ? wrap : 0ll)) = o;
+          *reinterpret_cast<Vec *>(dst) = o;
         }
       }
     } else {
@@ -158,8 +166,15 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
         const int jj = div_m.div(r), m = r - jj * d.M;
         const long long ss = s0 + jj;
         if (ss < d.S) {
+          long long at = out_offset(d, ss, tb + t2, m);
+          if (img.nd) {
+            const long long b = ss / d.K;
+            const long long in_plane = img.offset(int(ss - b * d.K), m);
+            if (in_plane < 0) continue;
+            at = (b * d.T + tb + t2) * img.plane + in_plane;
+          }
           const uint32_t key = r_key[jj * LDR + t2];
-          out[out_offset(d, ss, tb + t2, m)] = r_abs[jj * LDR + t2] * w[((long long)(tb + t2) * d.L + key) * d.M + m];
+          out[at] = r_abs[jj * LDR + t2] * w[((long long)(tb + t2) * d.L + key) * d.M + m];
         }
       }
     }
@@ -549,11 +564,11 @@ int dispatch_rows(const ForestDims &d, const Real *x, const void *vertices, cons
 
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
 int launch_forward_rec(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                       void *records, hipStream_t stream);
+                       void *records, hipStream_t stream, const ImageStore &img);
 
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW, bool RECORD, bool COMPACT>
 int launch_forward_vw(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                      void *records, hipStream_t stream) {
+                      void *records, hipStream_t stream, const ImageStore &img) {
   constexpr int NT = kForestThreads;
   constexpr int TP = NT / BT * ILP;
   const size_t lds = (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TP + 1) * BT * (sizeof(Real) + sizeof(KeyT));
@@ -567,46 +582,52 @@ int launch_forward_vw(const ForestDims &d, const Real *x, const Node<Real> *node
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(NT), lds, stream, d, x, nodes, w, out, rec,
-                     trees_per_block, FastDiv(d.M));
+                     trees_per_block, FastDiv(d.M), img);
   HT_LAUNCH_CHECK("forest forward");
   return HT_OK;
 }
 
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
 int launch_forward_rec(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                       void *records, hipStream_t stream) {
+                       void *records, hipStream_t stream, const ImageStore &img) {
   if (!records)
-    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, false, true>(d, x, nodes, w, out, records, stream);
+    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, false, true>(d, x, nodes, w, out, records, stream,
+                                                                               img);
   if (compact_ok(d))
-    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, true, true>(d, x, nodes, w, out, records, stream);
-  return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, true, false>(d, x, nodes, w, out, records, stream);
+    return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, true, true>(d, x, nodes, w, out, records, stream,
+                                                                              img);
+  return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, true, false>(d, x, nodes, w, out, records, stream, img);
 }
 
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT>
 int launch_forward_as(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                      void *records, hipStream_t stream) {
-  // widest output vector that M and the pointers allow (inner dimensions shorter than the tile keep scalar outputs)
+                      void *records, hipStream_t stream, const ImageStore &img) {
+  // widest output vector that M and the pointers allow (inner dimensions shorter than the tile keep scalar outputs);
+  // into an image, a vector must also stay inside one window row and keep the image rows aligned
   const uintptr_t pw = reinterpret_cast<uintptr_t>(w), po = reinterpret_cast<uintptr_t>(out);
   const bool runs = d.K == 1 || d.K >= BT;  // the branches of the kernel that store whole vectors
-  if (runs && d.M % 4 == 0 && pw % (4 * sizeof(Real)) == 0 && po % (4 * sizeof(Real)) == 0)
-    return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 4>(d, x, nodes, w, out, records, stream);
-  if (runs && d.M % 2 == 0 && pw % (2 * sizeof(Real)) == 0 && po % (2 * sizeof(Real)) == 0)
-    return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 2>(d, x, nodes, w, out, records, stream);
-  return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 1>(d, x, nodes, w, out, records, stream);
+  auto fits = [&](int vw) {
+    if (!runs || d.M % vw != 0 || pw % (vw * sizeof(Real)) != 0 || po % (vw * sizeof(Real)) != 0) return false;
+    return img.nd == 0 || (img.win[2] % vw == 0 && img.pad[2] % vw == 0 && img.size[2] % vw == 0);
+  };
+  if (fits(4)) return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 4>(d, x, nodes, w, out, records, stream, img);
+  if (fits(2)) return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 2>(d, x, nodes, w, out, records, stream, img);
+  return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 1>(d, x, nodes, w, out, records, stream, img);
 }
 
 // Four trees per thread with 16-bit parked keys where the depth allows it, else two trees with 32-bit keys: both keep
 // the per-pass results of a 1024-thread workgroup under the LDS left beside a 128 KB sample tile.
 template <typename Real, bool FERN, int BT, bool XLDS>
 int launch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                   void *records, hipStream_t stream) {
-  if (d.depth <= 16) return launch_forward_as<Real, FERN, BT, XLDS, 4, uint16_t>(d, x, nodes, w, out, records, stream);
-  return launch_forward_as<Real, FERN, BT, XLDS, 2, uint32_t>(d, x, nodes, w, out, records, stream);
+                   void *records, hipStream_t stream, const ImageStore &img) {
+  if (d.depth <= 16)
+    return launch_forward_as<Real, FERN, BT, XLDS, 4, uint16_t>(d, x, nodes, w, out, records, stream, img);
+  return launch_forward_as<Real, FERN, BT, XLDS, 2, uint32_t>(d, x, nodes, w, out, records, stream, img);
 }
 
 template <typename Real, bool FERN>
 int dispatch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                     void *records, hipStream_t stream) {
+                     void *records, hipStream_t stream, const ImageStore &img) {
   // room for the per-pass results: (4 trees x 1024 threads + one pad column) x (|margin| + key)
   const size_t reserve = size_t(4) * kForestThreads * (sizeof(Real) + sizeof(uint32_t));
   int bt = pick_tile<Real>(d.F, reserve);
@@ -614,11 +635,11 @@ int dispatch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes
   // pass (longer contiguous row segments per store burst, half the barriers) and one row per wavefront.
   if (d.M >= 8 && bt >= 32) bt /= 2;
   switch (bt) {
-    case 64: return launch_forward<Real, FERN, 64, true>(d, x, nodes, w, out, records, stream);
-    case 32: return launch_forward<Real, FERN, 32, true>(d, x, nodes, w, out, records, stream);
-    case 16: return launch_forward<Real, FERN, 16, true>(d, x, nodes, w, out, records, stream);
-    case 8: return launch_forward<Real, FERN, 8, true>(d, x, nodes, w, out, records, stream);
-    default: return launch_forward<Real, FERN, 64, false>(d, x, nodes, w, out, records, stream);
+    case 64: return launch_forward<Real, FERN, 64, true>(d, x, nodes, w, out, records, stream, img);
+    case 32: return launch_forward<Real, FERN, 32, true>(d, x, nodes, w, out, records, stream, img);
+    case 16: return launch_forward<Real, FERN, 16, true>(d, x, nodes, w, out, records, stream, img);
+    case 8: return launch_forward<Real, FERN, 8, true>(d, x, nodes, w, out, records, stream, img);
+    default: return launch_forward<Real, FERN, 64, false>(d, x, nodes, w, out, records, stream, img);
   }
 }
 
@@ -691,10 +712,14 @@ __global__ __launch_bounds__(256) void pad_rows_kernel(const Real *__restrict__ 
 
 template <typename Real>
 int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                   Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream) {
+                   Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream, const ImageStore *image) {
   if (is_empty(d)) return HT_OK;
   if (ws == nullptr || ws_bytes < forest_forward_workspace<Real>(d))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the forward pass.");
+  ImageStore img{};
+  if (image) img = *image;
+  if (img.nd && d.K == 1)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: an image result needs inner data positions (inData of 3 or more dimensions).");
   if (rows_ok<Real>(d)) {
     int wpitch = weight_pitch<Real>(d);
     if (wpitch != d.M) {
@@ -724,8 +749,8 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
   int rc = pack_nodes<Real>(d, thr, ord, ws, stream);
   if (rc != HT_OK) return rc;
   const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
-  return fern ? dispatch_forward<Real, true>(d, x, nodes, w, out, records, stream)
-              : dispatch_forward<Real, false>(d, x, nodes, w, out, records, stream);
+  return fern ? dispatch_forward<Real, true>(d, x, nodes, w, out, records, stream, img)
+              : dispatch_forward<Real, false>(d, x, nodes, w, out, records, stream, img);
 }
 
 #define HT_INSTANTIATE(Real)                                                                                          \
@@ -733,7 +758,7 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
   template int pack_nodes<Real>(const ForestDims &, const Real *, const int64_t *, void *, hipStream_t);              \
   template size_t forest_forward_workspace<Real>(const ForestDims &);                                                 \
   template int forest_forward<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,            \
-                                    const Real *, Real *, void *, void *, size_t, hipStream_t);
+                                    const Real *, Real *, void *, void *, size_t, hipStream_t, const ImageStore *);
 HT_INSTANTIATE(float)
 HT_INSTANTIATE(double)
 #undef HT_INSTANTIATE

@@ -272,6 +272,57 @@ class _Contract(torch.autograd.Function):
         return None, None, None
 
 
+class _ForestExpandedFunction(torch.autograd.Function):
+    """Forest with tile-shaped outputs per leaf followed by Expand, as one operator: the forward pass stores the image
+    directly (the tile-major intermediate [B, T, *tiles, *window] is never written); the backward pass contracts the
+    upstream gradient and runs the forest's backward. Same values as Expand(padding)(HingeTree.apply(...)), which is
+    how the reference's segmentation model composes the two (rcc/Net.py:99-109)."""
+    _prefix = None
+
+    @staticmethod
+    def _forward(cls, ctx, inData, inThresholds, inOrdinals, inWeights, padding):
+        nd = inWeights.dim() - 2
+        ctx.padding = [padding] * nd if isinstance(padding, int) else list(padding)
+        ctx.save_for_backward(inData, inThresholds, inOrdinals, inWeights)
+        return getattr(_ops, f"{cls._prefix}_forward_expanded")(inData, inThresholds, inOrdinals, inWeights, ctx.padding)
+
+    @staticmethod
+    def _backward(cls, ctx, outDataGrad):
+        inData, inThresholds, inOrdinals, inWeights = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        tiles = _ops.contract(outDataGrad.contiguous(), list(inWeights.shape[2:]), ctx.padding)
+        name = "backward_deterministic" if _is_deterministic() else "backward"
+        grads = getattr(_ops, f"{cls._prefix}_{name}")(inData, need[0], inThresholds, need[1], inOrdinals, need[2],
+                                                      inWeights, need[3], tiles)
+        return tuple(grads) + (None,)
+
+
+class HingeTreeExpanded(_ForestExpandedFunction):
+    _prefix = "tree"
+
+    @staticmethod
+    def forward(ctx, inData, inThresholds, inOrdinals, inWeights, padding=0):
+        return _ForestExpandedFunction._forward(HingeTreeExpanded, ctx, inData, inThresholds, inOrdinals, inWeights,
+                                                padding)
+
+    @staticmethod
+    def backward(ctx, outDataGrad):
+        return _ForestExpandedFunction._backward(HingeTreeExpanded, ctx, outDataGrad)
+
+
+class HingeFernExpanded(_ForestExpandedFunction):
+    _prefix = "fern"
+
+    @staticmethod
+    def forward(ctx, inData, inThresholds, inOrdinals, inWeights, padding=0):
+        return _ForestExpandedFunction._forward(HingeFernExpanded, ctx, inData, inThresholds, inOrdinals, inWeights,
+                                                padding)
+
+    @staticmethod
+    def backward(ctx, outDataGrad):
+        return _ForestExpandedFunction._backward(HingeFernExpanded, ctx, outDataGrad)
+
+
 class Expand(torch.nn.Module):
     """_HingeTree.py:75-81."""
 

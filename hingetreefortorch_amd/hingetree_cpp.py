@@ -407,6 +407,39 @@ def _forward(kind, inData, inThresholds, inOrdinals, inWeights):
     return out
 
 
+def _forward_expanded(kind, inData, inThresholds, inOrdinals, inWeights, padding):
+    """expand(forward(...), padding) in one pass: the forest stores its result as the image directly. No counterpart
+    in the reference, which runs hingetree forward and expand back to back (rcc/Net.py:99-109). Shapes the fused store
+    does not serve (no inner data positions) take the two calls."""
+    _common_checks([inData, inThresholds, inWeights], inOrdinals, False)
+    shape, out_sizes = _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights)
+    padding = [int(v) for v in padding]
+    nd = len(padding)
+    tiles, window = [int(v) for v in inData.shape[2:]], [int(v) for v in inWeights.shape[2:]]
+    if nd not in (2, 3):
+        _invalid("Error: Only 2D and 3D padding sizes are supported.")
+    if len(tiles) != nd or len(window) != nd or any(p < 0 for p in padding):
+        _invalid(f"Error: inData and inWeights must have {nd + 2} dimensions. Padding must be non-negative.")
+    size = [t * w - ((2 * p) // w) * w for t, w, p in zip(tiles, window, padding)]  # expand.cpp:180-181,239-241
+    if any(n < 1 for n in size):
+        _invalid("Error: The expanded size of the image must be non-empty.")
+    if shape.K == 1 or shape.B == 0 or shape.T == 0:
+        return expand(_forward(kind, inData, inThresholds, inOrdinals, inWeights), padding)
+    geom = L.TileShape()
+    geom.planes, geom.nd, geom.elem_size = int(shape.B) * int(shape.T), nd, inData.element_size()
+    for i in range(nd):
+        geom.size[i], geom.tiles[i], geom.window[i], geom.padding[i] = size[i], tiles[i], window[i], padding[i]
+    with torch.cuda.device(inData.device):
+        out = torch.empty(out_sizes[:2] + size, dtype=inData.dtype, device=inData.device)
+        lib = L.load()
+        nbytes = lib.ht_forest_forward_workspace(ctypes.byref(shape))
+        ws = _workspace(nbytes, inData.device)
+        L.check(lib.ht_forest_forward_image(ctypes.byref(shape), ctypes.byref(geom), _ptr(inData), _ptr(inThresholds),
+                                            _ptr(inOrdinals), _ptr(inWeights), _ptr(out), _ptr(ws), nbytes,
+                                            _stream(inData.device)))
+    return out
+
+
 def _backward(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad, inWeights,
               bInWeightsGrad, outDataGrad):
     _common_checks([inData, inThresholds, inWeights, outDataGrad], inOrdinals, True)
@@ -568,6 +601,14 @@ def tree_forward(inData, inThresholds, inOrdinals, inWeights):
 
 def fern_forward(inData, inThresholds, inOrdinals, inWeights):
     return _forward(L.HT_FERN, inData, inThresholds, inOrdinals, inWeights)
+
+
+def tree_forward_expanded(inData, inThresholds, inOrdinals, inWeights, padding):
+    return _forward_expanded(L.HT_TREE, inData, inThresholds, inOrdinals, inWeights, padding)
+
+
+def fern_forward_expanded(inData, inThresholds, inOrdinals, inWeights, padding):
+    return _forward_expanded(L.HT_FERN, inData, inThresholds, inOrdinals, inWeights, padding)
 
 
 def tree_forward_records(inData, inThresholds, inOrdinals, inWeights):

@@ -233,6 +233,32 @@ class RandomHingeFernFusedLinear(RandomHingeFern, _FusedLinearMixin):
                                               self.linear_bias)
 
 
+class RandomHingeForestExpanded(RandomHingeForest):
+    """RandomHingeForest with tile-shaped extra_outputs followed by Expand(padding) (the head of the reference's
+    segmentation model, rcc/Net.py:99-109) as one module: same parameters and state dict as RandomHingeForest, same
+    values as the two modules in sequence, one pass over memory less."""
+
+    def __init__(self, in_channels: int, out_channels: int, depth: int, extra_outputs, init_type: str = "random",
+                 padding=0):
+        super().__init__(in_channels, out_channels, depth, extra_outputs, init_type)
+        self.padding = padding
+
+    def forward(self, x):
+        return _fn.HingeTreeExpanded.apply(x, self.thresholds, self.ordinals, self.weights, self.padding)
+
+
+class RandomHingeFernExpanded(RandomHingeFern):
+    """RandomHingeFern followed by Expand(padding) as one module; see RandomHingeForestExpanded."""
+
+    def __init__(self, in_channels: int, out_channels: int, depth: int, extra_outputs, init_type: str = "random",
+                 padding=0):
+        super().__init__(in_channels, out_channels, depth, extra_outputs, init_type)
+        self.padding = padding
+
+    def forward(self, x):
+        return _fn.HingeFernExpanded.apply(x, self.thresholds, self.ordinals, self.weights, self.padding)
+
+
 class LinearHingeForest(nn.Module):
     """Linear(bias=False) -> BatchNorm1d(affine=False) -> RandomHingeForest(init_type="sequential") as one module: the
     model of the reference's README (README.md:117-129; experiments/run_letter_seq.py:45-52), where the linear layer

@@ -72,6 +72,16 @@ size_t ht_forest_forward_workspace(const ht_forest_shape *s);
 int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
                       void *out, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ht_forest_forward of a forest with inner data positions x [B, F, *tiles] and tile-shaped outputs per leaf
+ * w [T, L, *window], whose result is stored directly as the image [B, T, *size] that ht_expand makes of
+ * [B, T, *tiles, *window] (g: planes = B * T, elem_size = that of the data type; image positions no tile covers are 0).
+ * One call in place of the pair hingetree_gpu_forward (hingetree_gpu.cu:416-498) + expand_gpu (expand_gpu.cu:110-172)
+ * that the reference's segmentation model runs back to back (rcc/Net.py:99-109): the [B, T, *tiles, *window]
+ * intermediate is never written. Same workspace as ht_forest_forward. */
+int ht_forest_forward_image(const ht_forest_shape *s, const ht_tile_shape *g, const void *x, const void *thr,
+                            const int64_t *ord, const void *w, void *image, void *workspace, size_t workspace_bytes,
+                            void *stream);
+
 /* Gradients of the above w.r.t. x, thr and w; any of dx/dthr/dw may be NULL (not requested). The library clears the
  * requested buffers itself and then accumulates into them.
  * mode HT_BACKWARD_ATOMIC replaces hingetree_gpu_backward (hingetree.cpp:48,695-740; hingetree_gpu.cu:619-730);

@@ -100,3 +100,65 @@ def test_tile_autograd_and_modules(dev):
     # the segmentation models' use: extra_outputs = [8, 8] tiles expanded back to an image
     tiles = torch.randn([2, 5, 4, 6, 8, 8], device=dev)
     assert Expand()(tiles).shape == (2, 5, 32, 48)
+
+
+EXPANDED = [
+    # B, F, tiles, T, depth, window, padding
+    (2, 7, [9, 12], 3, 3, [8, 8], [0, 0]),        # vector stores, inner positions >= tile
+    (3, 5, [5, 7], 4, 2, [4, 4], [2, 4]),         # cropped borders; positions behind the last tile read 0
+    (2, 6, [3, 4], 2, 3, [2, 3], [1, 0]),         # scalar stores, few inner positions (generic addressing)
+    (1, 4, [2, 3, 5], 3, 2, [2, 2, 4], [0, 1, 4]),  # 3-d
+    (70, 9, [1, 2], 2, 2, [3, 2], [0, 1]),        # tiles that cross several batch rows
+]
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("case", EXPANDED, ids=[f"e{i}" for i in range(len(EXPANDED))])
+def test_forward_expanded_equals_forward_then_expand(dev, case, dtype, fern):
+    """The forest that stores its result as an image directly must give the bits of expand(forward(...)), and both
+    must give the oracle's (walk + permutation restated on the CPU)."""
+    B, F, tiles, T, depth, window, padding = case
+    g = torch.Generator().manual_seed(5)
+    V = depth if fern else 2 ** depth - 1
+    x = torch.randn([B, F] + tiles, generator=g, dtype=dtype)
+    thr = (2 * torch.rand([T, V], generator=g, dtype=dtype) - 1)
+    ordn = torch.randint(0, F, [T, V], generator=g, dtype=torch.int64)
+    w = torch.randn([T, 2 ** depth] + window, generator=g, dtype=dtype)
+    pre = "fern" if fern else "tree"
+    want = ho.expand(ho.forward(x, thr, ordn, w, fern=fern), padding)
+    d = [t.to(dev) for t in (x, thr, ordn, w)]
+    two = ops.expand(getattr(ops, pre + "_forward")(*d), padding)
+    one = getattr(ops, pre + "_forward_expanded")(*d, padding)
+    assert one.shape == two.shape == want.shape
+    assert torch.equal(two.cpu(), want) and torch.equal(one.cpu(), want)
+
+
+def test_expanded_module_and_gradients(dev):
+    from RandomHingeForest import RandomHingeForest, RandomHingeForestExpanded
+    torch.manual_seed(3)
+    ref = RandomHingeForest(6, 4, 3, extra_outputs=[4, 4]).to(dev)
+    one = RandomHingeForestExpanded(6, 4, 3, extra_outputs=[4, 4], padding=2).to(dev)
+    one.load_state_dict(ref.state_dict())
+    x1 = torch.randn([3, 6, 5, 6], device=dev, requires_grad=True)
+    x2 = x1.detach().clone().requires_grad_(True)
+    y1 = Expand(padding=2)(ref(x1))
+    y2 = one(x2)
+    assert torch.equal(y1, y2)
+    u = torch.randn_like(y1)
+    (y1 * u).sum().backward()
+    (y2 * u).sum().backward()
+    for a, b in ((x1.grad, x2.grad), (ref.thresholds.grad, one.thresholds.grad), (ref.weights.grad, one.weights.grad)):
+        assert torch.allclose(a, b, rtol=1e-5, atol=1e-6)
+
+
+def test_forward_expanded_errors(dev):
+    x = torch.zeros([2, 3, 4, 4], device=dev)
+    thr, ordn = torch.zeros([2, 3], device=dev), torch.zeros([2, 3], dtype=torch.int64, device=dev)
+    w = torch.zeros([2, 4, 2, 2], device=dev)
+    with pytest.raises(ValueError, match="Only 2D and 3D padding"):
+        ops.tree_forward_expanded(x, thr, ordn, w, [0])
+    with pytest.raises(ValueError, match="must have 5 dimensions"):
+        ops.tree_forward_expanded(x, thr, ordn, w, [0, 0, 0])
+    with pytest.raises(ValueError, match="expanded size of the image must be non-empty"):
+        ops.tree_forward_expanded(x[:, :, :1, :1].contiguous(), thr, ordn, w, [1, 1])
