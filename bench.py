@@ -207,9 +207,10 @@ def bench_projection(torch, ops, dev, args):
         if ev: ev[0].record()
         zhat, mean, rstd, var = ops.linear_bn_forward(x, lin, 1e-5)
         if ev: ev[1].record()
-        out = ops.tree_forward(zhat, thr, ordn, w)
+        # the training path of the autograd function: the forward keeps its walk records for the backward
+        out, rec = ops.tree_forward_records(zhat, thr, ordn, w)
         if ev: ev[2].record()
-        dz, dthr, _, dw = ops.tree_backward(zhat, True, thr, True, ordn, False, w, True, gout)
+        dz, dthr, _, dw = ops.tree_backward_records(rec, False, zhat, True, thr, True, ordn, False, w, True, gout)
         if ev: ev[3].record()
         ops.linear_bn_backward(x, False, lin, True, zhat, rstd, dz)
         if ev: ev[4].record()

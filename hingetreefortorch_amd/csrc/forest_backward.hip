@@ -247,7 +247,17 @@ __global__ __launch_bounds__(256) void fixed_to_real_kernel(const unsigned long 
 //
 // FIXED (deterministic mode): the accumulators are 64-bit fixed point (see above); partial sums of sample parts are
 // merged with integer atomics into dw_fixed and converted by fixed_to_real_kernel.
-constexpr int kMaxGroupTrees = 16;  // trees per workgroup (so a 64-pair step covers >= 4 consecutive samples per tree)
+constexpr int kMaxGroupTrees = 16;
+
+// Tree group of workgroup column x (a grid row has 8 * ceil(groups / 8) columns), or -1 for a surplus column.
+// Workgroups are dealt to the 8 XCDs round robin by index and each XCD has its own L2; adjacent tree groups read
+// adjacent pieces of the same 128-byte lines of the upstream gradient, so they are placed on the same XCD (group =
+// (index mod 8) * groups_per_xcd + index / 8): the line is then fetched from memory once instead of once per XCD.
+__device__ __forceinline__ int xcd_tree_group(unsigned x, int num_groups) {
+  const int per_xcd = (num_groups + kNumXCDs - 1) / kNumXCDs;
+  const int group = int(x % kNumXCDs) * per_xcd + int(x / kNumXCDs);
+  return group < num_groups ? group : -1;
+}
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_swap(float v) {
@@ -286,12 +296,8 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
     inv_scale = hdr->inv_scale_w;
     if (!dw && !need_c) return;
   }
-  // Workgroups are dealt to the 8 XCDs round robin by index, and each XCD has its own L2. Adjacent tree groups read
-  // adjacent pieces of the same 128-byte lines of the upstream gradient, so they are placed on the same XCD (group =
-  // (index mod 8) * groups_per_xcd + index / 8): the line is then fetched from memory once instead of once per XCD.
-  const int per_xcd = (num_groups + kNumXCDs - 1) / kNumXCDs;
-  const int group = int(blockIdx.x % kNumXCDs) * per_xcd + int(blockIdx.x / kNumXCDs);
-  if (group >= num_groups) return;
+  const int group = xcd_tree_group(blockIdx.x, num_groups);
+  if (group < 0) return;
   const int t0 = group * TB;
   const int nt = min(TB, d.T - t0);
   const long long LM = (long long)d.L * d.M;
@@ -535,9 +541,8 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     if (!dw && !need_c) return;
   }
   const int TB = 1 << log2_tb;
-  const int per_xcd = (num_groups + kNumXCDs - 1) / kNumXCDs;
-  const int group = int(blockIdx.x % kNumXCDs) * per_xcd + int(blockIdx.x / kNumXCDs);
-  if (group >= num_groups) return;
+  const int group = xcd_tree_group(blockIdx.x, num_groups);
+  if (group < 0) return;
   const int t0 = group * TB;
   const int nt = min(TB, d.T - t0);
   const uint32_t LM = uint32_t(d.L) * M;
@@ -748,6 +753,157 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     }
   }
   if (dw) {
+    float *dst = dw + (long long)t0 * LM;
+    const uint32_t n = uint32_t(nt) * LM;
+    if (FIXED) {
+      const unsigned long long *q = reinterpret_cast<const unsigned long long *>(acc);
+      if (dw_atomic) {
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads)
+          if (q[i] != 0ull) atomicAdd(dw_fixed + (long long)t0 * LM + i, q[i]);
+      } else {
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = from_fixed<float>(q[i], inv_scale);
+      }
+    } else {
+      const double *q = reinterpret_cast<const double *>(acc);
+      if (dw_atomic) {
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads)
+          if (q[i] != 0.0) atomicAdd(dst + i, float(q[i]));
+      } else {
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = float(q[i]);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// tree-stationary dW + c for wide leaf rows: float, compact records, M = 4 * P with P a power of two (16 ... 256
+// outputs per leaf, e.g. the 8 x 8 tiles of a segmentation head), any K
+// ---------------------------------------------------------------------------------------------------------------
+// A row of M values is one or more whole 64-byte sectors, so nothing is gained by interleaving trees: a wavefront
+// takes 64 / P consecutive samples of ONE tree per step, P adjacent lanes per pair, one 16-byte load of the upstream
+// gradient and one of the leaf row per lane, both perfectly coalesced per pair (for K > 1 consecutive samples of a tree
+// are even consecutive in memory). Everything that does not depend on the data is a lane constant; the sum over a
+// row for c runs over the lanes of a pair with DPP row operations. Two steps are in flight per wavefront.
+template <int P>
+__device__ __forceinline__ float row_group_sum(float v) {
+  if constexpr (P >= 2) v += dpp_swap<0xB1>(v);   // quad_perm [1,0,3,2]
+  if constexpr (P >= 4) v += dpp_swap<0x4E>(v);   // quad_perm [2,3,0,1]
+  if constexpr (P >= 8) v += dpp_swap<0x141>(v);  // row_half_mirror: the other quad of each 8 lanes
+  if constexpr (P >= 16) v += dpp_swap<0x140>(v); // row_mirror: the other half of each 16 lanes
+  if constexpr (P >= 32) v += __shfl_xor(v, 16, kWave);
+  if constexpr (P >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+template <int P, bool FIXED>
+__global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d, const float *__restrict__ w,
+                                                                   const float *__restrict__ gout,
+                                                                   Records<float, true> rec, float *dw,
+                                                                   unsigned long long *dw_fixed, const DetHeader *hdr,
+                                                                   int TB, long long part_size, bool need_c,
+                                                                   bool dw_atomic, int num_groups) {
+  typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
+  constexpr int NP = kWave / P;  // pairs per step
+  extern __shared__ __align__(16) unsigned char smem[];
+  Acc *acc = reinterpret_cast<Acc *>(smem);
+  double scale = 1.0, inv_scale = 1.0;
+  if (FIXED) {
+    if (hdr->fallback_w) dw = nullptr;
+    scale = hdr->scale_w;
+    inv_scale = hdr->inv_scale_w;
+    if (!dw && !need_c) return;
+  }
+  const int group = xcd_tree_group(blockIdx.x, num_groups);
+  if (group < 0) return;
+  const int t0 = group * TB;
+  const int nt = min(TB, d.T - t0);
+  const uint32_t M = uint32_t(d.M), LM = uint32_t(d.L) * M;
+  if (dw) {
+    for (uint32_t i = threadIdx.x; i < uint32_t(nt) * LM; i += kForestThreads) acc[i] = Acc(0);
+    __syncthreads();
+  }
+  const long long s_begin = (long long)blockIdx.y * part_size;
+  const long long s_end = min(d.S, s_begin + part_size);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  constexpr int kWaves = kForestThreads / kWave;
+  const int pr = lane / P, e0 = (lane & (P - 1)) * 4;  // this lane's pair of a step and its first element of the row
+  const uint32_t key_mask = rec.key_mask();
+
+  struct Step {
+    long long at;  // record index of this lane's pair
+    bool on;
+    uint32_t a;
+    float mg;
+    Float4U gv;
+  };
+  auto issue = [&](Step &st, long long sb, int tl) {
+    const long long s_raw = sb + pr;
+    st.on = s_raw < s_end;
+    const long long s = st.on ? s_raw : s_end - 1;
+    st.at = (long long)(t0 + tl) * d.S + s;
+    st.a = rec.a[st.at];
+    st.mg = rec.margin[st.at];
+    const long long row = d.K == 1 ? (s * d.T + (t0 + tl)) * (long long)M : out_offset(d, s, t0 + tl, 0);
+    st.gv = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(gout + row + e0));
+  };
+  auto finish = [&](Step &st, int tl) {
+    const uint32_t cell = (uint32_t(tl) * uint32_t(d.L) + (st.a & key_mask)) * M + uint32_t(e0);
+    if (need_c) {
+      const Float4U wv = *reinterpret_cast<const Float4U *>(w + (long long)t0 * LM + cell);
+      float partial = wv[0] * st.gv[0];
+      partial = __builtin_fmaf(wv[1], st.gv[1], partial);
+      partial = __builtin_fmaf(wv[2], st.gv[2], partial);
+      partial = __builtin_fmaf(wv[3], st.gv[3], partial);
+      const float total = row_group_sum<P>(partial);
+      if (st.on && e0 == 0) rec.c[st.at] = ht_sign(st.mg) * total;
+    }
+    if (dw && st.on) {
+      const float a = ht_abs(st.mg);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float term = a * st.gv[i];
+        if (FIXED)
+          atomicAdd(reinterpret_cast<unsigned long long *>(acc) + cell + i, to_fixed(double(term), scale));
+        else
+          atomicAdd(reinterpret_cast<double *>(acc) + cell + i, double(term));
+      }
+    }
+  };
+
+  // steps of this wavefront: (sample block, tree) with the tree running fastest; two in flight
+  const long long first = s_begin + (long long)wave * NP;
+  const long long stride = (long long)kWaves * NP;
+  const long long nblk = first < s_end ? (s_end - first + stride - 1) / stride : 0;
+  const long long nsteps = nblk * nt;
+  auto where = [&](long long i, long long *sb, int *tl) {
+    const long long blk = i / nt;
+    *tl = int(i - blk * nt);
+    *sb = first + blk * stride;
+  };
+  Step s0, s1;
+  long long sb0 = 0, sb1 = 0;
+  int tl0 = 0, tl1 = 0;
+  if (nsteps > 0) {
+    where(0, &sb0, &tl0);
+    issue(s0, sb0, tl0);
+  }
+  for (long long i = 0; i < nsteps; i += 2) {
+    const bool second = i + 1 < nsteps;
+    if (second) {
+      where(i + 1, &sb1, &tl1);
+      issue(s1, sb1, tl1);
+    }
+    finish(s0, tl0);
+    if (i + 2 < nsteps) {
+      where(i + 2, &sb0, &tl0);
+      issue(s0, sb0, tl0);
+    }
+    if (second) finish(s1, tl1);
+  }
+
+  if (dw) {
+    __syncthreads();
     float *dst = dw + (long long)t0 * LM;
     const uint32_t n = uint32_t(nt) * LM;
     if (FIXED) {
@@ -1223,11 +1379,18 @@ static bool plan_trees(const ForestDims &d, bool need_dw, bool lean, TreePlan *p
   long long parts = 1;
   if (p->groups < kNumCUs) parts = (kNumCUs + p->groups - 1) / p->groups;
   const long long max_parts = (d.S + 4 * kForestThreads - 1) / (4 * kForestThreads);  // >= 4 samples per thread
-  if (keep && p->groups < kNumCUs) {  // the split that leaves the fewest CUs idle in the last round
+  if (p->groups < kNumCUs) {
+    // The split that leaves the fewest CUs idle in the last round. An XCD (32 CUs) takes ceil(groups / 8) of the tree
+    // groups, each times the sample parts, and a CU holds as many of these workgroups as its LDS and its 2048 thread
+    // slots allow.
+    const size_t lds = size_t(tb) * ((need_dw ? per_tree : 0) + (keep ? w_tree + size_t(d.V) * sizeof(double) : 0));
+    const long long per_cu = lds * 2 <= size_t(kLdsBytes) ? 2 : 1;
+    const long long cap = per_cu * (kNumCUs / kNumXCDs);
+    const long long xcd_groups = (p->groups + kNumXCDs - 1) / kNumXCDs;
     double best = -1.0;
     for (long long c = 1; c <= 16 && c <= max_parts; ++c) {
-      const long long wgs = c * p->groups, rounds = (wgs + kNumCUs - 1) / kNumCUs;
-      const double eff = double(wgs) / double(rounds * kNumCUs);
+      const long long rounds = (xcd_groups * c + cap - 1) / cap;
+      const double eff = double(c * p->groups) / double(rounds * cap * kNumXCDs);
       if (eff > best + 0.02) best = eff, parts = c;
     }
   }
@@ -1309,6 +1472,35 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
                            rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
                            uint32_t(thr_off), uint32_t(w_off));
       HT_LAUNCH_CHECK("forest backward (trees)");
+      return HT_OK;
+    }
+  }
+  if constexpr (std::is_same<Real, float>::value && COMPACT) {
+    // wide leaf rows: M = 4 * P, P a power of two
+    const int P4 = d.M / 4;
+    if (d.M % 4 == 0 && P4 >= 4 && P4 <= kWave && (P4 & (P4 - 1)) == 0 &&
+        (long long)p.TB * d.L * d.M < (1ll << 31) && reinterpret_cast<uintptr_t>(gout) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+      const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
+      const dim3 grid((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts);
+#define HT_WIDE(PP)                                                                                                   \
+  case PP: {                                                                                                          \
+    auto kernel = tree_wide_kernel<PP, FIXED>;                                                                        \
+    HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                                          \
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(p.lds)));                        \
+    hipLaunchKernelGGL(kernel, grid, dim3(kForestThreads), p.lds, stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB,   \
+                       p.part_size, need_c, p.parts > 1, p.groups);                                                   \
+    break;                                                                                                            \
+  }
+      switch (P4) {
+        HT_WIDE(4)
+        HT_WIDE(8)
+        HT_WIDE(16)
+        HT_WIDE(32)
+        HT_WIDE(64)
+      }
+#undef HT_WIDE
+      HT_LAUNCH_CHECK("forest backward (trees, wide rows)");
       return HT_OK;
     }
   }

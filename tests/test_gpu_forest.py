@@ -37,11 +37,30 @@ CASES = [
     # staged backward with a feature space too wide for the dX tile: dX by one global atomic per pair
     (600, 6000, [], 500, 4, [10]),
     (40, 5000, [8], 900, 3, [2]),
+    # wide leaf rows (a multiple of four that is four times a power of two), staged backward: several lanes per pair,
+    # one tree per wavefront step; with inner positions, ragged sample tails and 16 to 256 outputs per leaf
+    (9, 14, [37, 29], 31, 4, [4, 4]),
+    (1031, 9, [], 260, 3, [32]),
+    (3, 30, [70, 33], 50, 5, [8, 8]),      # the segmentation head's shape in small
+    (2500, 11, [], 110, 2, [128]),
+    (1300, 8, [], 210, 2, [256]),
 ]
 
 
 def _gpu(dev, *ts):
     return [t.to(dev) for t in ts]
+
+
+def _reference_gradients(x, thr, ordn, w, gout, fern):
+    """The oracle's gradients in the data's own precision -- the reference's serial loop -- and, for float32 data, how
+    far each of them is from the same loop run in float64: with thousands of terms per threshold the serial float32
+    sum is itself more than 1e-5 from the exact gradient, so the bar for the GPU (whose sums run in wider
+    accumulators) is 1e-5 plus that distance, never tighter than the reference is to the truth."""
+    ref = ho.backward(x, thr, ordn, w, gout, fern=fern)
+    if x.dtype == torch.float64:
+        return ref, (0.0, 0.0, 0.0)
+    exact = ho.backward(x.double(), thr.double(), ordn, w.double(), gout.double(), fern=fern)
+    return ref, tuple(rel_err(a.double(), b) for a, b in zip(ref, exact))
 
 
 @pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
@@ -71,15 +90,15 @@ def test_forward_and_maps_bit_exact(dev, case, dtype, fern):
 def test_backward_atomic(dev, case, dtype, fern):
     B, F, Kd, T, D, Md = case
     x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype)
-    rdx, rdthr, rdw = ho.backward(x, thr, ordn, w, gout, fern=fern)
+    (rdx, rdthr, rdw), slack = _reference_gradients(x, thr, ordn, w, gout, fern)
     gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
     pre = "fern_" if fern else "tree_"
     dx, dthr, dord, dw = getattr(ops, pre + "backward")(gx, True, gthr, True, gord, False, gw, True, gg)
     assert dord is None
     tol = 1e-5 if dtype == torch.float32 else 1e-12
-    assert rel_err(dx.cpu(), rdx) <= tol
-    assert rel_err(dthr.cpu(), rdthr) <= tol
-    assert rel_err(dw.cpu(), rdw) <= tol
+    assert rel_err(dx.cpu(), rdx) <= tol + slack[0]
+    assert rel_err(dthr.cpu(), rdthr) <= tol + slack[1]
+    assert rel_err(dw.cpu(), rdw) <= tol + slack[2]
 
 
 @pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
@@ -88,7 +107,7 @@ def test_backward_atomic(dev, case, dtype, fern):
 def test_backward_deterministic(dev, case, dtype, fern):
     B, F, Kd, T, D, Md = case
     x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype)
-    rdx, rdthr, rdw = ho.backward(x, thr, ordn, w, gout, fern=fern)
+    (rdx, rdthr, rdw), slack = _reference_gradients(x, thr, ordn, w, gout, fern)
     gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
     fn = getattr(ops, ("fern_" if fern else "tree_") + "backward_deterministic")
     runs = [fn(gx, True, gthr, True, gord, False, gw, True, gg) for _ in range(3)]
@@ -97,9 +116,9 @@ def test_backward_deterministic(dev, case, dtype, fern):
             assert (a is None and b is None) or torch.equal(a, b)
     dx, dthr, _, dw = runs[0]
     tol = 1e-5 if dtype == torch.float32 else 1e-12
-    assert rel_err(dx.cpu(), rdx) <= tol
-    assert rel_err(dw.cpu(), rdw) <= tol
-    assert rel_err(dthr.cpu(), rdthr) <= tol
+    assert rel_err(dx.cpu(), rdx) <= tol + slack[0]
+    assert rel_err(dw.cpu(), rdw) <= tol + slack[2]
+    assert rel_err(dthr.cpu(), rdthr) <= tol + slack[1]
     if F == 5000:
         # too wide for an on-chip dX tile: the sequential kernels add dX and dW terms in the CPU loop's order
         assert torch.equal(dx.cpu(), rdx)
@@ -210,7 +229,7 @@ def test_records_path(dev, case, dtype, fern):
     backward, atomic gradients within tolerance."""
     B, F, Kd, T, D, Md = case
     x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype)
-    rdx, rdthr, rdw = ho.backward(x, thr, ordn, w, gout, fern=fern)
+    (rdx, rdthr, rdw), slack = _reference_gradients(x, thr, ordn, w, gout, fern)
     gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
     pre = "fern_" if fern else "tree_"
     out, records = getattr(ops, pre + "forward_records")(gx, gthr, gord, gw)
@@ -221,16 +240,17 @@ def test_records_path(dev, case, dtype, fern):
     tol = 1e-5 if dtype == torch.float32 else 1e-12
     dx, dthr, dord, dw = bwd(records, False, gx, True, gthr, True, gord, False, gw, True, gg)
     assert dord is None
-    assert rel_err(dx.cpu(), rdx) <= tol and rel_err(dthr.cpu(), rdthr) <= tol and rel_err(dw.cpu(), rdw) <= tol
+    assert rel_err(dx.cpu(), rdx) <= tol + slack[0] and rel_err(dthr.cpu(), rdthr) <= tol + slack[1]
+    assert rel_err(dw.cpu(), rdw) <= tol + slack[2]
     det = bwd(records, True, gx, True, gthr, True, gord, False, gw, True, gg)
     ref = getattr(ops, pre + "backward_deterministic")(gx, True, gthr, True, gord, False, gw, True, gg)
     for a, b in zip(det, ref):
         assert (a is None and b is None) or torch.equal(a, b)
     # subsets of the gradients
     only_w = bwd(records, False, gx, False, gthr, False, gord, False, gw, True, gg)
-    assert only_w[0] is None and only_w[1] is None and rel_err(only_w[3].cpu(), rdw) <= tol
+    assert only_w[0] is None and only_w[1] is None and rel_err(only_w[3].cpu(), rdw) <= tol + slack[2]
     only_x = bwd(records, False, gx, True, gthr, False, gord, False, gw, False, gg)
-    assert only_x[3] is None and rel_err(only_x[0].cpu(), rdx) <= tol
+    assert only_x[3] is None and rel_err(only_x[0].cpu(), rdx) <= tol + slack[0]
 
 
 EMPTY = {"no samples": (0, 5, [], 3, 2, []), "no inner positions": (4, 5, [0], 3, 2, []),
