@@ -53,14 +53,14 @@ def _gpu(dev, *ts):
 
 def _reference_gradients(x, thr, ordn, w, gout, fern):
     """The oracle's gradients in the data's own precision -- the reference's serial loop -- and, for float32 data, how
-    far each of them is from the same loop run in float64: with thousands of terms per threshold the serial float32
+    far each of them is from the same loop run in float64 (returned third): with thousands of terms per threshold the serial float32
     sum is itself more than 1e-5 from the exact gradient, so the bar for the GPU (whose sums run in wider
     accumulators) is 1e-5 plus that distance, never tighter than the reference is to the truth."""
     ref = ho.backward(x, thr, ordn, w, gout, fern=fern)
     if x.dtype == torch.float64:
-        return ref, (0.0, 0.0, 0.0)
+        return ref, (0.0, 0.0, 0.0), ref
     exact = ho.backward(x.double(), thr.double(), ordn, w.double(), gout.double(), fern=fern)
-    return ref, tuple(rel_err(a.double(), b) for a, b in zip(ref, exact))
+    return ref, tuple(rel_err(a.double(), b) for a, b in zip(ref, exact)), exact
 
 
 @pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
@@ -90,7 +90,7 @@ def test_forward_and_maps_bit_exact(dev, case, dtype, fern):
 def test_backward_atomic(dev, case, dtype, fern):
     B, F, Kd, T, D, Md = case
     x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype)
-    (rdx, rdthr, rdw), slack = _reference_gradients(x, thr, ordn, w, gout, fern)
+    (rdx, rdthr, rdw), slack, exact = _reference_gradients(x, thr, ordn, w, gout, fern)
     gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
     pre = "fern_" if fern else "tree_"
     dx, dthr, dord, dw = getattr(ops, pre + "backward")(gx, True, gthr, True, gord, False, gw, True, gg)
@@ -99,6 +99,9 @@ def test_backward_atomic(dev, case, dtype, fern):
     assert rel_err(dx.cpu(), rdx) <= tol + slack[0]
     assert rel_err(dthr.cpu(), rdthr) <= tol + slack[1]
     assert rel_err(dw.cpu(), rdw) <= tol + slack[2]
+    # and without any slack against the float64 evaluation of the same gradients
+    for got, want in zip((dx, dthr, dw), exact):
+        assert rel_err(got.cpu().double(), want.double()) <= tol
 
 
 @pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
@@ -107,7 +110,7 @@ def test_backward_atomic(dev, case, dtype, fern):
 def test_backward_deterministic(dev, case, dtype, fern):
     B, F, Kd, T, D, Md = case
     x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype)
-    (rdx, rdthr, rdw), slack = _reference_gradients(x, thr, ordn, w, gout, fern)
+    (rdx, rdthr, rdw), slack, exact = _reference_gradients(x, thr, ordn, w, gout, fern)
     gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
     fn = getattr(ops, ("fern_" if fern else "tree_") + "backward_deterministic")
     runs = [fn(gx, True, gthr, True, gord, False, gw, True, gg) for _ in range(3)]
@@ -119,6 +122,8 @@ def test_backward_deterministic(dev, case, dtype, fern):
     assert rel_err(dx.cpu(), rdx) <= tol + slack[0]
     assert rel_err(dw.cpu(), rdw) <= tol + slack[2]
     assert rel_err(dthr.cpu(), rdthr) <= tol + slack[1]
+    for got, want in zip((dx, dthr, dw), exact):
+        assert rel_err(got.cpu().double(), want.double()) <= tol
     if F == 5000:
         # too wide for an on-chip dX tile: the sequential kernels add dX and dW terms in the CPU loop's order
         assert torch.equal(dx.cpu(), rdx)
@@ -229,7 +234,7 @@ def test_records_path(dev, case, dtype, fern):
     backward, atomic gradients within tolerance."""
     B, F, Kd, T, D, Md = case
     x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, dtype)
-    (rdx, rdthr, rdw), slack = _reference_gradients(x, thr, ordn, w, gout, fern)
+    (rdx, rdthr, rdw), slack, exact = _reference_gradients(x, thr, ordn, w, gout, fern)
     gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
     pre = "fern_" if fern else "tree_"
     out, records = getattr(ops, pre + "forward_records")(gx, gthr, gord, gw)
