@@ -50,6 +50,9 @@ SIGNATURES = {
                                      _P]),
     "ht_forest_backward_workspace": (_SZ, [ctypes.POINTER(ForestShape), _I, _I, _I, _I]),
     "ht_forest_backward": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _SZ, _P]),
+    "ht_forest_backward_image_supported": (_I, [ctypes.POINTER(ForestShape), ctypes.POINTER(TileShape), _I, _I, _I, _I]),
+    "ht_forest_backward_image": (_I, [ctypes.POINTER(ForestShape), ctypes.POINTER(TileShape), _P, _P, _P, _P, _P, _P, _P,
+                                      _P, _I, _P, _SZ, _P]),
     "ht_forest_records_bytes": (_SZ, [ctypes.POINTER(ForestShape)]),
     "ht_forest_forward_records": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _SZ, _P, _SZ, _P]),
     "ht_forest_backward_records_workspace": (_SZ, [ctypes.POINTER(ForestShape), _I, _I, _I, _I]),

@@ -284,6 +284,46 @@ int ht_forest_backward(const ht_forest_shape *s, const void *x, const void *thr,
                                  workspace_bytes, st);
 }
 
+static int image_backward_geometry(const ht_forest_shape *s, const ht_tile_shape *g, ForestDims *d, ImageStore *img) {
+  int rc = make_dims(s, d);
+  if (rc != HT_OK) return rc;
+  bool clear = false;
+  if ((rc = make_image_store(g, *d, s->B, img, &clear)) != HT_OK) return rc;
+  if (g->elem_size != (s->dtype == HT_F32 ? 4 : 8))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: the element size of the tile geometry must be that of the forest's data type.");
+  return HT_OK;
+}
+
+int ht_forest_backward_image_supported(const ht_forest_shape *s, const ht_tile_shape *g, int mode, int need_dx,
+                                       int need_dthr, int need_dw) {
+  (void)need_dthr;
+  ForestDims d;
+  ImageStore img{};
+  if (image_backward_geometry(s, g, &d, &img) != HT_OK) return 0;
+  if (s->dtype != HT_F32) return 0;
+  return forest_backward_image_ok<float>(d, mode, need_dx != 0, need_dw != 0, img) ? 1 : 0;
+}
+
+int ht_forest_backward_image(const ht_forest_shape *s, const ht_tile_shape *g, const void *x, const void *thr,
+                             const int64_t *ord, const void *w, const void *gout_image, void *dx, void *dthr, void *dw,
+                             int mode, void *workspace, size_t workspace_bytes, void *stream) {
+  ForestDims d;
+  ImageStore img{};
+  int rc = image_backward_geometry(s, g, &d, &img);
+  if (rc != HT_OK) return rc;
+  if (mode != HT_BACKWARD_ATOMIC && mode != HT_BACKWARD_DETERMINISTIC)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: unknown backward mode.");
+  if (!is_empty(d) && (!x || !thr || !ord || !w || !gout_image))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (!is_empty(d) && (s->dtype != HT_F32 || !forest_backward_image_ok<float>(d, mode, dx != nullptr, dw != nullptr, img)))
+    return fail(HT_ERR_INVALID_ARGUMENT,
+                "Error: this shape, data type or mode cannot read the upstream gradient as an image (ask "
+                "ht_forest_backward_image_supported; contract the gradient and call ht_forest_backward instead).");
+  return forest_backward<float>(d, s->kind == HT_FERN, (const float *)x, (const float *)thr, ord, (const float *)w,
+                                (const float *)gout_image, (float *)dx, (float *)dthr, (float *)dw, mode, workspace,
+                                workspace_bytes, static_cast<hipStream_t>(stream), &img);
+}
+
 size_t ht_forest_maps_workspace(const ht_forest_shape *s) {
   ForestDims d;
   if (make_dims(s, &d) != HT_OK) return 0;

@@ -113,7 +113,11 @@ size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bo
 template <typename Real>
 int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
                     const Real *gout, Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes,
-                    hipStream_t stream);
+                    hipStream_t stream, const ImageStore *gout_image = nullptr);
+// gout_image: gout is the image [B, T, *size] whose contraction by that tile geometry is the upstream gradient
+// [B, T, *tiles, *window]; served where forest_backward_image_ok says so.
+template <typename Real>
+bool forest_backward_image_ok(const ForestDims &d, int mode, bool need_dx, bool need_dw, const ImageStore &img);
 
 // Training path: backward from the records a forward pass wrote (0 bytes: not offered for this shape).
 template <typename Real>

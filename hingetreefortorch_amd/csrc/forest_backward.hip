@@ -795,13 +795,17 @@ __device__ __forceinline__ float row_group_sum(float v) {
   return v;
 }
 
-template <int P, bool FIXED>
+//
+// IMAGE: the upstream gradient is the image [B, T, *size] of which the tile-major [B, T, *tiles, *window] is the
+// contraction (tile-shaped outputs per leaf); a lane's four outputs are a 16-byte run of an image row (the window's,
+// the padding's and the image's innermost extents are multiples of four), read as zero outside the image.
+template <int P, bool FIXED, bool IMAGE>
 __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d, const float *__restrict__ w,
                                                                    const float *__restrict__ gout,
                                                                    Records<float, true> rec, float *dw,
                                                                    unsigned long long *dw_fixed, const DetHeader *hdr,
                                                                    int TB, long long part_size, bool need_c,
-                                                                   bool dw_atomic, int num_groups) {
+                                                                   bool dw_atomic, int num_groups, ImageStore img) {
   typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
   constexpr int NP = kWave / P;  // pairs per step
   extern __shared__ __align__(16) unsigned char smem[];
@@ -844,8 +848,18 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
     st.at = (long long)(t0 + tl) * d.S + s;
     st.a = rec.a[st.at];
     st.mg = rec.margin[st.at];
-    const long long row = d.K == 1 ? (s * d.T + (t0 + tl)) * (long long)M : out_offset(d, s, t0 + tl, 0);
-    st.gv = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(gout + row + e0));
+    if constexpr (IMAGE) {
+      const long long b = s / d.K;
+      const long long at = img.offset(int(s - b * d.K), e0);
+      const Float4U zero = {0.f, 0.f, 0.f, 0.f};
+      st.gv = zero;
+      if (at >= 0)
+        st.gv = __builtin_nontemporal_load(
+            reinterpret_cast<const Float4U *>(gout + (b * d.T + (t0 + tl)) * img.plane + at));
+    } else {
+      const long long row = d.K == 1 ? (s * d.T + (t0 + tl)) * (long long)M : out_offset(d, s, t0 + tl, 0);
+      st.gv = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(gout + row + e0));
+    }
   };
   auto finish = [&](Step &st, int tl) {
     const uint32_t cell = (uint32_t(tl) * uint32_t(d.L) + (st.a & key_mask)) * M + uint32_t(e0);
@@ -1428,11 +1442,27 @@ int launch_tree_kernel_u(const ForestDims &d, const TreePlan &p, int P, const Re
   return HT_OK;
 }
 
+// Shapes of tree_wide_kernel: M = 4 * P with P a power of two from 4 to 64, leaf offsets of a tree group in 32 bits.
+static bool wide_rows_ok(const ForestDims &d, const TreePlan &p) {
+  const int P4 = d.M / 4;
+  return d.M % 4 == 0 && P4 >= 4 && P4 <= kWave && (P4 & (P4 - 1)) == 0 && (long long)p.TB * d.L * d.M < (1ll << 31);
+}
+
+// gout_image: the upstream gradient is stored as the image of the tile geometry (only tree_wide_kernel reads it so).
 template <typename Real, bool COMPACT, bool FIXED>
 int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, const Real *gout,
                        Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
-                       bool need_c, Real *dthr, bool *dthr_done, hipStream_t stream) {
+                       bool need_c, Real *dthr, bool *dthr_done, hipStream_t stream, const ImageStore *gout_image) {
   *dthr_done = false;
+  if constexpr (std::is_same<Real, float>::value && COMPACT) {
+    if (gout_image != nullptr &&
+        (d.K == 1 || !wide_rows_ok(d, p) || reinterpret_cast<uintptr_t>(gout) % 16 != 0 ||
+         reinterpret_cast<uintptr_t>(w) % 16 != 0))
+      return fail(HT_ERR_RUNTIME, "Error: this shape cannot read the upstream gradient as an image.");
+  } else {
+    if (gout_image != nullptr)
+      return fail(HT_ERR_RUNTIME, "Error: this shape cannot read the upstream gradient as an image.");
+  }
   if constexpr (std::is_same<Real, float>::value && COMPACT) {
     // the specialised kernel: contiguous rows, a power-of-two tree group, 32-bit offsets inside a block and a group
     int log2_tb = 0;
@@ -1478,18 +1508,18 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
   if constexpr (std::is_same<Real, float>::value && COMPACT) {
     // wide leaf rows: M = 4 * P, P a power of two
     const int P4 = d.M / 4;
-    if (d.M % 4 == 0 && P4 >= 4 && P4 <= kWave && (P4 & (P4 - 1)) == 0 &&
-        (long long)p.TB * d.L * d.M < (1ll << 31) && reinterpret_cast<uintptr_t>(gout) % 16 == 0 &&
+    if (wide_rows_ok(d, p) && reinterpret_cast<uintptr_t>(gout) % 16 == 0 &&
         reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+      const ImageStore img = gout_image ? *gout_image : ImageStore{};
       const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
       const dim3 grid((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts);
 #define HT_WIDE(PP)                                                                                                   \
   case PP: {                                                                                                          \
-    auto kernel = tree_wide_kernel<PP, FIXED>;                                                                        \
+    auto kernel = gout_image ? tree_wide_kernel<PP, FIXED, true> : tree_wide_kernel<PP, FIXED, false>;                \
     HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                                          \
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(p.lds)));                        \
     hipLaunchKernelGGL(kernel, grid, dim3(kForestThreads), p.lds, stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB,   \
-                       p.part_size, need_c, p.parts > 1, p.groups);                                                   \
+                       p.part_size, need_c, p.parts > 1, p.groups, img);                                              \
     break;                                                                                                            \
   }
       switch (P4) {
@@ -1588,8 +1618,10 @@ int launch_absmax(const Real *p, long long n, unsigned long long *slot, hipStrea
 template <typename Real, bool FERN, bool COMPACT, bool FIXED>
 int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, const Real *gout,
                     Real *dx, Real *dthr, Real *dw, Records<Real, COMPACT> rec, bool walk, void *fixed_ws,
-                    hipStream_t stream) {
+                    hipStream_t stream, const ImageStore *gout_image = nullptr) {
   int rc = HT_OK;
+  if (FIXED && gout_image != nullptr)
+    return fail(HT_ERR_RUNTIME, "Error: the deterministic mode cannot read the upstream gradient as an image.");
   if (walk && (rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream)) != HT_OK) return rc;
   const bool need_c = dx || dthr;
   const long long pairs = (long long)d.T * d.S;
@@ -1621,7 +1653,8 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
   }
 
   bool dthr_done = false;
-  rc = launch_tree_kernel<Real, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, dthr, &dthr_done, stream);
+  rc = launch_tree_kernel<Real, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, need_c, dthr, &dthr_done, stream,
+                                                gout_image);
   if (rc != HT_OK) return rc;
 
   if (FIXED) {
@@ -1755,12 +1788,15 @@ size_t route_bytes(const ForestDims &d, Route r, bool need_dthr, bool need_dw, b
 template <typename Real>
 int run_route(const ForestDims &d, Route route, bool fern, const Real *x, const Node<Real> *nodes, const Real *w,
               const Real *gout, Real *dx, Real *dthr, Real *dw, void *saved, void *scratch, bool walk,
-              hipStream_t stream) {
+              hipStream_t stream, const ImageStore *gout_image = nullptr) {
+  if (gout_image != nullptr && route != Route::kStaged)
+    return fail(HT_ERR_RUNTIME, "Error: this shape cannot read the upstream gradient as an image.");
   void *fixed_ws = static_cast<unsigned char *>(scratch) + records_scratch_bytes<Real>(d);
   const bool compact = compact_ok(d);
 #define HT_STAGED(FERN_, COMPACT_, FIXED_)                                                            \
   backward_staged<Real, FERN_, COMPACT_, FIXED_>(d, x, nodes, w, gout, dx, dthr, dw,                  \
-                                                 carve_records<Real, COMPACT_>(d, saved, scratch), walk, fixed_ws, stream)
+                                                 carve_records<Real, COMPACT_>(d, saved, scratch), walk, fixed_ws, stream, \
+                                                 gout_image)
 #define HT_SEQ(FERN_, COMPACT_)                                                                       \
   backward_sequential<Real, FERN_, COMPACT_>(d, x, nodes, w, gout, dx, dthr, dw,                      \
                                              carve_records<Real, COMPACT_>(d, saved, scratch), walk, stream)
@@ -1805,12 +1841,27 @@ size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bo
   return packed_nodes_bytes<Real>(d) + route_bytes<Real>(d, r, need_dthr, need_dw, false);
 }
 
+// Whether the stateless backward can read the upstream gradient as the image of this tile geometry: atomic mode on
+// the staged kernels, float data with compact records, leaf rows that tree_wide_kernel serves, and 16-byte runs that
+// neither straddle a window row nor leave the image rows misaligned.
+template <typename Real>
+bool forest_backward_image_ok(const ForestDims &d, int mode, bool need_dx, bool need_dw, const ImageStore &img) {
+  if (!std::is_same<Real, float>::value || is_empty(d) || d.K == 1 || img.nd == 0) return false;
+  if (mode != HT_BACKWARD_ATOMIC || !compact_ok(d)) return false;
+  if (pick_route<Real>(d, mode, need_dx, need_dw, false) != Route::kStaged) return false;
+  TreePlan plan;
+  if (!plan_trees(d, need_dw, false, &plan) || !wide_rows_ok(d, plan)) return false;
+  return img.win[2] % 4 == 0 && img.pad[2] % 4 == 0 && img.size[2] % 4 == 0 && img.plane % 4 == 0;
+}
+
 template <typename Real>
 int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
                     const Real *gout, Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes,
-                    hipStream_t stream) {
+                    hipStream_t stream, const ImageStore *gout_image) {
   int rc;
   const Route route = is_empty(d) ? Route::kFused : pick_route<Real>(d, mode, dx != nullptr, dw != nullptr, false);
+  if (gout_image != nullptr && !is_empty(d) && !forest_backward_image_ok<Real>(d, mode, dx != nullptr, dw != nullptr, *gout_image))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: this shape cannot read the upstream gradient as an image.");
   bool done;
   if ((rc = clear_gradients<Real>(d, route, dx, dthr, dw, stream, &done)) != HT_OK || done) return rc;
   const size_t node_bytes = packed_nodes_bytes<Real>(d);
@@ -1821,7 +1872,7 @@ int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *t
   const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
   unsigned char *saved = static_cast<unsigned char *>(ws) + node_bytes;
   unsigned char *scratch = saved + records_saved_bytes<Real>(d);
-  return run_route<Real>(d, route, fern, x, nodes, w, gout, dx, dthr, dw, saved, scratch, true, stream);
+  return run_route<Real>(d, route, fern, x, nodes, w, gout, dx, dthr, dw, saved, scratch, true, stream, gout_image);
 }
 
 template <typename Real>
@@ -1858,7 +1909,8 @@ int forest_backward_records(const ForestDims &d, bool fern, const Real *w, const
   template size_t forest_backward_workspace<Real>(const ForestDims &, int, bool, bool, bool);                         \
   template int forest_backward<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,           \
                                      const Real *, const Real *, Real *, Real *, Real *, int, void *, size_t,         \
-                                     hipStream_t);                                                                    \
+                                     hipStream_t, const ImageStore *);                                                \
+  template bool forest_backward_image_ok<Real>(const ForestDims &, int, bool, bool, const ImageStore &);                                                                 \
   template size_t forest_records_bytes<Real>(const ForestDims &);                                                     \
   template size_t forest_backward_records_workspace<Real>(const ForestDims &, int, bool, bool, bool);                 \
   template int forest_backward_records<Real>(const ForestDims &, bool, const Real *, const Real *, const void *,      \

@@ -274,8 +274,8 @@ class _Contract(torch.autograd.Function):
 
 class _ForestExpandedFunction(torch.autograd.Function):
     """Forest with tile-shaped outputs per leaf followed by Expand, as one operator: the forward pass stores the image
-    directly (the tile-major intermediate [B, T, *tiles, *window] is never written); the backward pass contracts the
-    upstream gradient and runs the forest's backward. Same values as Expand(padding)(HingeTree.apply(...)), which is
+    directly (the tile-major intermediate [B, T, *tiles, *window] is never written); the backward pass reads the upstream
+    gradient as the image where the library serves the shape, and otherwise contracts it and runs the forest's backward. Same values as Expand(padding)(HingeTree.apply(...)), which is
     how the reference's segmentation model composes the two (rcc/Net.py:99-109)."""
     _prefix = None
 
@@ -290,10 +290,9 @@ class _ForestExpandedFunction(torch.autograd.Function):
     def _backward(cls, ctx, outDataGrad):
         inData, inThresholds, inOrdinals, inWeights = ctx.saved_tensors
         need = ctx.needs_input_grad
-        tiles = _ops.contract(outDataGrad.contiguous(), list(inWeights.shape[2:]), ctx.padding)
-        name = "backward_deterministic" if _is_deterministic() else "backward"
-        grads = getattr(_ops, f"{cls._prefix}_{name}")(inData, need[0], inThresholds, need[1], inOrdinals, need[2],
-                                                      inWeights, need[3], tiles)
+        grads = getattr(_ops, f"{cls._prefix}_backward_expanded")(
+            _is_deterministic(), ctx.padding, inData, need[0], inThresholds, need[1], inOrdinals, need[2], inWeights,
+            need[3], outDataGrad.contiguous())
         return tuple(grads) + (None,)
 
 

@@ -460,6 +460,49 @@ def _backward(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, 
     return [dx, dthr, None, dw]
 
 
+def _backward_expanded(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad,
+                       inWeights, bInWeightsGrad, outImageGrad, padding):
+    """backward(..., contract(outImageGrad, window, padding)): the gradients of `_forward_expanded`. Where the library
+    can read the upstream gradient as the image (ht_forest_backward_image_supported) the tile-major gradient is never
+    written; every other shape, data type and mode takes the two calls. No counterpart in the reference, whose
+    autograd graph runs contract and the forest backward back to back (_HingeTree.py:54-60, rcc/Net.py:99-109)."""
+    padding = [int(v) for v in padding]
+    nd = len(padding)
+    window = [int(v) for v in inWeights.shape[2:]]
+    tiles = [int(v) for v in inData.shape[2:]]
+    fused = (nd in (2, 3) and len(window) == nd and len(tiles) == nd and all(p >= 0 for p in padding)
+             and outImageGrad.is_contiguous() and outImageGrad.dtype == inData.dtype == torch.float32
+             and outImageGrad.device == inData.device and not bInOrdinalsGrad
+             and inData.numel() > 0 and inWeights.numel() > 0)
+    if fused:
+        _common_checks([inData, inThresholds, inWeights], inOrdinals, True)
+        shape, out_sizes = _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights)
+        size = [t * w - ((2 * p) // w) * w for t, w, p in zip(tiles, window, padding)]
+        fused = list(outImageGrad.shape) == list(out_sizes[:2]) + size
+    if fused:
+        geom = L.TileShape()
+        geom.planes, geom.nd, geom.elem_size = int(shape.B) * int(shape.T), nd, inData.element_size()
+        for i in range(nd):
+            geom.size[i], geom.tiles[i], geom.window[i], geom.padding[i] = size[i], tiles[i], window[i], padding[i]
+        lib = L.load()
+        needs = (int(bool(bInDataGrad)), int(bool(bInThresholdsGrad)), int(bool(bInWeightsGrad)))
+        fused = lib.ht_forest_backward_image_supported(ctypes.byref(shape), ctypes.byref(geom), mode, *needs) == 1
+    if not fused:
+        tiled = contract(outImageGrad.contiguous(), window, padding)
+        return _backward(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals, bInOrdinalsGrad,
+                         inWeights, bInWeightsGrad, tiled)
+    with torch.cuda.device(inData.device):
+        dx = torch.empty_like(inData) if bInDataGrad else None
+        dthr = torch.empty_like(inThresholds) if bInThresholdsGrad else None
+        dw = torch.empty_like(inWeights) if bInWeightsGrad else None
+        nbytes = lib.ht_forest_backward_workspace(ctypes.byref(shape), mode, *needs)
+        ws = _workspace(nbytes, inData.device)
+        L.check(lib.ht_forest_backward_image(ctypes.byref(shape), ctypes.byref(geom), _ptr(inData), _ptr(inThresholds),
+                                             _ptr(inOrdinals), _ptr(inWeights), _ptr(outImageGrad), _ptr(dx), _ptr(dthr),
+                                             _ptr(dw), mode, _ptr(ws), nbytes, _stream(inData.device)))
+    return [dx, dthr, None, dw]
+
+
 def _forward_records(kind, inData, inThresholds, inOrdinals, inWeights):
     """Forward that also returns the walk records for `_backward_records` (None where the library does not offer
     them). Not part of the reference's module: its backward walks the trees again (hingetree_gpu.cu:619-730)."""
@@ -609,6 +652,17 @@ def tree_forward_expanded(inData, inThresholds, inOrdinals, inWeights, padding):
 
 def fern_forward_expanded(inData, inThresholds, inOrdinals, inWeights, padding):
     return _forward_expanded(L.HT_FERN, inData, inThresholds, inOrdinals, inWeights, padding)
+
+
+def tree_backward_expanded(deterministic, padding, *args):
+    """Gradients of tree_forward_expanded; args as for tree_backward with the image gradient last."""
+    mode = L.HT_BACKWARD_DETERMINISTIC if deterministic else L.HT_BACKWARD_ATOMIC
+    return _backward_expanded(L.HT_TREE, mode, *args, padding)
+
+
+def fern_backward_expanded(deterministic, padding, *args):
+    mode = L.HT_BACKWARD_DETERMINISTIC if deterministic else L.HT_BACKWARD_ATOMIC
+    return _backward_expanded(L.HT_FERN, mode, *args, padding)
 
 
 def tree_forward_records(inData, inThresholds, inOrdinals, inWeights):

@@ -92,6 +92,20 @@ int ht_forest_backward(const ht_forest_shape *s, const void *x, const void *thr,
                        const void *gout, void *dx, void *dthr, void *dw, int mode, void *workspace,
                        size_t workspace_bytes, void *stream);
 
+/* ht_forest_backward whose upstream gradient is still the image [B, T, *size] (the gradient of what
+ * ht_forest_forward_image stored): one call in place of the pair contract2d_gpu / contract3d_gpu (expand_gpu.cu:110-151,
+ * 198-295, reached through _Expand.backward, _HingeTree.py:54-60) + hingetree_gpu_backward (hingetree_gpu.cu:619-730) -- the tile-major
+ * [B, T, *tiles, *window] gradient is never written; image positions outside the tiles are not read. Same workspace
+ * as ht_forest_backward. Served for float32 data in atomic mode with 16 to 256 outputs per leaf (four times a power of
+ * two) whose innermost window, padding and image extents are multiples of four; ht_forest_backward_image_supported
+ * returns 1 for those and 0 otherwise (contract the gradient and call ht_forest_backward then), and
+ * ht_forest_backward_image fails with HT_ERR_INVALID_ARGUMENT where it would return 0. */
+int ht_forest_backward_image_supported(const ht_forest_shape *s, const ht_tile_shape *g, int mode, int need_dx,
+                                       int need_dthr, int need_dw);
+int ht_forest_backward_image(const ht_forest_shape *s, const ht_tile_shape *g, const void *x, const void *thr,
+                             const int64_t *ord, const void *w, const void *gout_image, void *dx, void *dthr, void *dw,
+                             int mode, void *workspace, size_t workspace_bytes, void *stream);
+
 /* Training path, no counterpart in the reference (whose backward walks every tree again, hingetree_gpu.cu:619-730):
  * ht_forest_forward_records is ht_forest_forward that also writes what its walks found -- leaf key, selected vertex,
  * its ordinal and the signed margin of every (tree, sample) pair -- into `records`, an opaque device buffer of

@@ -134,6 +134,102 @@ def test_forward_expanded_equals_forward_then_expand(dev, case, dtype, fern):
     assert torch.equal(two.cpu(), want) and torch.equal(one.cpu(), want)
 
 
+BACKWARD_EXPANDED = [
+    # B, F, tiles, T, depth, window, padding, whether the library reads the image gradient directly (float32, atomic)
+    (2, 7, [40, 44], 90, 3, [8, 8], [0, 0], True),
+    (3, 5, [36, 30], 100, 2, [4, 4], [4, 8], True),            # cropped borders: runs outside the image read 0
+    (1, 4, [8, 9, 10], 400, 2, [2, 2, 4], [0, 1, 4], True),    # 3-d, 16 outputs per leaf
+    (2, 7, [40, 44], 90, 3, [8, 8], [3, 2], False),            # innermost padding not a multiple of four
+    (2, 7, [40, 44], 90, 3, [8, 6], [0, 0], False),            # 48 outputs per leaf: not four times a power of two
+    (2, 6, [3, 4], 2, 3, [2, 3], [1, 0], False),               # small: the single-launch backward
+]
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("case", BACKWARD_EXPANDED, ids=[f"b{i}" for i in range(len(BACKWARD_EXPANDED))])
+def test_backward_expanded_equals_contract_then_backward(dev, case, fern):
+    """Gradients from the image-shaped upstream gradient: the oracle's contract + backward within 1e-5, on the path
+    that reads the image inside the tree kernel where the library offers it and on the two-call path elsewhere; all
+    subsets of the gradients; float64 and the deterministic mode (two calls) agree with their own two-call results."""
+    import ctypes
+    from hingetreefortorch_amd import _lib as L
+    from conftest import rel_err
+    B, F, tiles, T, depth, window, padding, fused = case
+    g = torch.Generator().manual_seed(11)
+    V = depth if fern else 2 ** depth - 1
+    x = torch.randn([B, F] + tiles, generator=g)
+    thr = (2 * torch.rand([T, V], generator=g) - 1)
+    ordn = torch.randint(0, F, [T, V], generator=g, dtype=torch.int64)
+    w = torch.randn([T, 2 ** depth] + window, generator=g)
+    size = [t * k - ((2 * p) // k) * k for t, k, p in zip(tiles, window, padding)]
+    gimg = torch.randn([B, T] + size, generator=g)
+    pre = "fern" if fern else "tree"
+
+    shape = L.ForestShape()
+    shape.kind, shape.dtype = (L.HT_FERN if fern else L.HT_TREE), L.HT_F32
+    K, M = int(np.prod(tiles)), int(np.prod(window))
+    shape.B, shape.F, shape.K, shape.T, shape.depth, shape.M = B, F, K, T, depth, M
+    geom = L.TileShape()
+    geom.planes, geom.nd, geom.elem_size = B * T, len(tiles), 4
+    for i in range(len(tiles)):
+        geom.size[i], geom.tiles[i], geom.window[i], geom.padding[i] = size[i], tiles[i], window[i], padding[i]
+    lib = L.load()
+    ask = lambda mode: lib.ht_forest_backward_image_supported(ctypes.byref(shape), ctypes.byref(geom), mode, 1, 1, 1)
+    assert ask(L.HT_BACKWARD_ATOMIC) == int(fused)
+    assert ask(L.HT_BACKWARD_DETERMINISTIC) == 0
+    shape.dtype, geom.elem_size = L.HT_F64, 8
+    assert ask(L.HT_BACKWARD_ATOMIC) == 0
+
+    gtiles = ho.contract(gimg, window, padding)
+    want = ho.backward(x, thr, ordn, w, gtiles, fern=fern)
+    exact = ho.backward(x.double(), thr.double(), ordn, w.double(), gtiles.double(), fern=fern)
+    d = [t.to(dev) for t in (x, thr, ordn, w)]
+    gi = gimg.to(dev)
+    bwd = getattr(ops, pre + "_backward_expanded")
+    dx, dthr, dord, dw = bwd(False, padding, d[0], True, d[1], True, d[2], False, d[3], True, gi)
+    assert dord is None
+    for got, ref, ex in zip((dx, dthr, dw), want, exact):
+        assert got.shape == ref.shape
+        assert rel_err(got.cpu().double(), ex) <= 1e-5
+        assert rel_err(got.cpu(), ref) <= 1e-5 + rel_err(ref.double(), ex)
+    only_w = bwd(False, padding, d[0], False, d[1], False, d[2], False, d[3], True, gi)
+    assert only_w[0] is None and only_w[1] is None and rel_err(only_w[3].cpu().double(), exact[2]) <= 1e-5
+    only_x = bwd(False, padding, d[0], True, d[1], False, d[2], False, d[3], False, gi)
+    assert only_x[3] is None and only_x[1] is None and rel_err(only_x[0].cpu().double(), exact[0]) <= 1e-5
+    # the deterministic mode and float64 take contract + backward: the same bits as the two calls made by hand
+    det = bwd(True, padding, d[0], True, d[1], True, d[2], False, d[3], True, gi)
+    two = getattr(ops, pre + "_backward_deterministic")(d[0], True, d[1], True, d[2], False, d[3], True,
+                                                        ops.contract(gi, window, padding))
+    for a, b in zip(det, two):
+        assert (a is None and b is None) or torch.equal(a, b)
+    d64 = [t.double() if t.is_floating_point() else t for t in d]
+    got64 = bwd(False, padding, d64[0], True, d64[1], True, d64[2], False, d64[3], True, gi.double())
+    for got, ex in zip((got64[0], got64[1], got64[3]), exact):
+        assert rel_err(got.cpu(), ex) <= 1e-12
+
+
+def test_backward_image_entry_refuses_unserved_shapes(dev):
+    """The C entry point fails loudly (ValueError through the status code) for what _supported answers 0 to."""
+    import ctypes
+    from hingetreefortorch_amd import _lib as L
+    shape = L.ForestShape()
+    shape.kind, shape.dtype = L.HT_TREE, L.HT_F32
+    shape.B, shape.F, shape.K, shape.T, shape.depth, shape.M = 2, 6, 12, 2, 3, 6
+    geom = L.TileShape()
+    geom.planes, geom.nd, geom.elem_size = 4, 2, 4
+    for i, (n, t, k, p) in enumerate(zip([6, 12], [3, 4], [2, 3], [0, 0])):
+        geom.size[i], geom.tiles[i], geom.window[i], geom.padding[i] = n, t, k, p
+    buf = torch.zeros(4096, device=dev)
+    ordn = torch.zeros(64, dtype=torch.int64, device=dev)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    lib = L.load()
+    rc = lib.ht_forest_backward_image(ctypes.byref(shape), ctypes.byref(geom), P(buf), P(buf), P(ordn), P(buf), P(buf),
+                                      P(buf), None, None, L.HT_BACKWARD_ATOMIC, P(buf), 4096 * 4, None)
+    assert rc == L.HT_ERR_INVALID_ARGUMENT
+    with pytest.raises(ValueError, match="cannot read the upstream gradient as an image"):
+        L.check(rc)
+
+
 def test_expanded_module_and_gradients(dev):
     from RandomHingeForest import RandomHingeForest, RandomHingeForestExpanded
     torch.manual_seed(3)
