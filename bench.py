@@ -334,6 +334,12 @@ def bench_tiles(torch, ops, dev, args):
                        ops.expand(ops.tree_forward(x, thr, ordn, wts), [0, 0]))
     two_ms = _timed(torch, lambda: ops.expand(ops.tree_forward(x, thr, ordn, wts), [0, 0]), args.steps, args.warmup)
     one_ms = _timed(torch, lambda: ops.tree_forward_expanded(x, thr, ordn, wts, [0, 0]), args.steps, args.warmup)
+    # ... and its backward from the gradient of the image: contract + backward against the one call that reads the image
+    gimg = torch.randn([B, T, H, W], generator=gg, device=dev)
+    bwd_two_ms = _timed(torch, lambda: ops.tree_backward(x, True, thr, True, ordn, False, wts, True,
+                                                         ops.contract(gimg, [P, P], [0, 0])), args.steps, args.warmup)
+    bwd_one_ms = _timed(torch, lambda: ops.tree_backward_expanded(False, [0, 0], x, True, thr, True, ordn, False, wts,
+                                                                  True, gimg), args.steps, args.warmup)
     return {
         "metric": "contract + expand GB/s (tiles [8,100,64,64,8,8] <-> images [8,100,512,512])",
         "value": 2 * nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -344,6 +350,9 @@ def bench_tiles(torch, ops, dev, args):
         "forest_then_expand": {"ms": two_ms, "what": "tree_forward [8,100,64,64] x 100 trees of depth 6 x [8,8] outputs, then expand"},
         "forest_expanded": {"ms": one_ms, "what": "the same image from one pass (tree_forward_expanded)",
                             "gbps": (nbytes // 2 + x.numel() * 4) / (one_ms * 1e-3) / 1e9},
+        "contract_then_backward": {"ms": bwd_two_ms, "what": "contract of the image gradient, then tree_backward (x, thresholds, leaf weights)"},
+        "backward_expanded": {"ms": bwd_one_ms, "what": "the same gradients from one call that reads the image gradient (tree_backward_expanded)",
+                              "gbps": (nbytes // 2) / (bwd_one_ms * 1e-3) / 1e9},
         "roofline": {"bound": "hbm", "kernel": "tile_permute_kernel", "achieved": 2 * nbytes / (ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": 2 * nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": None, "algorithmic_bytes": nbytes},
