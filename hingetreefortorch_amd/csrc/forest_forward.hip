@@ -445,30 +445,69 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
     const int total = n_live * U;
     Real *obase = out + ((long long)s0 * d.T + tb) * d.M;
     const Real *wbase = w + (long long)tb * d.L * wpitch;  // wpitch: elements between leaf rows (M, or padded)
-    for (int u0 = lane; u0 < total; u0 += kWave * kRowUnroll) {
-      Real a[kRowUnroll];
-      Vec wv[kRowUnroll];
-      uint32_t off[kRowUnroll];
+    constexpr int kBurst = kWave * kRowUnroll;  // vectors a wavefront handles per iteration
+    if (total % kBurst == 0 && kBurst % U == 0) {
+      // Whole bursts, and a burst is a whole number of samples: which tree and output a lane serves in slot q of a
+      // burst is the same in every burst, so the divisions are done once per step and a burst only advances the
+      // sample (complete tiles of the benchmark shapes: 32 samples x 8 trees x 10 outputs = 4 bursts of 8 samples).
+      uint32_t park[kRowUnroll], wcol[kRowUnroll], off[kRowUnroll];
 #pragma unroll
       for (int q = 0; q < kRowUnroll; ++q) {
-        const int u = min(u0 + q * kWave, total - 1);
+        const int u = lane + q * kWave;
         const int jj = div_u.div(u);
         const int e = (u - jj * U) * GW;
         const int tt = div_m.div(e), m = e - tt * d.M;
-        const uint32_t key = p_key[jj * LDP + tt];
-        a[q] = p_abs[jj * LDP + tt];
-        wv[q] = *reinterpret_cast<const Vec *>(wbase + (uint32_t(tt) * uint32_t(d.L) + key) * uint32_t(wpitch) + m);
+        park[q] = uint32_t(jj * LDP + tt);
+        wcol[q] = uint32_t(tt) * uint32_t(d.L) * uint32_t(wpitch) + uint32_t(m);
         off[q] = uint32_t(jj) * TM + uint32_t(e);
       }
+      const uint32_t park_step = uint32_t(kBurst / U) * LDP, off_step = uint32_t(kBurst / U) * TM;
+      for (int burst = 0; burst < total; burst += kBurst) {
+        Real a[kRowUnroll];
+        Vec wv[kRowUnroll];
 #pragma unroll
-      for (int q = 0; q < kRowUnroll; ++q) {
-        if (u0 + q * kWave < total) {
+        for (int q = 0; q < kRowUnroll; ++q) {
+          const uint32_t key = p_key[park[q]];
+          a[q] = p_abs[park[q]];
+          wv[q] = *reinterpret_cast<const Vec *>(wbase + key * uint32_t(wpitch) + wcol[q]);
+        }
+#pragma unroll
+        for (int q = 0; q < kRowUnroll; ++q) {
           Vec o;
 #pragma unroll
           for (int i = 0; i < GW; ++i) o[i] = a[q] * wv[q][i];
-          // streaming store: the output is written once and not read here, so it should not displace the vertices
-          // and leaf weights that the gathers keep re-reading from L2 (measured: 1.45 -> 1.17 ms at the headline shape)
           __builtin_nontemporal_store(o, reinterpret_cast<Vec *>(obase + off[q]));
+          park[q] += park_step;
+          off[q] += off_step;
+        }
+      }
+    } else {
+      for (int u0 = lane; u0 < total; u0 += kWave * kRowUnroll) {
+        Real a[kRowUnroll];
+        Vec wv[kRowUnroll];
+        uint32_t off[kRowUnroll];
+#pragma unroll
+        for (int q = 0; q < kRowUnroll; ++q) {
+          const int u = min(u0 + q * kWave, total - 1);
+          const int jj = div_u.div(u);
+          const int e = (u - jj * U) * GW;
+          const int tt = div_m.div(e), m = e - tt * d.M;
+          const uint32_t key = p_key[jj * LDP + tt];
+          a[q] = p_abs[jj * LDP + tt];
+          wv[q] = *reinterpret_cast<const Vec *>(wbase + (uint32_t(tt) * uint32_t(d.L) + key) * uint32_t(wpitch) + m);
+          off[q] = uint32_t(jj) * TM + uint32_t(e);
+        }
+#pragma unroll
+        for (int q = 0; q < kRowUnroll; ++q) {
+          if (u0 + q * kWave < total) {
+            Vec o;
+#pragma unroll
+            for (int i = 0; i < GW; ++i) o[i] = a[q] * wv[q][i];
+            // streaming store: the output is written once and not read here, so it should not displace the vertices
+            // and leaf weights that the gathers keep re-reading from L2 (measured: 1.45 -> 1.17 ms at the headline
+            // shape)
+            __builtin_nontemporal_store(o, reinterpret_cast<Vec *>(obase + off[q]));
+          }
         }
       }
     }
