@@ -64,6 +64,8 @@ SIGNATURES = {
     "ht_conv_backward": (_I, [ctypes.POINTER(ConvShape), _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "ht_tree_mix_forward": (_I, [ctypes.c_int64] * 4 + [_P, _P, _P, _P, _P]),
     "ht_tree_mix_backward": (_I, [ctypes.c_int64] * 4 + [_P, _P, _P, _P, _P, ctypes.c_int, _P]),
+    "ht_tree_mix_forward_f64": (_I, [ctypes.c_int64] * 4 + [_P, _P, _P, _P, _P]),
+    "ht_tree_mix_backward_f64": (_I, [ctypes.c_int64] * 4 + [_P, _P, _P, _P, _P, _P]),
     "ht_contract": (_I, [ctypes.POINTER(TileShape), _P, _P, _P]),
     "ht_expand": (_I, [ctypes.POINTER(TileShape), _P, _P, _P]),
     "ht_projection_workspace": (_SZ, [ctypes.c_int64]),

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libhingetree_hip.so")
 
-SOURCES = ["capi.hip", "forest_forward.hip", "forest_backward.hip", "forest_maps.hip", "conv.hip", "projection.hip", "expand.hip"]
+SOURCES = ["capi.hip", "forest_forward.hip", "forest_backward.hip", "forest_maps.hip", "conv.hip", "projection.hip", "mix_f64.hip", "expand.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

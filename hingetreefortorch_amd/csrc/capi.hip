@@ -412,6 +412,20 @@ int ht_tree_mix_backward(int64_t B, int64_t T, int64_t O, int64_t R, const float
   return mix_backward(B, T, O, R, f, lin, g, h, dlin, deterministic != 0, static_cast<hipStream_t>(stream));
 }
 
+int ht_tree_mix_forward_f64(int64_t B, int64_t T, int64_t O, int64_t R, const double *f, const double *lin,
+                            const double *bias, double *out, void *stream) {
+  if (B < 0 || T < 0 || O < 0 || R < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if (B * O * R > 0 && (!out || (T > 0 && (!f || !lin)))) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return mix_forward_f64(B, T, O, R, f, lin, bias, out, static_cast<hipStream_t>(stream));
+}
+
+int ht_tree_mix_backward_f64(int64_t B, int64_t T, int64_t O, int64_t R, const double *f, const double *lin,
+                             const double *g, double *h, double *dlin, void *stream) {
+  if (B < 0 || T < 0 || O < 0 || R < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if (B * O * R > 0 && (!g || (h && !lin) || (dlin && !f))) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return mix_backward_f64(B, T, O, R, f, lin, g, h, dlin, static_cast<hipStream_t>(stream));
+}
+
 int ht_contract(const ht_tile_shape *s, const void *image, void *tiles, void *stream) {
   if (s && s->planes > 0 && (!image || !tiles)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
   return tile_contract(s, image, tiles, static_cast<hipStream_t>(stream));

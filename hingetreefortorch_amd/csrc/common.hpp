@@ -143,6 +143,12 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
 
 int conv_output_size(const ht_conv_shape &s, int64_t *out_size);
 
+// Linear mix over the tree axis behind a forest, float64 (mix_f64.hip; plain kernels, fixed summation order).
+int mix_forward_f64(long long B, long long T, long long O, long long R, const double *f, const double *lin,
+                    const double *bias, double *out, hipStream_t stream);
+int mix_backward_f64(long long B, long long T, long long O, long long R, const double *f, const double *lin,
+                     const double *g, double *h, double *dlin, hipStream_t stream);
+
 // Linear mix over the tree axis behind a forest (projection.hip), fp32.
 int mix_forward(long long B, long long T, long long O, long long R, const float *f, const float *lin,
                 const float *bias, float *out, hipStream_t stream);

@@ -111,8 +111,6 @@ def _fused_linear_checks(inData, inThresholds, inOrdinals, inWeights, inLinearWe
             inWeights.shape[0] != inLinearWeights.shape[1] or inLinearWeights.shape[0] != inLinearBias.shape[0]:
         _invalid("Error: inThresholds and inOrdinals must be the same shape. inWeights.shape[0] must be the same as "
                  "inThresholds.shape[0]. inLinearWeightrs.shape[0] must be the same as inLinearBias.shape[0].")
-    if inData.dtype != torch.float32:
-        _runtime("Error: the forest -> linear operators of this build support torch.float32 only.")
 
 
 def _mix_sizes(inData, inWeights, inLinearWeights):
@@ -135,8 +133,8 @@ def _fused_linear_forward(kind, inData, inThresholds, inOrdinals, inWeights, inL
     B, T, O, R, out_sizes = _mix_sizes(inData, inWeights, inLinearWeights)
     with torch.cuda.device(inData.device):
         out = torch.empty(out_sizes, dtype=inData.dtype, device=inData.device)
-        L.check(L.load().ht_tree_mix_forward(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(inLinearBias), _ptr(out),
-                                             _stream(inData.device)))
+        mix = L.load().ht_tree_mix_forward if inData.dtype == torch.float32 else L.load().ht_tree_mix_forward_f64
+        L.check(mix(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(inLinearBias), _ptr(out), _stream(inData.device)))
     return (out, f, records) if keep else out
 
 
@@ -164,9 +162,13 @@ def _fused_linear_backward(kind, mode, inData, bInDataGrad, inThresholds, bInThr
                         device=inData.device) if need_forest else None
         dlin = torch.empty_like(inLinearWeights) if bInLinearWeightsGrad else None
         if h is not None or dlin is not None:
-            L.check(lib.ht_tree_mix_backward(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(outDataGrad), _ptr(h),
-                                             _ptr(dlin), int(mode == L.HT_BACKWARD_DETERMINISTIC),
-                                             _stream(inData.device)))
+            if inData.dtype == torch.float32:
+                L.check(lib.ht_tree_mix_backward(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(outDataGrad), _ptr(h),
+                                                 _ptr(dlin), int(mode == L.HT_BACKWARD_DETERMINISTIC),
+                                                 _stream(inData.device)))
+            else:  # float64: plain kernels with a fixed summation order in either mode
+                L.check(lib.ht_tree_mix_backward_f64(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(outDataGrad),
+                                                     _ptr(h), _ptr(dlin), _stream(inData.device)))
         grads[4] = dlin
         if need_forest and state is not None and state[1] is not None:
             grads[0], grads[1], _, grads[3] = _backward_records(kind, mode, state[1], inData, bInDataGrad, inThresholds,

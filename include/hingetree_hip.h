@@ -176,6 +176,13 @@ int ht_tree_mix_forward(int64_t B, int64_t T, int64_t O, int64_t R, const float 
 int ht_tree_mix_backward(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin, const float *g,
                          float *h, float *dlin, int deterministic, void *stream);
 
+/* The same three products for float64 data (the reference instantiates its fused-linear operators for double as well,
+ * hingetree_fused_linear.cpp:798-806,845-853): plain kernels with a fixed summation order, always reproducible. */
+int ht_tree_mix_forward_f64(int64_t B, int64_t T, int64_t O, int64_t R, const double *f, const double *lin,
+                            const double *bias, double *out, void *stream);
+int ht_tree_mix_backward_f64(int64_t B, int64_t T, int64_t O, int64_t R, const double *f, const double *lin,
+                             const double *g, double *h, double *dlin, void *stream);
+
 /* ---- contract / expand -----------------------------------------------------------------------------------------------
  * Replace contract2d/3d and expand2d/3d of the reference (expand.cpp:37-227 on the CPU, expand_gpu.cu:110-172 on the
  * GPU; exported as `contract` / `expand`, hingetree.cpp:2029-2030). Tile j of a dimension covers image positions

@@ -25,7 +25,7 @@ from RandomHingeForest import RandomHingeFernFusedLinear, RandomHingeForestFused
 pytestmark = pytest.mark.gpu
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-MIX_FILES = sorted(glob.glob(os.path.join(GOLDEN, "mix_*f32*.npz")))
+MIX_FILES = sorted(glob.glob(os.path.join(GOLDEN, "mix_*.npz")))   # float32 and float64 fixtures
 TOL = 1e-5
 
 CASES = [
@@ -41,29 +41,30 @@ CASES = [
 ]
 
 
-def _inputs(case, fern, seed=0):
+def _inputs(case, fern, seed=0, dtype=torch.float32):
     B, F, Kd, T, D, Md, O = case
-    x, thr, ordn, w, _ = make_forest(B, F, Kd, T, D, Md, fern, torch.float32, seed=seed)
+    x, thr, ordn, w, _ = make_forest(B, F, Kd, T, D, Md, fern, dtype, seed=seed)
     g = torch.Generator().manual_seed(77 + seed)
-    lin = torch.randn([O, T], generator=g) / T ** 0.5
-    bias = torch.randn([O], generator=g)
-    gout = torch.randn([B, O] + list(Kd) + list(Md), generator=g)
+    lin = torch.randn([O, T], generator=g, dtype=dtype) / T ** 0.5
+    bias = torch.randn([O], generator=g, dtype=dtype)
+    gout = torch.randn([B, O] + list(Kd) + list(Md), generator=g, dtype=dtype)
     return x, thr, ordn, w, lin, bias, gout
 
 
 def _check(dev, fern, x, thr, ordn, w, lin, bias, gout, want=None):
     pre = "fern_" if fern else "tree_"
+    TOL = 1e-5 if x.dtype == torch.float32 else 1e-12   # float64: only the order of the sums differs from the oracle's
     if want is None:
         want = dict(out=ho.fused_linear_forward(x, thr, ordn, w, lin, bias, fern))
         want["dx"], want["dthr"], want["dw"], want["dlin"] = ho.fused_linear_backward(x, thr, ordn, w, lin, gout, fern=fern)
-        want["dbias"] = gout.double().sum(dim=[0] + list(range(2, gout.dim()))).float()
+        want["dbias"] = gout.double().sum(dim=[0] + list(range(2, gout.dim()))).to(x.dtype)
         x64 = [t.double() if t.is_floating_point() else t for t in (x, thr, ordn, w, lin, gout)]
         exact = dict(zip(("dx", "dthr", "dw", "dlin"), ho.fused_linear_backward(*x64, fern=fern)))
     else:
         exact = {}
     d = [t.to(dev) for t in (x, thr, ordn, w, lin, bias, gout)]
     out = getattr(ops, pre + "fused_linear_forward")(*d[:6])
-    assert out.shape == want["out"].shape and out.dtype == torch.float32
+    assert out.shape == want["out"].shape and out.dtype == x.dtype
     assert rel_err(out.cpu(), want["out"]) <= TOL
     for name in ("fused_linear_backward", "fused_linear_backward_deterministic"):
         dx, dthr, dord, dw, dlin, dbias = getattr(ops, pre + name)(d[0], True, d[1], True, d[2], False, d[3], True,
@@ -91,6 +92,28 @@ def _check(dev, fern, x, thr, ordn, w, lin, bias, gout, want=None):
 @pytest.mark.parametrize("case", CASES, ids=[f"c{i}" for i in range(len(CASES))])
 def test_against_oracle(dev, case, fern):
     _check(dev, fern, *_inputs(case, fern))
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("case", [CASES[1], CASES[4], CASES[6], CASES[7]], ids=["c1", "c4", "c6", "c7"])
+def test_against_oracle_float64(dev, case, fern):
+    """The float64 instantiation (plain kernels for the linear mix): oracle agreement to 1e-12, both backward modes and
+    the training path."""
+    _check(dev, fern, *_inputs(case, fern, seed=5, dtype=torch.float64))
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+def test_gradcheck_float64(dev, fern):
+    """Finite differences through the autograd function in float64 (the model is piecewise linear, so they are exact
+    away from the kinks; inputs whose margins come within 1e-3 of a kink are pushed off it)."""
+    x, thr, ordn, w, lin, bias, _ = (t.to(dev) for t in _inputs((5, 6, [2], 4, 3, [2], 3), fern, seed=9,
+                                                                dtype=torch.float64))
+    margins, _ = getattr(ops, ("fern_" if fern else "tree_") + "marginmap")(x, thr, ordn, w)
+    assert float(margins.abs().min()) > 1e-3, "test inputs sit on a kink; change the seed"
+    fn = HingeFernFusedLinear if fern else HingeTreeFusedLinear
+    leaves = [t.clone().requires_grad_(True) for t in (x, thr, w, lin, bias)]
+    assert torch.autograd.gradcheck(lambda a, b, c, d, e: fn.apply(a, b, ordn, c, d, e), leaves, eps=1e-6, atol=1e-7,
+                                    rtol=1e-6, nondet_tol=1e-12)
 
 
 @pytest.mark.parametrize("path", MIX_FILES, ids=[os.path.basename(p)[:-4] for p in MIX_FILES])
@@ -127,8 +150,8 @@ def test_rejects_bad_input(dev):
     with pytest.raises(ValueError):
         ops.tree_fused_linear_backward(x, True, thr, True, ordn, False, w, True, lin, True, bias, True,
                                        gout[:, :-1].contiguous())
-    with pytest.raises(RuntimeError):
-        ops.tree_fused_linear_forward(*(t.double() if t.is_floating_point() else t for t in (x, thr, ordn, w, lin, bias)))
+    with pytest.raises(ValueError):   # data types disagree
+        ops.tree_fused_linear_forward(x, thr, ordn, w, lin.double(), bias)
     with pytest.raises(RuntimeError):
         ops.tree_fused_linear_forward(x.cpu(), thr.cpu(), ordn.cpu(), w.cpu(), lin.cpu(), bias.cpu())
 
