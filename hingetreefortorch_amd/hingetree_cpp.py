@@ -69,10 +69,10 @@ def _require_gpu(t):
 
 # ---- ordinal range check ------------------------------------------------------------------------------------------
 # The reference reduces inOrdinals to its min and max and reads them back on every call (hingetree.cpp:91,
-# hingetree_gpu.cu:445). The same check runs here, but its verdict is remembered per tensor object and version
+# hingetree_gpu.cu:445). The same check runs here, but its result is remembered per tensor object and version
 # counter, so a module's fixed `ordinals` parameter costs one device->host read in its lifetime rather than one per
 # call. (Writes through `.data` do not advance the version counter; the kernels therefore also clamp every ordinal
-# into range, so a stale verdict can give wrong numbers but never an out-of-bounds access.)
+# into range, so a stale result can give wrong numbers but never an out-of-bounds access.)
 _range_ok = {}  # id(tensor) -> (weakref, version, bound) with the proven fact 0 <= ordinals < bound
 
 
