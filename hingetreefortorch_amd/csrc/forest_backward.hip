@@ -967,6 +967,19 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
   Acc top[kTop];
 #pragma unroll
   for (int k = 0; k < kTop; ++k) top[k] = Acc(0);
+  auto add = [&](uint32_t v, Real c) {
+    Acc val;
+    if constexpr (FIXED)
+      val = to_fixed(-double(c), scale);
+    else
+      val = -double(c);
+    if (v < uint32_t(kTop)) {
+#pragma unroll
+      for (int k = 0; k < kTop; ++k) top[k] += v == uint32_t(k) ? val : Acc(0);
+    } else {
+      atomicAdd(acc + v, val);
+    }
+  };
   for (long long s0 = s_begin + threadIdx.x; s0 < s_end; s0 += 256 * kBatch) {
     uint32_t v[kBatch];
     Real cv[kBatch];
@@ -980,17 +993,7 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
 #pragma unroll
     for (int i = 0; i < kBatch; ++i) {
       if (s0 + i * 256 >= s_end) break;
-      Acc val;
-      if constexpr (FIXED)
-        val = to_fixed(-double(cv[i]), scale);
-      else
-        val = -double(cv[i]);
-      if (v[i] < uint32_t(kTop)) {
-#pragma unroll
-        for (int k = 0; k < kTop; ++k) top[k] += v[i] == uint32_t(k) ? val : Acc(0);
-      } else {
-        atomicAdd(acc + v[i], val);
-      }
+      add(v[i], cv[i]);
     }
   }
   // the lanes' sums for the top vertices: reduced over the wavefront, then one atomic each
@@ -1043,7 +1046,51 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
   const long long s0 = (long long)blockIdx.x * BT;
   const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
   const long long s = s0 + j;
-  if (s < d.S) {
+  // Packed records of a sample count that is a multiple of four: a lane takes four consecutive samples of a tree with
+  // one 16-byte load of the record words and one of c, a quarter of the vector-memory instructions of the
+  // sample-per-lane loop below (which costs the CU ~16 cycles per instruction however few bytes it moves).
+  bool quads = false;
+  if constexpr (COMPACT && BT % 4 == 0) {
+    quads = rec.oshift != 0 && d.S % 4 == 0 && reinterpret_cast<uintptr_t>(rec.a) % 16 == 0 &&
+            reinterpret_cast<uintptr_t>(rec.c) % (4 * sizeof(Real)) == 0;
+  }
+  if constexpr (COMPACT && BT % 4 == 0) {
+    if (quads) {
+      typedef uint32_t Word4 __attribute__((ext_vector_type(4)));
+      typedef Real Real4 __attribute__((ext_vector_type(4)));
+      constexpr int LPT = BT / 4;    // lanes per tree
+      constexpr int TCQ = NT / LPT;  // trees in flight per pass of the workgroup
+      constexpr int kBatchQ = 4;
+      const int jq = 4 * (threadIdx.x % LPT), tq = threadIdx.x / LPT;
+      if (s0 + jq < d.S) {
+        for (int t0 = tq; t0 < d.T; t0 += TCQ * kBatchQ) {
+          Word4 av[kBatchQ];
+          Real4 cv[kBatchQ];
+#pragma unroll
+          for (int i = 0; i < kBatchQ; ++i) {
+            const int t = min(t0 + i * TCQ, d.T - 1);
+            const long long at = (long long)t * d.S + s0 + jq;
+            av[i] = *reinterpret_cast<const Word4 *>(rec.a + at);
+            cv[i] = __builtin_nontemporal_load(reinterpret_cast<const Real4 *>(rec.c + at));
+          }
+#pragma unroll
+          for (int i = 0; i < kBatchQ; ++i) {
+            if (t0 + i * TCQ >= d.T) break;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const uint32_t o = av[i][e] >> rec.oshift;
+              if (FIXED)
+                atomicAdd(reinterpret_cast<unsigned long long *>(acc) + o * LD + jq + e,
+                          to_fixed(double(cv[i][e]), scale));
+              else
+                lds_add(reinterpret_cast<Real *>(acc) + o * LD + jq + e, cv[i][e]);
+            }
+          }
+        }
+      }
+    }
+  }
+  if (!quads && s < d.S) {
     // the loads of several trees are issued together: the loop is otherwise bound by one memory round trip per tree
     constexpr int kBatch = 8;
     for (int t0 = tt; t0 < d.T; t0 += TC * kBatch) {
