@@ -749,6 +749,21 @@ __global__ __launch_bounds__(256) void pad_rows_kernel(const Real *__restrict__ 
   }
 }
 
+// The same copy for a power-of-two pitch and an even row length: one thread per pair of elements, index arithmetic by
+// shifts, one store per thread over a flat grid (the form in which plain stores run fastest).
+template <typename Real>
+__global__ __launch_bounds__(256) void pad_rows_pairs_kernel(const Real *__restrict__ w, Real *__restrict__ dst,
+                                                             long long pairs, int M, int log2_pairs_per_row) {
+  typedef Real Vec2 __attribute__((ext_vector_type(2)));
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= pairs) return;
+  const long long r = i >> log2_pairs_per_row;
+  const int m = int(i - (r << log2_pairs_per_row)) * 2;
+  Vec2 v = {Real(0), Real(0)};
+  if (m < M) v = *reinterpret_cast<const Vec2 *>(w + r * M + m);
+  *reinterpret_cast<Vec2 *>(dst + 2 * i) = v;
+}
+
 template <typename Real>
 int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
                    Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream, const ImageStore *image) {
@@ -764,9 +779,19 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
     if (wpitch != d.M) {
       Real *padded = reinterpret_cast<Real *>(static_cast<unsigned char *>(ws) + vertex_bytes<Real>(d));
       const long long rows = (long long)d.T * d.L;
-      long long blocks = (rows * wpitch + 255) / 256;
-      if (blocks > 16 * kNumCUs) blocks = 16 * kNumCUs;
-      hipLaunchKernelGGL(pad_rows_kernel<Real>, dim3((unsigned)blocks), dim3(256), 0, stream, w, padded, rows, d.M, wpitch);
+      const long long pairs = rows * wpitch / 2;
+      int log2_ppr = 0;
+      while ((2 << log2_ppr) < wpitch) ++log2_ppr;
+      if (d.M % 2 == 0 && (2 << log2_ppr) == wpitch && reinterpret_cast<uintptr_t>(w) % (2 * sizeof(Real)) == 0 &&
+          (pairs + 255) / 256 <= 0x7fffffffLL) {
+        hipLaunchKernelGGL(pad_rows_pairs_kernel<Real>, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream, w,
+                           padded, pairs, d.M, log2_ppr);
+      } else {
+        long long blocks = (rows * wpitch + 255) / 256;
+        if (blocks > 16 * kNumCUs) blocks = 16 * kNumCUs;
+        hipLaunchKernelGGL(pad_rows_kernel<Real>, dim3((unsigned)blocks), dim3(256), 0, stream, w, padded, rows, d.M,
+                           wpitch);
+      }
       HT_LAUNCH_CHECK("pad leaf rows");
       w = padded;
     }
