@@ -1873,8 +1873,22 @@ int clear_gradients(const ForestDims &d, Route route, Real *dx, Real *dthr, Real
   const bool empty = is_empty(d);
   const bool clear_dx = route != Route::kStaged || empty || pick_dx_tile(d.F, sizeof(Real)) == 0;
   if (dx && clear_dx && (rc = zero_fill(dx, size_t(d.S) * d.F * sizeof(Real), stream)) != HT_OK) return rc;
-  if (dthr && (rc = zero_fill(dthr, size_t(d.T) * d.V * sizeof(Real), stream)) != HT_OK) return rc;
-  if (dw && (rc = zero_fill(dw, size_t(d.T) * d.L * d.M * sizeof(Real), stream)) != HT_OK) return rc;
+  // The staged atomic route stores dW and dThr from its LDS tables (every cell, by the workgroup that owns the tree)
+  // unless the samples are split over several workgroups, whose shares then meet in atomics on the cleared buffers.
+  bool clear_dthr = true, clear_dw = true;
+  if (route == Route::kStaged && !empty) {
+    TreePlan plan;
+    long long dthr_part;
+    int dthr_gy;
+    plan_dthr(d, &dthr_part, &dthr_gy);
+    if (plan_trees(d, dw != nullptr, std::is_same<Real, float>::value && compact_ok(d) && d.K == 1, &plan) &&
+        plan.parts == 1) {
+      clear_dw = false;
+      clear_dthr = dthr_gy > 1;
+    }
+  }
+  if (dthr && clear_dthr && (rc = zero_fill(dthr, size_t(d.T) * d.V * sizeof(Real), stream)) != HT_OK) return rc;
+  if (dw && clear_dw && (rc = zero_fill(dw, size_t(d.T) * d.L * d.M * sizeof(Real), stream)) != HT_OK) return rc;
   *done = empty || (!dx && !dthr && !dw);
   return HT_OK;
 }

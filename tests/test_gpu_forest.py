@@ -258,6 +258,38 @@ def test_records_path(dev, case, dtype, fern):
     assert only_x[3] is None and rel_err(only_x[0].cpu(), rdx) <= tol + slack[0]
 
 
+@pytest.mark.parametrize("mode", ["atomic", "deterministic"])
+@pytest.mark.parametrize("case", [CASES[3], CASES[8], CASES[10], CASES[11], CASES[14], CASES[17]],
+                         ids=["c3", "c8", "c10", "c11", "c14", "c17"])
+def test_backward_owns_its_output_buffers(dev, case, mode):
+    """Through the C ABI with dX, dThr and dW handed over full of NaN: the library clears or overwrites every cell
+    itself on every route (single launch, staged with and without split samples, wide rows), whatever was there."""
+    import ctypes
+    from hingetreefortorch_amd import _lib as L
+    B, F, Kd, T, D, Md = case
+    x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, False, torch.float32)
+    _, slack, exact = _reference_gradients(x, thr, ordn, w, gout, False)
+    gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
+    shape = L.ForestShape()
+    shape.kind, shape.dtype = L.HT_TREE, L.HT_F32
+    shape.B, shape.F, shape.T, shape.depth = B, F, T, D
+    shape.K = int(torch.tensor(Kd).prod()) if Kd else 1
+    shape.M = int(torch.tensor(Md).prod()) if Md else 1
+    m = L.HT_BACKWARD_DETERMINISTIC if mode == "deterministic" else L.HT_BACKWARD_ATOMIC
+    lib = L.load()
+    nbytes = lib.ht_forest_backward_workspace(ctypes.byref(shape), m, 1, 1, 1)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
+    dx, dthr, dw = (torch.full_like(t, float("nan")) for t in (gx, gthr, gw))
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    L.check(lib.ht_forest_backward(ctypes.byref(shape), P(gx), P(gthr), P(gord), P(gw), P(gg), P(dx), P(dthr), P(dw), m,
+                                   P(ws), nbytes, stream))
+    torch.cuda.synchronize()
+    for got, want in zip((dx, dthr, dw), exact):
+        assert not got.isnan().any()
+        assert rel_err(got.cpu().double(), want.double()) <= 1e-5
+
+
 EMPTY = {"no samples": (0, 5, [], 3, 2, []), "no inner positions": (4, 5, [0], 3, 2, []),
          "no outputs per leaf": (4, 5, [], 3, 2, [0]), "no trees": (4, 5, [], 0, 2, [2]),
          "no samples, staged sizes": (0, 64, [], 300, 6, [10])}
