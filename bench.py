@@ -43,7 +43,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the forward kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (KiB per dispatch,
 # scaled by what the same counters read for a plain 1 GiB copy: x2.0 for FETCH_SIZE, x1.0 for WRITE_SIZE); the
 # summaries are under profiles/.
-MEASURED_TRAFFIC = {("c3", "train"): 4388945470}   # 1151 MB fetched + 3238 MB written (2621 MB out, 524 MB walk records)
+MEASURED_TRAFFIC = {("c3", "train"): 4384142362}   # 1146 MB fetched + 3238 MB written (2621 MB out, 524 MB walk records)
 
 WORKLOADS = {
     # name: (B, F, T, depth, M, kind, x distribution, description)
