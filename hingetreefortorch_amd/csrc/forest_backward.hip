@@ -841,6 +841,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
     float mg;
     Float4U gv;
   };
+  long long img_sb = -1, img_at = -1, img_base = 0;  // IMAGE: the sample block the cached offsets belong to
   auto issue = [&](Step &st, long long sb, int tl) {
     const long long s_raw = sb + pr;
     st.on = s_raw < s_end;
@@ -849,13 +850,18 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
     st.a = rec.a[st.at];
     st.mg = rec.margin[st.at];
     if constexpr (IMAGE) {
-      const long long b = s / d.K;
-      const long long at = img.offset(int(s - b * d.K), e0);
+      // the trees of a group run fastest, so the image offset of this lane's run changes once per nt steps
+      if (sb != img_sb) {
+        img_sb = sb;
+        const long long b = s / d.K;
+        img_at = img.offset(int(s - b * d.K), e0);
+        img_base = b * d.T * img.plane + img_at;
+      }
       const Float4U zero = {0.f, 0.f, 0.f, 0.f};
       st.gv = zero;
-      if (at >= 0)
+      if (img_at >= 0)
         st.gv = __builtin_nontemporal_load(
-            reinterpret_cast<const Float4U *>(gout + (b * d.T + (t0 + tl)) * img.plane + at));
+            reinterpret_cast<const Float4U *>(gout + img_base + (long long)(t0 + tl) * img.plane));
     } else {
       const long long row = d.K == 1 ? (s * d.T + (t0 + tl)) * (long long)M : out_offset(d, s, t0 + tl, 0);
       st.gv = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(gout + row + e0));
@@ -874,13 +880,16 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
     }
     if (dw && st.on) {
       const float a = ht_abs(st.mg);
+      // In LDS a row is kept transposed, element 4 k + i of the row at slot i * P + k: the P lanes of a pair then hit
+      // P consecutive cells in each of the four atomic instructions instead of every fourth cell (half the banks).
+      const uint32_t slot = cell - uint32_t(e0) + uint32_t(e0 >> 2);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float term = a * st.gv[i];
         if (FIXED)
-          atomicAdd(reinterpret_cast<unsigned long long *>(acc) + cell + i, to_fixed(double(term), scale));
+          atomicAdd(reinterpret_cast<unsigned long long *>(acc) + slot + i * P, to_fixed(double(term), scale));
         else
-          atomicAdd(reinterpret_cast<double *>(acc) + cell + i, double(term));
+          atomicAdd(reinterpret_cast<double *>(acc) + slot + i * P, double(term));
       }
     }
   };
@@ -920,21 +929,23 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
     __syncthreads();
     float *dst = dw + (long long)t0 * LM;
     const uint32_t n = uint32_t(nt) * LM;
+    // element i of the group's rows sits at its row's transposed slot
+    auto at = [&](uint32_t i) { return (i & ~(M - 1u)) + (i & 3u) * uint32_t(P) + ((i & (M - 1u)) >> 2); };
     if (FIXED) {
       const unsigned long long *q = reinterpret_cast<const unsigned long long *>(acc);
       if (dw_atomic) {
         for (uint32_t i = threadIdx.x; i < n; i += kForestThreads)
-          if (q[i] != 0ull) atomicAdd(dw_fixed + (long long)t0 * LM + i, q[i]);
+          if (q[at(i)] != 0ull) atomicAdd(dw_fixed + (long long)t0 * LM + i, q[at(i)]);
       } else {
-        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = from_fixed<float>(q[i], inv_scale);
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = from_fixed<float>(q[at(i)], inv_scale);
       }
     } else {
       const double *q = reinterpret_cast<const double *>(acc);
       if (dw_atomic) {
         for (uint32_t i = threadIdx.x; i < n; i += kForestThreads)
-          if (q[i] != 0.0) atomicAdd(dst + i, float(q[i]));
+          if (q[at(i)] != 0.0) atomicAdd(dst + i, float(q[at(i)]));
       } else {
-        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = float(q[i]);
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = float(q[at(i)]);
       }
     }
   }
