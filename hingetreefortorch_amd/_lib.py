@@ -46,6 +46,7 @@ SIGNATURES = {
     "ht_ordinal_range": (_I, [_P, ctypes.c_int64, _P, _P]),
     "ht_forest_forward_workspace": (_SZ, [ctypes.POINTER(ForestShape)]),
     "ht_forest_forward": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "ht_forest_forward_static": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P]),
     "ht_forest_forward_image": (_I, [ctypes.POINTER(ForestShape), ctypes.POINTER(TileShape), _P, _P, _P, _P, _P, _P, _SZ,
                                      _P]),
     "ht_forest_backward_workspace": (_SZ, [ctypes.POINTER(ForestShape), _I, _I, _I, _I]),

@@ -1,8 +1,15 @@
 // extern "C" surface of libhingetree_hip.so (declared in include/hingetree_hip.h) and the host-only pieces.
 #include <cmath>
 #include <limits>
+#include <mutex>
 
 #include "common.hpp"
+
+// Workspace of ht_forest_forward_static (the forward pass for callers that cannot allocate): one array per GPU, part
+// of the library's code object, held by every GPU the library runs on until the process ends. In host code the array's
+// name is only a handle for hipGetSymbolAddress; the device address that call yields (one per device) is what the
+// kernels and the packing pre-passes receive.
+static __device__ __align__(256) unsigned char scratch[HT_STATIC_SCRATCH_BYTES];
 
 namespace ht {
 
@@ -135,6 +142,27 @@ static bool tree_repair(Real *thr, const int64_t *ord, int64_t V) {
   return changed;
 }
 
+// ---- the static workspace's device address, per device -------------------------------------------------------------
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up once per device, with that device current).
+static int static_scratch(void **ptr) {
+  int dev = -1;
+  HT_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(HT_ERR_RUNTIME, "Error: device index beyond the static workspace table.");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    HT_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(HT_ERR_HIP, "hipGetSymbolAddress returned a null address for the static workspace.");
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return HT_OK;
+}
+
 }  // namespace ht
 
 using namespace ht;
@@ -169,6 +197,30 @@ int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, 
                                  nullptr, workspace, workspace_bytes, st);
   return forest_forward<double>(d, fern, (const double *)x, (const double *)thr, ord, (const double *)w, (double *)out,
                                 nullptr, workspace, workspace_bytes, st);
+}
+
+int ht_forest_forward_static(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord,
+                             const void *w, void *out, void *stream) {
+  ForestDims d;
+  int rc = make_dims(s, &d);
+  if (rc != HT_OK) return rc;
+  const size_t need = ht_forest_forward_workspace(s);
+  if (need > size_t(HT_STATIC_SCRATCH_BYTES))
+    return fail(HT_ERR_INVALID_ARGUMENT,
+                "Error: this forest needs " + std::to_string(need) + " bytes of workspace, more than the " +
+                    std::to_string(size_t(HT_STATIC_SCRATCH_BYTES)) +
+                    " bytes ht_forest_forward_static holds; call ht_forest_forward with a workspace of your own.");
+  void *ws = nullptr;
+  if ((rc = static_scratch(&ws)) != HT_OK) return rc;  // also for an empty shape: a caller's set-up call
+  if (is_empty(d)) return HT_OK;
+  if (!x || !thr || !ord || !w || !out) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool fern = s->kind == HT_FERN;
+  if (s->dtype == HT_F32)
+    return forest_forward<float>(d, fern, (const float *)x, (const float *)thr, ord, (const float *)w, (float *)out,
+                                 nullptr, ws, size_t(HT_STATIC_SCRATCH_BYTES), st);
+  return forest_forward<double>(d, fern, (const double *)x, (const double *)thr, ord, (const double *)w, (double *)out,
+                                nullptr, ws, size_t(HT_STATIC_SCRATCH_BYTES), st);
 }
 
 int ht_forest_forward_image(const ht_forest_shape *s, const ht_tile_shape *g, const void *x, const void *thr,

@@ -72,6 +72,20 @@ size_t ht_forest_forward_workspace(const ht_forest_shape *s);
 int ht_forest_forward(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, const void *w,
                       void *out, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ht_forest_forward for callers that cannot allocate device memory -- code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc. No counterpart in the reference. Same result as ht_forest_forward, bit for
+ * bit; the workspace (packed vertices, leaf rows at a line-friendly pitch) is an array of HT_STATIC_SCRATCH_BYTES bytes
+ * inside the library's code object, one copy per GPU, held until the process ends. The call allocates and frees
+ * nothing. A forest whose ht_forest_forward_workspace exceeds HT_STATIC_SCRATCH_BYTES is refused with
+ * HT_ERR_INVALID_ARGUMENT (the headline forest -- 1000 trees of depth 10 with 10 outputs per leaf, 71 MB -- fits).
+ * The first call on a device looks up that device's copy of the array; a call with an empty shape (B = 0) does only
+ * that and launches nothing, so a caller can do it before a capture starts. All calls on one GPU share its array:
+ * the kernels of a call rewrite what they read from it, so calls in stream order are independent of each other, and
+ * calls that overlap on one GPU (different streams, different threads) race. */
+#define HT_STATIC_SCRATCH_BYTES (80u << 20)
+int ht_forest_forward_static(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord,
+                             const void *w, void *out, void *stream);
+
 /* ht_forest_forward of a forest with inner data positions x [B, F, *tiles] and tile-shaped outputs per leaf
  * w [T, L, *window], whose result is stored directly as the image [B, T, *size] that ht_expand makes of
  * [B, T, *tiles, *window] (g: planes = B * T, elem_size = that of the data type; image positions no tile covers are 0).
