@@ -511,6 +511,15 @@ int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, cons
   return projection_backward(B, K, N, x, lin, zhat, rstd, g, dlin, dx, workspace, static_cast<hipStream_t>(stream));
 }
 
+int ht_gemm_tile_map(int32_t tiles_i, int32_t tiles_j, int32_t *tile_i, int32_t *tile_j, int64_t capacity) {
+  if (tiles_i < 1 || tiles_j < 1) return fail(HT_ERR_INVALID_ARGUMENT, "Error: a tile grid needs at least one tile.");
+  const long long slots = (long long)((tiles_i + kNumXCDs - 1) / kNumXCDs) * tiles_j * kNumXCDs;
+  if (!tile_i || !tile_j || capacity < slots)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: the tile map needs room for " + std::to_string(slots) + " launch slots.");
+  gemm_tile_map(tiles_i, tiles_j, tile_i, tile_j);
+  return HT_OK;
+}
+
 int ht_check_thresholds(const void *thr, const int64_t *ord, int64_t T, int64_t depth, int32_t dtype, int32_t kind,
                         uint8_t *flags) {
   int64_t V;

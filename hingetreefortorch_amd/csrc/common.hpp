@@ -165,6 +165,9 @@ int projection_forward(long long B, long long K, long long N, const float *x, co
                        float *zhat, float *mean, float *rstd, float *var, void *ws, hipStream_t stream);
 int projection_backward(long long B, long long K, long long N, const float *x, const float *lin, const float *zhat,
                         const float *rstd, float *g, float *dlin, float *dx, void *ws, hipStream_t stream);
+// Host-side view of the matrix-product kernel's workgroup -> result-tile map for tiles_i x tiles_j tiles: writes the
+// tile of every launch slot (-1, -1 for a slot without a tile) and returns the number of slots.
+int gemm_tile_map(int tiles_i, int tiles_j, int *tile_i, int *tile_j);
 int ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, hipStream_t stream);
 
 // Fills `bytes` bytes with zero through a kernel (safe to record into a HIP graph, unlike a memset node).

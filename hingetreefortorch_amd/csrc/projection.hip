@@ -98,6 +98,31 @@ __device__ __forceinline__ void stash_tile(float *tile, const Fetch &f) {
   }
 }
 
+// Workgroup -> result tile. Workgroups are dealt to the 8 XCDs (each with its own L2) round robin by index, so
+// index % 8 names the L2 a workgroup will use. Every XCD takes a contiguous band of tile rows and walks it in panels
+// of 8 tile columns, row by row inside a panel: the ~100 workgroups an XCD runs at a time then cover about 12 x 8
+// tiles and share their 12 + 8 operand tiles through that L2, instead of each fetching its own pair.
+// Returns false for a launch slot that has no tile (bands are padded to the same number of slots).
+__host__ __device__ inline bool gemm_tile_of(int block, int tiles_i, int tiles_j, int rows_per_xcd, int *tile_i,
+                                             int *tile_j) {
+  const int xcd = block % kNumXCDs, slot = block / kNumXCDs;
+  const int row0 = xcd * rows_per_xcd;
+  const int rows = rows_per_xcd < tiles_i - row0 ? rows_per_xcd : tiles_i - row0;
+  if (rows <= 0 || slot >= rows * tiles_j) return false;
+  constexpr int kPanel = 8;
+  const int full = tiles_j / kPanel;  // panels of the full width
+  int panel = slot / (rows * kPanel), rem = slot - panel * (rows * kPanel), width = kPanel;
+  if (panel >= full) {
+    panel = full;
+    rem = slot - full * (rows * kPanel);
+    width = tiles_j - full * kPanel;
+  }
+  const int r = rem / width;
+  *tile_i = row0 + r;
+  *tile_j = panel * kPanel + (rem - r * width);
+  return true;
+}
+
 // C[i, j] = sum_r A(i, r) * B(j, r) (+ bias_i[i] + bias_j[j]), i < n_i, j < n_j, r < n_r; C row-major with leading
 // dimension ldc. A launch covers `batches` such problems whose operands lie stride_a / stride_b / stride_c elements
 // apart: either one result per batch (blockIdx.z), or -- SUM_BATCHES -- one result summed over all of them (the
@@ -121,28 +146,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
   __shared__ float As[2][kRed * kPitch];
   __shared__ float Bs[2][kRed * kPitch];
   const int n_i = g.n_i, n_j = g.n_j, n_r = g.n_r;
-  // Workgroup -> result tile. Workgroups are dealt to the 8 XCDs (each with its own L2) round robin by index, so
-  // index % 8 names the L2 a workgroup will use. Every XCD takes a contiguous band of tile rows and walks it in panels
-  // of 8 tile columns, row by row inside a panel: the ~100 workgroups an XCD runs at a time then cover about 12 x 8
-  // tiles and share their 12 + 8 operand tiles through that L2, instead of each fetching its own pair.
   int tile_i, tile_j;
-  {
-    const int xcd = blockIdx.x % kNumXCDs, slot = blockIdx.x / kNumXCDs;
-    const int row0 = xcd * g.rows_per_xcd;
-    const int rows = min(g.rows_per_xcd, g.tiles_i - row0);
-    if (rows <= 0 || slot >= rows * g.tiles_j) return;
-    constexpr int kPanel = 8;
-    const int full = g.tiles_j / kPanel;              // panels of the full width
-    int panel = slot / (rows * kPanel), rem = slot - panel * (rows * kPanel), width = kPanel;
-    if (panel >= full) {
-      panel = full;
-      rem = slot - full * (rows * kPanel);
-      width = g.tiles_j - full * kPanel;
-    }
-    const int r = rem / width;
-    tile_i = row0 + r;
-    tile_j = panel * kPanel + (rem - r * width);
-  }
+  if (!gemm_tile_of(int(blockIdx.x), g.tiles_i, g.tiles_j, g.rows_per_xcd, &tile_i, &tile_j)) return;
   const int i0 = tile_i * kTile, j0 = tile_j * kTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wavefront's 64 x 64 corner
@@ -387,6 +392,8 @@ __global__ __launch_bounds__(256) void bn_backward_apply_kernel(float *g, const 
   }
 }
 
+constexpr long long kMaxGridZ = 65535;  // limit of gridDim.z
+
 bool aligned16(const void *p, long long ld, long long stride) {
   return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0 && stride % 4 == 0;
 }
@@ -397,10 +404,21 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
                         long long n_r, long long batches, double *stats, const float *bias_i, const float *bias_j,
                         hipStream_t stream, bool allow_split = false) {
   if (n_i <= 0 || n_j <= 0 || batches <= 0) return HT_OK;
+  if (!SUM_BATCHES && batches > kMaxGridZ) {
+    // one result per batch rides on blockIdx.z: longer batch lists go out in several launches
+    for (long long b0 = 0; b0 < batches; b0 += kMaxGridZ) {
+      const long long nb = batches - b0 < kMaxGridZ ? batches - b0 : kMaxGridZ;
+      int rc = launch_gemm_batched<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES>(
+          A + b0 * stride_a, lda, stride_a, B + b0 * stride_b, ldb, stride_b, C + b0 * stride_c, ldc, stride_c, n_i, n_j,
+          n_r, nb, stats, bias_i, bias_j, stream, allow_split);
+      if (rc != HT_OK) return rc;
+    }
+    return HT_OK;
+  }
   const long long gi = (n_i + kTile - 1) / kTile, gj = (n_j + kTile - 1) / kTile;
   const long long per_batch = (n_r + kRed - 1) / kRed;
   if (gi > 0x7fffffffLL || gj > 0x7fffffffLL || n_r > 0x7fffffffLL || n_i > 0x7fffffffLL || n_j > 0x7fffffffLL ||
-      batches > 0x7fffffffLL || (!SUM_BATCHES && batches > 65535) || per_batch * batches > 0x7fffffffLL)
+      batches > 0x7fffffffLL || per_batch * batches > 0x7fffffffLL)
     return fail(HT_ERR_RUNTIME, "Error: matrix product too large for this build.");
   GemmArgs g;
   g.A = A, g.B = B, g.C = C;
@@ -444,6 +462,14 @@ int launch_gemm(const float *A, long long lda, const float *B, long long ldb, fl
 long long rows_grid(long long B) { return B < 64 ? (B < 1 ? 1 : B) : 64; }
 
 }  // namespace
+
+int gemm_tile_map(int tiles_i, int tiles_j, int *tile_i, int *tile_j) {
+  const int rows_per_xcd = (tiles_i + kNumXCDs - 1) / kNumXCDs;
+  const long long slots = (long long)rows_per_xcd * tiles_j * kNumXCDs;
+  for (long long b = 0; b < slots; ++b)
+    if (!gemm_tile_of(int(b), tiles_i, tiles_j, rows_per_xcd, &tile_i[b], &tile_j[b])) tile_i[b] = tile_j[b] = -1;
+  return int(slots);
+}
 
 size_t projection_workspace(long long N) { return align_up(size_t(2) * size_t(N) * sizeof(double), 256); }
 

@@ -71,15 +71,24 @@ def _require_gpu(t):
 # The reference reduces inOrdinals to its min and max and reads them back on every call (hingetree.cpp:91,
 # hingetree_gpu.cu:445). The same check runs here, but its result is remembered per tensor object and version
 # counter, so a module's fixed `ordinals` parameter costs one device->host read in its lifetime rather than one per
-# call. (Writes through `.data` do not advance the version counter; the kernels therefore also clamp every ordinal
-# into range, so a stale result can give wrong numbers but never an out-of-bounds access.)
-_range_ok = {}  # id(tensor) -> (weakref, version, bound) with the proven fact 0 <= ordinals < bound
+# call. The remembered result is tied to the tensor's version counter, storage address and size, so in-place
+# operations on the tensor and `param.data = other` both force a new check. In-place writes THROUGH `.data`
+# (`param.data.copy_(...)`) advance no counter the tensor can see: call `forget_ordinal_checks()` after them. The
+# kernels also clamp every ordinal into range, so a stale result can give wrong numbers but never an out-of-bounds
+# access.
+_range_ok = {}  # id(tensor) -> (weakref, version, data_ptr, numel, bound) with the proven fact 0 <= ordinals < bound
+
+
+def forget_ordinal_checks():
+    """Drop every remembered ordinal range check (for callers that overwrite ordinals through `.data`)."""
+    _range_ok.clear()
 
 
 def _validate_ordinals(ordinals, limit):
     key = id(ordinals)
     hit = _range_ok.get(key)
-    if hit is not None and hit[0]() is ordinals and hit[1] == ordinals._version and hit[2] <= limit:
+    if hit is not None and hit[0]() is ordinals and hit[1] == ordinals._version and hit[2] == ordinals.data_ptr() and \
+            hit[3] == ordinals.numel() and hit[4] <= limit:
         return
     bound = 0
     if ordinals.numel() > 0:
@@ -94,7 +103,7 @@ def _validate_ordinals(ordinals, limit):
         ref = weakref.ref(ordinals, lambda _r, k=key: _range_ok.pop(k, None))
     except TypeError:
         return
-    _range_ok[key] = (ref, ordinals._version, bound)
+    _range_ok[key] = (ref, ordinals._version, ordinals.data_ptr(), ordinals.numel(), bound)
 
 
 # ---- forest -> linear ("fused linear") ------------------------------------------------------------------------------
@@ -593,13 +602,18 @@ def _thresholds(kind, fix, inThresholds, inOrdinals, inWeights):
     return [bool(flags[i]) for i in range(T)]
 
 
+# the sweep of the reference's speed test (hingetree.cpp:1361-1438): batches per cell, tree counts 1, 2, .. 2^(steps-1),
+# depths 1 .. max depth
+SPEEDTEST_BATCHES, SPEEDTEST_TREE_STEPS, SPEEDTEST_MAX_DEPTH = 100, 10, 12
+
+
 def _speedtest(kind, inData, bDeterministic):
     """hingetree.cpp:1361-1438: T in {1,2,..,512} x depth in 1..12, 100 forwards then 100 backwards each, wall clock.
     Unlike the reference this synchronises the device around each timed loop, so it reports execution time."""
     if inData.dim() < 2:
         _invalid("Error: inData tensor expected to have at least 2 dimensions (i.e. [batch_size, num_channels, ...]).")
     name = "hingefern" if kind == L.HT_FERN else "hingetree"
-    num_batches, tree_steps, max_depth = 100, 10, 12
+    num_batches, tree_steps, max_depth = SPEEDTEST_BATCHES, SPEEDTEST_TREE_STEPS, SPEEDTEST_MAX_DEPTH
     timings = torch.zeros([4, tree_steps * max_depth], dtype=torch.float32)
     fwd = fern_forward if kind == L.HT_FERN else tree_forward
     if bDeterministic:

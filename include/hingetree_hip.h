@@ -174,6 +174,13 @@ int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, cons
                            const float *rstd, float *g, float *dlin, float *dx, void *workspace,
                            size_t workspace_bytes, void *stream);
 
+/* Diagnostic, host only, no counterpart in the reference: the matrix-product kernel's launch-slot -> result-tile map
+ * for a grid of tiles_i x tiles_j result tiles (slots are dealt to the 8 L2 domains round robin; each domain walks a
+ * band of tile rows in panels of 8 tile columns). tile_i / tile_j receive one entry per launch slot, (-1, -1) for a
+ * slot that has no tile; ((tiles_i + 7) / 8) * tiles_j * 8 slots exist and `capacity` entries must be available.
+ * Exists so that a host-side test can check that every tile is computed exactly once. */
+int ht_gemm_tile_map(int32_t tiles_i, int32_t tiles_j, int32_t *tile_i, int32_t *tile_j, int64_t capacity);
+
 /* ---- linear mix over the tree axis behind a forest (fp32) ------------------------------------------------------------
  * The dense half of the reference's fused-linear operators tree_fused_linear_forward / _backward and fern_*
  * (hingetree_fused_linear.cpp:75-412; GPU: hingetree_fused_linear_gpu.cu, which accumulates the forward with global

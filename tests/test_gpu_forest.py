@@ -219,6 +219,21 @@ def test_errors(dev):
     bad[0, 0] = -1
     with pytest.raises(RuntimeError, match="ordinal"):
         ops.tree_forward(x, thr, bad, w)
+    # the remembered verdict of the range check does not survive a new storage behind the same tensor object
+    par = torch.nn.Parameter(ordn.clone(), requires_grad=False)
+    ops.tree_forward(x, thr, par, w)
+    worse = ordn.clone()
+    worse[1, 1] = 7
+    par.data = worse
+    with pytest.raises(RuntimeError, match="ordinal"):
+        ops.tree_forward(x, thr, par, w)
+    # ... and a write through .data is caught once the caller says so
+    par.data = ordn.clone()
+    ops.tree_forward(x, thr, par, w)
+    par.data[2, 0] = -3
+    ops.forget_ordinal_checks()
+    with pytest.raises(RuntimeError, match="ordinal"):
+        ops.tree_forward(x, thr, par, w)
     with pytest.raises(RuntimeError, match="never has a gradient"):
         ops.tree_backward(x, True, thr, True, ordn, True, w, True, gout)
     with pytest.raises(ValueError, match="outDataGrad.shape"):
@@ -368,3 +383,51 @@ def test_special_values(dev, special, fern):
     dx, dthr, _, dw = getattr(ops, pre + "backward_records")(records, False, d[0], True, d[1], True, d[2], False, d[3],
                                                              True, d[4])
     assert rel_err(dx.cpu(), rdx) <= 1e-5 and rel_err(dthr.cpu(), rdthr) <= 1e-5 and rel_err(dw.cpu(), rdw) <= 1e-5
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+def test_reference_configuration_elementwise(dev, fern):
+    """The reference's CPU-runnable configuration (100 x 1000 inputs, 100 trees of depth 7, one output per leaf): every
+    gradient entry above 1e-2 of its tensor's largest is within 1e-5 of the float64 evaluation RELATIVE TO THAT ENTRY,
+    both backward modes and the training path; entries below that are held to the norm-wise bar. (The sums are short
+    here -- at most 100 terms -- which is what makes an element-wise bar possible at all; an entry 100 times below the
+    largest can be the sum of terms 100 times its size, each carrying a float32 rounding of 6e-8 from the product that
+    formed it, so 1e-5 of the entry is the most that float32 operands promise at that level and below it nothing is.)"""
+    B, F, Kd, T, D, Md = CASES[2]
+    x, thr, ordn, w, gout = make_forest(B, F, Kd, T, D, Md, fern, torch.float32)
+    exact = ho.backward(x.double(), thr.double(), ordn, w.double(), gout.double(), fern=fern)
+    gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
+    pre = "fern_" if fern else "tree_"
+    results = {"atomic": getattr(ops, pre + "backward")(gx, True, gthr, True, gord, False, gw, True, gg),
+               "deterministic": getattr(ops, pre + "backward_deterministic")(gx, True, gthr, True, gord, False, gw, True, gg)}
+    _, rec = getattr(ops, pre + "forward_records")(gx, gthr, gord, gw)
+    if rec is not None:
+        results["records"] = getattr(ops, pre + "backward_records")(rec, False, gx, True, gthr, True, gord, False, gw, True, gg)
+    for name, d in results.items():
+        for got, want in zip((d[0], d[1], d[3]), exact):
+            got = got.cpu().double()
+            big = want.abs() > 1e-2 * want.abs().max()
+            assert big.any()
+            rel = ((got - want).abs()[big] / want.abs()[big]).max().item()
+            assert rel <= 1e-5, (name, rel)
+            assert rel_err(got, want) <= 1e-5
+
+
+def test_speedtest_cell(dev, monkeypatch, capsys):
+    """tree_speedtest / fern_speedtest (hingetree.cpp:1361-1438) on a 2 x 2 corner of their sweep: the timings tensor
+    has the reference's layout (rows: trees, depth, forward ms, backward ms; one column per cell) and the printed lines
+    its wording."""
+    monkeypatch.setattr(ops, "SPEEDTEST_BATCHES", 3)
+    monkeypatch.setattr(ops, "SPEEDTEST_TREE_STEPS", 2)
+    monkeypatch.setattr(ops, "SPEEDTEST_MAX_DEPTH", 2)
+    x = torch.randn([64, 9], device=dev)
+    for fn, name, det in ((ops.tree_speedtest, "hingetree", False), (ops.fern_speedtest, "hingefern", True)):
+        timings = fn(x, det)
+        assert timings.shape == (4, 4) and timings.dtype == torch.float32
+        assert timings[0].tolist() == [1, 1, 2, 2] and timings[1].tolist() == [1, 2, 1, 2]
+        assert (timings[2:] > 0).all()
+        text = capsys.readouterr().out
+        assert f"{name}_forward: numBatches = 3, numTrees = 2, depth = 2:" in text
+        assert (f"{name}_backward_deterministic:" if det else f"{name}_backward:") in text
+    with pytest.raises(ValueError):
+        ops.tree_speedtest(x[0], False)

@@ -91,3 +91,107 @@ def test_offsets_beyond_32_bits(dev):
     want = torch.zeros([2 ** D, M], dtype=torch.float64, device=dev)
     want.index_add_(0, leaf[:, T - 1], margins[:, T - 1].abs().double()[:, None] * gout[:, T - 1, :].double())
     assert rel_err(dw[T - 1].double().cpu(), want.cpu()) <= 1e-5
+
+
+def test_projection_full_size(dev):
+    """The dense front of the README model at its benchmark size (16384 x 784 inputs -> 12700 private vertex features =
+    128 x 100 result tiles of the forward product, 100 x 7 of the dLin product): the XCD bands hold several tile rows
+    and the panels reach the ragged edge, which no small case does. Nothing in the reference pins a matrix product's
+    rounding (parity unpinned beyond fp32 tolerance), so the checks are what the mathematics fixes:
+      zhat      every column has mean 0 and variance var / (var + eps) over the batch;
+      z         slabs of 64 rows x 256 columns (first, middle, last tiles) of zhat / rstd + mean against the fp64 product;
+      forest    bit-exact against the oracle on 48 rows of the projection's own zhat;
+      dLin      slabs of 256 rows of dLin against the fp64 closed form of the batch-norm + linear gradient."""
+    B, K, T, depth, M = 16384, 784, 100, 7, 10
+    V = 2 ** depth - 1
+    N = T * V
+    eps = 1e-5
+    g = torch.Generator().manual_seed(6112)
+    x = torch.rand([B, K], generator=g).to(dev)
+    lin = (torch.randn([N, K], generator=g) / K ** 0.5).to(dev)
+    thr = 6.0 * torch.rand([T, V], generator=g) - 3.0
+    ordn = torch.arange(N, dtype=torch.int64).reshape(T, V)
+    w = torch.randn([T, 2 ** depth, M], generator=g)
+    ops.tree_fix_thresholds(thr, ordn, w)
+    print("case projection full size: forward", flush=True)
+    zhat, mean, rstd, var = ops.linear_bn_forward(x, lin, eps)
+    col_mean = zhat.double().mean(0)
+    col_var = zhat.double().var(0, unbiased=False)
+    assert col_mean.abs().max().item() <= 1e-5
+    assert (col_var - var.double() / (var.double() + eps)).abs().max().item() <= 1e-5
+    row_sets = [slice(0, 64), slice(B // 2 - 32, B // 2 + 32), slice(B - 64, B)]
+    col_sets = [slice(0, 256), slice(N // 2 - 128, N // 2 + 128), slice(N - 256, N)]
+    for rs in row_sets:
+        for cs in col_sets:
+            want = x[rs].double() @ lin[cs].double().t()
+            got = zhat[rs, cs].double() / rstd[cs].double() + mean[cs].double()
+            assert rel_err(got, want) <= 1e-5, (rs, cs)
+    rows = torch.cat([torch.arange(0, 24), torch.arange(B - 24, B)]).to(dev)
+    gthr, gord, gw = thr.to(dev), ordn.to(dev), w.to(dev)
+    out, rec = ops.tree_forward_records(zhat, gthr, gord, gw)
+    assert torch.equal(out[rows].cpu(), ho.forward(zhat[rows].cpu(), thr, ordn, w, False))
+    print("case projection full size: backward", flush=True)
+    gout = torch.randn([B, T, M], generator=torch.Generator(device=dev).manual_seed(6113), device=dev)
+    dz_in, dthr, _, dw = ops.tree_backward_records(rec, False, zhat, True, gthr, True, gord, False, gw, True, gout)
+    rdz, _, _ = ho.backward(zhat[rows].cpu(), thr, ordn, w, gout[rows].cpu())
+    assert rel_err(dz_in[rows].cpu(), rdz) <= 1e-5
+    up = dz_in.clone()
+    _, dlin = ops.linear_bn_backward(x, False, lin, True, zhat, rstd, dz_in)
+    x64 = x.double()
+    for cs in col_sets:
+        gd, rz = up[:, cs].double(), zhat[:, cs].double()
+        dz = rstd[cs].double() * (gd - gd.mean(0) - rz * (gd * rz).mean(0))
+        want = dz.t() @ x64
+        assert rel_err(dlin[cs].double(), want) <= 2e-5, cs
+        # the in-place batch-norm backward left dL/dz in the gradient buffer
+        assert rel_err(dz_in[:, cs].double(), dz) <= 1e-5, cs
+
+
+def test_conv_full_size(dev):
+    """The convolutional benchmark shape (images [32, 16, 128, 128] -> 64 channels, depth 6, 3 x 3 taps; the tiled
+    kernels run 2048 tiles per image batch with every interior / border combination) against the oracle on what it can
+    finish in seconds: all output rows of 2 images x 4 out channels, dX of one image restricted to those out channels,
+    and the conservation law over the whole batch: every (position, out channel, in channel) walk adds +c to one input
+    tap and -c to one threshold, and taps in the padding are dropped, so sum(dX) + sum(dThr) = -(sum of c over padding
+    taps) -- checked by a second backward on zero-padded images whose border takes those taps."""
+    B, C, Cout, H, W, depth = 32, 16, 64, 128, 128, 6
+    V, L = 2 ** depth - 1, 2 ** depth
+    g = torch.Generator().manual_seed(6112)
+    thr = 6.0 * torch.rand([Cout, C, V], generator=g) - 3.0
+    ordn = torch.randint(0, 9, [Cout, C, V], generator=g, dtype=torch.int64)
+    w = torch.randn([Cout, C, L], generator=g)
+    gg = torch.Generator(device=dev).manual_seed(6113)
+    x = torch.randn([B, C, H, W], generator=gg, device=dev)
+    gout = torch.randn([B, Cout, H, W], generator=gg, device=dev)
+    geo = ([3, 3], [1, 1], [1, 1], [1, 1])
+    gthr, gord, gw = thr.to(dev), ordn.to(dev), w.to(dev)
+    print("case conv full size: forward", flush=True)
+    out = ops.tree_conv2d_forward(x, gthr, gord, gw, *geo)
+    assert out.shape == (B, Cout, H, W)
+    imgs = [0, B - 1]
+    chans = [0, 21, 42, Cout - 1]
+    xs = x[imgs].cpu()
+    want = ho.conv_forward(xs, thr[chans].contiguous(), ordn[chans].contiguous(), w[chans].contiguous(), *geo, False)
+    assert torch.equal(out[imgs][:, chans].cpu(), want)
+    print("case conv full size: backward", flush=True)
+    dx, dthr, _, dw = ops.tree_conv2d_backward(x, True, gthr, True, gord, False, gw, True, gout, *geo)
+    # dX of one image from a subset of the out channels: the operator is linear in gout, so zero the other channels
+    gsub = torch.zeros_like(gout[:1])
+    gsub[:, chans] = gout[B - 1:, chans]
+    dx1, dthr1, _, dw1 = ops.tree_conv2d_backward(x[B - 1:].contiguous(), True, gthr, True, gord, False, gw, True, gsub, *geo)
+    rdx, rdthr, rdw = ho.conv_backward(x[B - 1:].cpu(), thr[chans].contiguous(), ordn[chans].contiguous(),
+                                       w[chans].contiguous(), gsub[:, chans].cpu().contiguous(), *geo)
+    assert rel_err(dx1.cpu(), rdx) <= 1e-5
+    assert rel_err(dthr1[chans].cpu(), rdthr) <= 1e-5 and rel_err(dw1[chans].cpu(), rdw) <= 1e-5
+    others = [c for c in range(Cout) if c not in chans]
+    assert dthr1[others].abs().max().item() == 0.0 and dw1[others].abs().max().item() == 0.0
+    # conservation over the whole batch: with the images zero-padded by hand (padding 0 on a 130 x 130 image is the
+    # same convolution) the border cells collect what the padded operator drops
+    xp = torch.nn.functional.pad(x, (1, 1, 1, 1))
+    dxp, dthrp, _, _ = ops.tree_conv2d_backward(xp, True, gthr, True, gord, False, gw, False, gout, [3, 3], [1, 1], [0, 0],
+                                                [1, 1])
+    mass = dxp.double().abs().sum().item()
+    assert abs(dxp.double().sum().item() + dthrp.double().sum().item()) <= 1e-5 * mass
+    assert rel_err(dxp[:, :, 1:-1, 1:-1], dx) <= 1e-5 and rel_err(dthrp, dthr) <= 1e-5
+    border = dxp.double().sum().item() - dxp[:, :, 1:-1, 1:-1].double().sum().item()
+    assert abs(dx.double().sum().item() + dthr.double().sum().item() + border) <= 1e-5 * mass

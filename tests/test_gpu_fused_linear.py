@@ -215,3 +215,34 @@ def test_empty_batch(dev):
     grads = ops.tree_fused_linear_backward(x, True, thr, True, ordn, False, w, True, lin, True, bias, True, gout)
     assert grads[2] is None and all(g.shape == t.shape and not g.any() for g, t in
                                     zip(grads[:2] + grads[3:], (x, thr, w, lin, bias)))
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+def test_batch_beyond_one_launch(dev, fern):
+    """More samples than one launch of the per-sample matrix product takes (one sample per blockIdx.z, at most 65535)
+    with several outputs per leaf: the product goes out in chunks. Rows from both chunks against the oracle (the
+    operator is row-wise in the forward and in dX), the parameter gradients against sums over the whole batch built
+    from the forest's own outputs."""
+    B, F, T, D, M, O = 65536 + 300, 12, 6, 3, 3, 4
+    x, thr, ordn, w, lin, bias, gout = _inputs((B, F, [], T, D, [M], O), fern, seed=3)
+    d = [t.to(dev) for t in (x, thr, ordn, w, lin, bias, gout)]
+    pre = "fern_" if fern else "tree_"
+    out = getattr(ops, pre + "fused_linear_forward")(*d[:6])
+    rows = torch.cat([torch.arange(0, 40), torch.arange(65535 - 20, 65535 + 20), torch.arange(B - 40, B)])
+    want = ho.fused_linear_forward(x[rows], thr, ordn, w, lin, bias, fern)
+    assert rel_err(out[rows.to(dev)].cpu(), want) <= TOL
+    for name in ("fused_linear_backward", "fused_linear_backward_deterministic"):
+        dx, dthr, _, dw, dlin, dbias = getattr(ops, pre + name)(d[0], True, d[1], True, d[2], False, d[3], True, d[4],
+                                                                True, d[5], True, d[6])
+        rdx, _, _, _ = ho.fused_linear_backward(x[rows], thr, ordn, w, lin, gout[rows], fern=fern)
+        assert rel_err(dx[rows.to(dev)].cpu(), rdx) <= TOL, name
+        f = getattr(ops, pre + "forward")(*d[:4]).double()                    # [B, T, M], bit-exact forest stage
+        want_dlin = torch.einsum("bom,btm->ot", d[6].double(), f)
+        # 197 508 terms per entry, summed in float32 (unsplit in deterministic mode): sqrt(n) * 2^-24 = 2.6e-5 of the
+        # terms' scale is what a float32 accumulator promises there; the reference's serial float32 loop gives no more
+        assert rel_err(dlin.double(), want_dlin) <= 4 * TOL, name
+        assert rel_err(dbias.double(), d[6].double().sum(dim=(0, 2))) <= 4 * TOL, name
+        # forest gradients: the plain forest backward on the mixed-down upstream gradient h = lin^T g
+        h = torch.einsum("ot,bom->btm", d[4].double(), d[6].double()).float().contiguous()
+        pdx, pdthr, _, pdw = getattr(ops, pre + "backward")(d[0], True, d[1], True, d[2], False, d[3], True, h)
+        assert rel_err(dthr, pdthr) <= 2 * TOL and rel_err(dw, pdw) <= 2 * TOL, name

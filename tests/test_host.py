@@ -218,3 +218,33 @@ def test_reference_snapshots_load_into_the_modules():
     wanted = ("forestbn1.", "features.", "forest.", "agg.")
     net.load_state_dict({k: v for k, v in sd.items() if k.startswith(wanted)})
     assert net.forest.ordinals.dtype == torch.int64 and torch.equal(net.forest.ordinals.data.float(), sd["forest.ordinals"])
+
+
+def test_gemm_tile_map_is_a_bijection():
+    """The matrix-product kernel deals its launch slots to result tiles in XCD bands and panels of 8 tile columns: every
+    tile must be named by exactly one slot, every other slot by none, for ragged and large tile grids alike (the
+    projection benchmark's products are 128 x 100 and 100 x 7 tiles; bands of more than one tile row and panels
+    narrower than 8 columns occur there)."""
+    lib = _lib.load()
+    grids = [(i, j) for i in range(1, 40) for j in range(1, 40)]
+    grids += [(128, 100), (100, 7), (100, 128), (129, 99), (7, 100), (1, 513), (513, 1), (512, 9)]
+    for ti, tj in grids:
+        slots = (ti + 7) // 8 * tj * 8
+        a = np.empty(slots, dtype=np.int32)
+        b = np.empty(slots, dtype=np.int32)
+        rc = lib.ht_gemm_tile_map(ti, tj, a.ctypes.data_as(ctypes.c_void_p), b.ctypes.data_as(ctypes.c_void_p), slots)
+        assert rc == _lib.HT_OK
+        live = a >= 0
+        assert ((b >= 0) == live).all()
+        assert int(live.sum()) == ti * tj, (ti, tj)
+        assert (a[live] < ti).all() and (b[live] < tj).all()
+        flat = a[live].astype(np.int64) * tj + b[live]
+        assert np.unique(flat).size == ti * tj, (ti, tj)
+        # slot s runs on L2 domain s % 8, which owns the band of tile rows [d * rows, (d + 1) * rows)
+        rows = (ti + 7) // 8
+        dom = np.arange(slots)[live] % 8
+        assert (a[live] // rows == dom).all(), (ti, tj)
+    # too little room for the slots is refused
+    small = np.empty(8, dtype=np.int32)
+    assert lib.ht_gemm_tile_map(128, 100, small.ctypes.data_as(ctypes.c_void_p), small.ctypes.data_as(ctypes.c_void_p),
+                                8) == _lib.HT_ERR_INVALID_ARGUMENT
