@@ -564,7 +564,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": f"{name}: {desc}", "backward_mode": args.mode, "path": args.path, "B": B, "F": F, "T": T, "depth": depth,
+        "config": {"workload": f"{name}: {desc}", "backward_mode": args.mode, "path": args.path, "host": ops.host, "B": B, "F": F, "T": T, "depth": depth,
                    "extra_outputs": M},
         "roofline": {"bound": "hbm",
                      "kernel": dominant or "forward kernel + tree kernel (the step's two large kernels; no current profile names the larger)",

@@ -1,8 +1,10 @@
-"""Builds hingetreefortorch_amd/libhingetree_hip.so from csrc/*.hip with hipcc for gfx950 (cross-compiles without a GPU).
+"""Builds hingetreefortorch_amd/libhingetree_hip.so from csrc/*.hip with hipcc for gfx950 (cross-compiles without a GPU)
+and, on top of it, the native host module hingetreefortorch_amd/_hingetree_host.so from csrc_host/hingetree_host.cpp
+with the host compiler against the installed torch headers.
 
     python -m hingetreefortorch_amd.build
 
-The objects go to hingetreefortorch_amd/build/, the shared library next to this file (in-tree, git-ignored).
+The objects go to hingetreefortorch_amd/build/, the two libraries next to this file (in-tree, git-ignored).
 """
 import concurrent.futures
 import os
@@ -64,6 +66,41 @@ def build_library(verbose=True):
     return LIB_PATH
 
 
+HOST_SRC = os.path.join(HERE, "csrc_host", "hingetree_host.cpp")
+HOST_PATH = os.path.join(HERE, "_hingetree_host.so")
+
+
+def build_host(verbose=True):
+    """The pybind11 / ATen host module (the compiled counterpart of hingetree_cpp.py's forest / fern / convolution
+    operators). Needs libhingetree_hip.so, which it links."""
+    import sysconfig
+
+    import torch
+
+    torch_dir = os.path.dirname(torch.__file__)
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cxx = os.environ.get("CXX") or shutil.which("g++") or "g++"
+    tmp = HOST_PATH + ".tmp"
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-w",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_hingetree_host",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=1",
+           "-I" + os.path.join(torch_dir, "include"),
+           "-I" + os.path.join(torch_dir, "include", "torch", "csrc", "api", "include"),
+           "-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(rocm, "include"),
+           HOST_SRC, "-o", tmp,
+           "-L" + os.path.join(torch_dir, "lib"), "-Wl,-rpath," + os.path.join(torch_dir, "lib"),
+           "-L" + HERE, "-Wl,-rpath,$ORIGIN", "-lhingetree_hip",
+           "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building the native host module failed:\n{proc.stdout}")
+    if verbose and proc.stdout.strip():
+        print(proc.stdout)
+    os.replace(tmp, HOST_PATH)
+    return HOST_PATH
+
+
 if __name__ == "__main__":
     print(build_library())
+    print(build_host())
     sys.exit(0)

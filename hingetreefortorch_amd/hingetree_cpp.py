@@ -7,6 +7,7 @@ device. This build has a single back-end, the HIP library: CPU tensors are rejec
 which the reference also keeps on the CPU), and operators outside the path raise.
 """
 import ctypes
+import os
 import time
 import weakref
 
@@ -82,6 +83,8 @@ _range_ok = {}  # id(tensor) -> (weakref, version, data_ptr, numel, bound) with 
 def forget_ordinal_checks():
     """Drop every remembered ordinal range check (for callers that overwrite ordinals through `.data`)."""
     _range_ok.clear()
+    if _native is not None:
+        _native.forget_ordinal_checks()
 
 
 def _validate_ordinals(ordinals, limit):
@@ -885,3 +888,69 @@ for _name in ["sparse_tree_backward", "sparse_fern_backward", "tree_init_medians
     globals()[_name] = _outside(_name)
 
 __all__ = [n for n in list(globals()) if n.split("_")[0] in ("tree", "fern", "sparse", "trie", "contract", "expand", "linear")]
+
+
+# ---- native host ----------------------------------------------------------------------------------------------------
+# Where the compiled host module has been built (csrc_host/hingetree_host.cpp -> _hingetree_host.so, a pybind11 / ATen
+# extension like the reference's own hingetree_cpp), the operators of the forest / fern / convolution path are ITS
+# functions: validation, allocation and the launch happen in C++ on torch's current stream, which halves the cost of a
+# call for launch-bound shapes. The functions above stay as the host for everything else (forest -> linear, the
+# expanded forest, contract / expand, the projection) and as the whole host where the module is not built or
+# HINGETREE_HOST=python is set. `host` names the one in use; `use_host` switches at run time.
+_NATIVE_NAMES = [f"{kind}_{op}" for kind in ("tree", "fern")
+                 for op in ("forward", "backward", "backward_deterministic", "forward_records", "backward_records",
+                            "leafmap", "marginmap", "reachability", "check_thresholds", "fix_thresholds",
+                            "conv1d_forward", "conv1d_backward", "conv2d_forward", "conv2d_backward", "conv3d_forward",
+                            "conv3d_backward")]
+_INTERNAL_NAMES = ["_forward", "_backward", "_forward_records", "_backward_records", "_maps", "_thresholds",
+                   "_conv_forward", "_conv_backward"]
+_python_host = {n: globals()[n] for n in _NATIVE_NAMES + _INTERNAL_NAMES}
+_native = None
+host = "python"
+
+
+def _load_native():
+    try:
+        from . import _hingetree_host as native
+    except ImportError:
+        return None
+    if native.abi_version != L.load().ht_abi_version():
+        raise RuntimeError("hingetreefortorch_amd/_hingetree_host.so was built against another libhingetree_hip.so; "
+                           "run `python -m hingetreefortorch_amd.build`.")
+    return native
+
+
+def use_host(name):
+    """Select the host layer of the forest / fern / convolution operators: "native" (the compiled module; raises if it
+    has not been built) or "python" (this file over ctypes)."""
+    global _native, host
+    g = globals()
+    if name == "python":
+        g.update(_python_host)
+        host = "python"
+        return
+    if name != "native":
+        raise ValueError("host must be 'native' or 'python'")
+    if _native is None:
+        _native = _load_native()
+        if _native is None:
+            raise RuntimeError("the native host module is not built; run `python -m hingetreefortorch_amd.build`.")
+    n = _native
+    for fn in _NATIVE_NAMES:
+        g[fn] = getattr(n, fn)
+    wants = {"leaf": 0, "margin": 1, "reach": 2}
+    g["_forward"], g["_backward"] = n.forest_forward, n.forest_backward
+    g["_forward_records"], g["_backward_records"] = n.forest_forward_records, n.forest_backward_records
+    g["_maps"] = lambda kind, x, thr, ordn, w, want: n.forest_maps(kind, x, thr, ordn, w, wants[want])
+    g["_thresholds"] = n.forest_thresholds
+    g["_conv_forward"], g["_conv_backward"] = n.conv_forward, n.conv_backward
+    host = "native"
+
+
+if os.environ.get("HINGETREE_HOST", "native") != "python":
+    try:
+        use_host("native")
+    except RuntimeError as _e:
+        if "another libhingetree_hip.so" in str(_e):
+            raise
+

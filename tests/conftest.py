@@ -52,3 +52,17 @@ def rel_err(a, b):
     """max |a-b| relative to max |b| (norm-wise)."""
     denom = b.abs().max().item()
     return (a - b).abs().max().item() / (denom if denom > 0 else 1.0)
+
+
+@pytest.fixture(params=["native", "python"])
+def either_host(request):
+    """Runs a test once per host layer of the operator module: the compiled pybind11 / ATen module and the Python file
+    over ctypes. Skips the native run where that module has not been built."""
+    import hingetree_cpp as ops
+    before = ops.host
+    try:
+        ops.use_host(request.param)
+    except RuntimeError as e:
+        pytest.skip(str(e))
+    yield request.param
+    ops.use_host(before)

@@ -37,7 +37,7 @@ def test_no_fallback_when_library_missing(monkeypatch):
         _lib.load()
 
 
-def test_validation_order_on_cpu_tensors():
+def test_validation_order_on_cpu_tensors(either_host):
     x, thr, ordn, w, gout = make_forest(8, 5, [], 3, 2, [], False, torch.float32)
     with pytest.raises(ValueError, match="share the same torch real number data type"):
         ops.tree_forward(x.double(), thr, ordn, w)
@@ -78,7 +78,7 @@ def test_validation_order_on_cpu_tensors():
         ops.tree_fused_linear_forward(x, thr, ordn, w, lin, bias)
 
 
-def test_conv_validation_on_cpu_tensors():
+def test_conv_validation_on_cpu_tensors(either_host):
     x = torch.randn(2, 3, 8, 8)
     thr, ordn, w = torch.randn(4, 3, 7), torch.randint(0, 9, (4, 3, 7)), torch.randn(4, 3, 8)
     with pytest.raises(ValueError, match="expected to have 2 dimensions"):
@@ -113,7 +113,7 @@ def test_conv_output_size_matches_torch():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-def test_thresholds_match_oracle_and_golden(dtype):
+def test_thresholds_match_oracle_and_golden(dtype, either_host):
     z = np.load(os.path.join(GOLDEN, "fix_thresholds.npz"))
     thr = torch.from_numpy(z["before"]).clone()
     ordn, w = torch.from_numpy(z["ord"]), torch.from_numpy(z["w"])
