@@ -96,8 +96,10 @@ int make_dims(const ht_forest_shape *s, ForestDims *d);
 // Packed (threshold, ordinal) vertices: layout in walk.hpp (Node<Real>), T*V entries.
 template <typename Real>
 size_t packed_nodes_bytes(const ForestDims &d);
+// zero_slots (optional): kBoundSlots 64-bit words (records.hpp) that the same launch clears.
 template <typename Real>
-int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *dst, hipStream_t stream);
+int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *dst, hipStream_t stream,
+               unsigned long long *zero_slots = nullptr);
 
 template <typename Real>
 size_t forest_forward_workspace(const ForestDims &d);

@@ -46,11 +46,12 @@ __global__ __launch_bounds__(kForestThreads) void records_kernel(ForestDims d, c
   }
   const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
   const long long s = s0 + j;
-  if (s >= d.S) return;
-  const long long xbase = (s / d.K) * d.FK + (s % d.K);
+  const bool live = s < d.S;  // (dead lanes stay for the wavefront-wide publication of the margin bound)
+  const long long xbase = live ? (s / d.K) * d.FK + (s % d.K) : 0;
   const int t_begin = blockIdx.y * trees_per_block;
   const int t_end = min(d.T, t_begin + trees_per_block);
-  for (int tb = t_begin + tt; tb < t_end; tb += TC * kIlp) {
+  MarginBits margin_bound;
+  for (int tb = t_begin + tt; live && tb < t_end; tb += TC * kIlp) {
     const Node<Real> *nd[kIlp];
     int t[kIlp];
 #pragma unroll
@@ -65,9 +66,12 @@ __global__ __launch_bounds__(kForestThreads) void records_kernel(ForestDims d, c
       walk_many<Real, FERN, kIlp>(d.depth, nd, [&](int, int f) { return x[xbase + (long long)f * d.K]; }, r);
 #pragma unroll
     for (int i = 0; i < kIlp; ++i)
-      if (t[i] < t_end)
+      if (t[i] < t_end) {
         rec.put((long long)t[i] * d.S + s, r[i].key, r[i].vertex, r[i].ord, r[i].margin);
+        margin_bound.take(r[i].margin);
+      }
   }
+  bound_publish(margin_bound_value<Real>(margin_bound.bits), rec.bound, (blockIdx.y * gridDim.x + blockIdx.x) % unsigned(kBoundSlots));
 }
 
 template <typename Real, bool FERN, int BT, bool XLDS, bool COMPACT>
@@ -117,62 +121,66 @@ struct DetHeader {
   double scale_w, inv_scale_w, scale_c, inv_scale_c;
   int fallback_w, fallback_c;
 };
-constexpr size_t kDetHeaderBytes = 256;
+// The bound on |c| is taken by the tree kernels as they store c (one running maximum per lane, one atomic per
+// wavefront): the atomics go to kDetSlots slots behind the header, spread by workgroup, because thousands of atomics
+// on ONE address serialise in L2 for longer than a pass over c takes; the scale kernel folds the slots.
+constexpr int kDetSlots = 4096;
+constexpr size_t kDetHeaderBytes = 256 + size_t(kDetSlots) * sizeof(unsigned long long);
+__device__ __forceinline__ unsigned long long *det_slots(DetHeader *h) {
+  return reinterpret_cast<unsigned long long *>(reinterpret_cast<unsigned char *>(h) + 256);
+}
 
-__global__ void det_init_kernel(DetHeader *h) {
+__global__ __launch_bounds__(256) void det_init_kernel(DetHeader *h) {
   if (threadIdx.x == 0) {
     h->max_g = h->max_a = h->max_c = 0ull;
     h->scale_w = h->inv_scale_w = h->scale_c = h->inv_scale_c = 1.0;
     h->fallback_w = h->fallback_c = 0;
   }
+  for (int i = threadIdx.x; i < kDetSlots; i += 256) det_slots(h)[i] = 0ull;
 }
 
-// max |p[i]| (NaN counts as +inf) folded into *slot. Four independent 16-byte loads are in flight per thread.
+// A lane's bound on |c| (bound_take, records.hpp) over the wavefront into the workgroup's slot.
 template <typename Real>
-__global__ __launch_bounds__(256) void absmax_kernel(const Real *__restrict__ p, long long n,
-                                                     unsigned long long *slot) {
+__device__ __forceinline__ void publish_c_bound(Real m, const DetHeader *hdr) {
+  bound_publish(double(m), det_slots(const_cast<DetHeader *>(hdr)),
+                (blockIdx.y * gridDim.x + blockIdx.x) % unsigned(kDetSlots));
+}
+
+// max |p[i]| (NaN counts as +inf) folded into *slot. A grid-stride loop of plain 16-byte loads, one in flight per
+// thread: with 2048 workgroups of 512 threads that is the form in which a read stream runs fastest here (6.4 TB/s
+// measured; four loads in flight per thread gave 5.4).
+constexpr int kAbsmaxThreads = 512;
+template <typename Real>
+__global__ __launch_bounds__(kAbsmaxThreads) void absmax_kernel(const Real *__restrict__ p, long long n,
+                                                                unsigned long long *slot) {
   constexpr int VEC = 16 / sizeof(Real);
-  constexpr int kInFlight = 4;
   typedef Real Vec __attribute__((ext_vector_type(VEC)));
   Real m = Real(0);
-  auto take = [&](Real r) {
-    const Real v = ht_abs(r);
-    if (!(v <= m)) m = (v != v) ? Real(INFINITY) : v;
-  };
-  const long long tid = (long long)blockIdx.x * 256 + threadIdx.x, nthreads = (long long)gridDim.x * 256;
+  const long long tid = (long long)blockIdx.x * kAbsmaxThreads + threadIdx.x;
+  const long long nthreads = (long long)gridDim.x * kAbsmaxThreads;
   long long body = 0;
   if (reinterpret_cast<uintptr_t>(p) % 16 == 0) {
     body = n / VEC;
     const Vec *pv = reinterpret_cast<const Vec *>(p);
-    long long i = tid;
-    for (; i + (kInFlight - 1) * nthreads < body; i += kInFlight * nthreads) {
-      Vec v[kInFlight];
+    for (long long i = tid; i < body; i += nthreads) {
+      const Vec v = pv[i];
 #pragma unroll
-      for (int q = 0; q < kInFlight; ++q) v[q] = __builtin_nontemporal_load(pv + i + q * nthreads);
-#pragma unroll
-      for (int q = 0; q < kInFlight; ++q)
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) take(v[q][e]);
-    }
-    for (; i < body; i += nthreads) {
-      const Vec v = __builtin_nontemporal_load(pv + i);
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) take(v[e]);
+      for (int e = 0; e < VEC; ++e) bound_take(m, v[e]);
     }
     body *= VEC;
   }
-  for (long long i = body + tid; i < n; i += nthreads) take(p[i]);
+  for (long long i = body + tid; i < n; i += nthreads) bound_take(m, p[i]);
   double md = double(m);
   for (int off = 32; off > 0; off >>= 1) {
     const double o = __shfl_xor(md, off, kWave);
     if (!(o <= md)) md = o;
   }
   // one atomic per workgroup: thousands of atomics on the one slot would serialise in L2 for longer than the pass reads
-  __shared__ double part[256 / kWave];
+  __shared__ double part[kAbsmaxThreads / kWave];
   if ((threadIdx.x & (kWave - 1)) == 0) part[threadIdx.x / kWave] = md;
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int i = 1; i < 256 / kWave; ++i)
+    for (int i = 1; i < kAbsmaxThreads / kWave; ++i)
       if (!(part[i] <= md)) md = part[i];
     if (md > 0.0) atomicMax(slot, (unsigned long long)__double_as_longlong(md));
   }
@@ -200,7 +208,21 @@ __device__ inline void det_pick_scale(double bound, double count, double *scale,
   *inv = ldexp(1.0, -k);
 }
 
-__global__ void det_scale_kernel(DetHeader *h, int which, double count) {
+__global__ __launch_bounds__(kWave) void det_scale_kernel(DetHeader *h, int which, double count, bool fold_slots,
+                                                          const unsigned long long *margin_slots) {
+  if (which == 0 && margin_slots) {
+    unsigned long long m = 0ull;
+    for (int i = threadIdx.x; i < kBoundSlots; i += kWave) m = max(m, margin_slots[i]);
+    for (int off = 32; off > 0; off >>= 1) m = max(m, (unsigned long long)__shfl_xor((long long)m, off, kWave));
+    if (threadIdx.x == 0) h->max_a = m;
+  }
+  if (which == 1 && fold_slots) {
+    // bit patterns of non-negative doubles order like the values
+    unsigned long long m = 0ull;
+    for (int i = threadIdx.x; i < kDetSlots; i += kWave) m = max(m, det_slots(h)[i]);
+    for (int off = 32; off > 0; off >>= 1) m = max(m, (unsigned long long)__shfl_xor((long long)m, off, kWave));
+    if (threadIdx.x == 0) h->max_c = m;
+  }
   if (threadIdx.x != 0) return;
   if (which == 0)
     det_pick_scale(__longlong_as_double((long long)h->max_g) * __longlong_as_double((long long)h->max_a), count,
@@ -389,7 +411,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
     }
   };
 
-  Real c_mine = Real(0);
+  Real c_mine = Real(0), c_bound = Real(0);
   for (long long c = 0; c < nchunks; ++c) {
     const int sub0 = int(c & (CPB - 1)) * U;
     Chunk cur;
@@ -434,8 +456,12 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
         if (my_sub == sub0 + u) c_mine = got;
       }
     }
-    if (need_c && sub0 + U == P && cur.have) rec.c[cur.at] = c_mine;
+    if (need_c && sub0 + U == P && cur.have) {
+      rec.c[cur.at] = c_mine;
+      if (FIXED) bound_take(c_bound, c_mine);
+    }
   }
+  if (FIXED && need_c) publish_c_bound(c_bound, hdr);
   if (dw) {
     __syncthreads();
     Real *dst = dw + (long long)t0 * LM;
@@ -652,6 +678,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
       }
     });
   };
+  float c_bound = 0.f;  // FIXED: largest |c| this lane stored
   auto compute = [&](Stage &st, long long sblk, bool have, const bool (&on)[P], auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
     float c_mine = 0.f;
@@ -688,6 +715,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     if (need_c && (FULL || have)) {
       const float c = ht_sign(st.mg_own) * c_mine;
       rec.c[record_index(sblk, have)] = c;
+      if (FIXED) bound_take(c_bound, c);
       if (dthr_fold) atomicAdd(acc_thr + uint32_t(rec_t) * uint32_t(d.V) + st.v_own, -double(c));
     }
   };
@@ -803,7 +831,13 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
         c4[2] = consume(l0, cur, 2);
         issue(l0, sb_next, nxt, 0);
         c4[3] = consume(l1, cur, 3);
-        if (need_c) *reinterpret_cast<Float4 *>(rec.c + rec_lane_at + sb) = c4;
+        if (need_c) {
+          *reinterpret_cast<Float4 *>(rec.c + rec_lane_at + sb) = c4;
+          if (FIXED) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) bound_take(c_bound, c4[k]);
+          }
+        }
         cur = nxt;
       }
       s_rest = s_begin + rounds * stride4;
@@ -858,6 +892,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     issue_w(st, on);
     compute(st, sblk, have, on, std::false_type{});
   }
+  if (FIXED && need_c) publish_c_bound(c_bound, hdr);
   if (dw || dthr_fold) __syncthreads();
   if (dthr_fold) {
     float *dst = dthr_fold + (long long)t0 * d.V;
@@ -959,6 +994,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
     float mg;
     Float4U gv;
   };
+  float c_bound = 0.f;  // FIXED: largest |c| this lane stored
   long long img_sb = -1, img_at = -1, img_base = 0;  // IMAGE: the sample block the cached offsets belong to
   auto issue = [&](Step &st, long long sb, int tl) {
     const long long s_raw = sb + pr;
@@ -994,7 +1030,11 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
       partial = __builtin_fmaf(wv[2], st.gv[2], partial);
       partial = __builtin_fmaf(wv[3], st.gv[3], partial);
       const float total = row_group_sum<P>(partial);
-      if (st.on && e0 == 0) rec.c[st.at] = ht_sign(st.mg) * total;
+      if (st.on && e0 == 0) {
+        const float c = ht_sign(st.mg) * total;
+        rec.c[st.at] = c;
+        if (FIXED) bound_take(c_bound, c);
+      }
     }
     if (dw && st.on) {
       const float a = ht_abs(st.mg);
@@ -1042,6 +1082,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
     }
     if (second) finish(s1, tl1);
   }
+  if (FIXED && need_c) publish_c_bound(c_bound, hdr);
 
   if (dw) {
     __syncthreads();
@@ -1781,10 +1822,10 @@ static FixedLayout fixed_layout(const ForestDims &d, bool need_dthr, bool need_d
 template <typename Real>
 int launch_absmax(const Real *p, long long n, unsigned long long *slot, hipStream_t stream) {
   if (n <= 0) return HT_OK;
-  long long blocks = (n / (16 / (long long)sizeof(Real)) + 255) / 256;
+  long long blocks = (n / (16 / (long long)sizeof(Real)) + kAbsmaxThreads - 1) / kAbsmaxThreads;
   if (blocks > 8 * kNumCUs) blocks = 8 * kNumCUs;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL((absmax_kernel<Real>), dim3((unsigned)blocks), dim3(256), 0, stream, p, n, slot);
+  hipLaunchKernelGGL((absmax_kernel<Real>), dim3((unsigned)blocks), dim3(kAbsmaxThreads), 0, stream, p, n, slot);
   HT_LAUNCH_CHECK("forest backward (magnitude bound)");
   return HT_OK;
 }
@@ -1816,12 +1857,13 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
     hdr = reinterpret_cast<DetHeader *>(base + lay.header);
     dw_fixed = reinterpret_cast<unsigned long long *>(base + lay.dw);
     dthr_fixed = reinterpret_cast<unsigned long long *>(base + lay.dthr);
-    hipLaunchKernelGGL(det_init_kernel, dim3(1), dim3(kWave), 0, stream, hdr);
+    hipLaunchKernelGGL(det_init_kernel, dim3(1), dim3(256), 0, stream, hdr);
     HT_LAUNCH_CHECK("forest backward (deterministic header)");
     if (dw) {
       if ((rc = launch_absmax<Real>(gout, pairs * d.M, &hdr->max_g, stream)) != HT_OK) return rc;
-      if ((rc = launch_absmax<Real>(rec.margin, pairs, &hdr->max_a, stream)) != HT_OK) return rc;
-      hipLaunchKernelGGL(det_scale_kernel, dim3(1), dim3(kWave), 0, stream, hdr, 0, double(d.S));
+      // (the bound on |margin| came with the records)
+      hipLaunchKernelGGL(det_scale_kernel, dim3(1), dim3(kWave), 0, stream, hdr, 0, double(d.S), false,
+                         (const unsigned long long *)rec.bound);
       HT_LAUNCH_CHECK("forest backward (dW scale)");
       if (plan.parts > 1 && (rc = zero_fill(dw_fixed, size_t(d.T) * d.L * d.M * 8, stream)) != HT_OK) return rc;
     }
@@ -1856,9 +1898,9 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
       HT_LAUNCH_CHECK("forest backward (dW fallback)");
     }
     if (need_c) {
-      if ((rc = launch_absmax<Real>(rec.c, pairs, &hdr->max_c, stream)) != HT_OK) return rc;
+      // the tree kernel left its bound on |c| in the header's slots
       hipLaunchKernelGGL(det_scale_kernel, dim3(1), dim3(kWave), 0, stream, hdr, 1,
-                         double(d.S > d.T ? d.S : (long long)d.T));
+                         double(d.S > d.T ? d.S : (long long)d.T), true, (const unsigned long long *)nullptr);
       HT_LAUNCH_CHECK("forest backward (c scale)");
     }
   }
@@ -2058,9 +2100,10 @@ int forest_backward(const ForestDims &d, bool fern, const Real *x, const Real *t
   const size_t need = node_bytes + route_bytes<Real>(d, route, dthr != nullptr, dw != nullptr, false);
   if (ws == nullptr || ws_bytes < need)
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the backward pass.");
-  if ((rc = pack_nodes<Real>(d, thr, ord, ws, stream)) != HT_OK) return rc;
-  const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
   unsigned char *saved = static_cast<unsigned char *>(ws) + node_bytes;
+  unsigned long long *slots = route == Route::kFused ? nullptr : records_bound_slots<Real>(d, saved);
+  if ((rc = pack_nodes<Real>(d, thr, ord, ws, stream, slots)) != HT_OK) return rc;
+  const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
   unsigned char *scratch = saved + records_saved_bytes<Real>(d);
   return run_route<Real>(d, route, fern, x, nodes, w, gout, dx, dthr, dw, saved, scratch, true, stream, gout_image);
 }

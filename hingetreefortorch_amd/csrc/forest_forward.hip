@@ -18,7 +18,10 @@ namespace {
 
 template <typename Real>
 __global__ __launch_bounds__(256) void pack_nodes_kernel(const Real *__restrict__ thr, const int64_t *__restrict__ ord,
-                                                         Node<Real> *__restrict__ nodes, long long n, int F) {
+                                                         Node<Real> *__restrict__ nodes, long long n, int F,
+                                                         unsigned long long *zero_slots) {
+  if (zero_slots && blockIdx.x == 0)
+    for (int k = threadIdx.x; k < kBoundSlots; k += 256) zero_slots[k] = 0ull;
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) {
     Node<Real> v;
@@ -67,6 +70,7 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
 
   const int t_begin = blockIdx.y * trees_per_block;
   const int t_end = min(d.T, t_begin + trees_per_block);
+  MarginBits margin_bound;  // RECORD: bound on the |margin| this lane recorded
   for (int tb = t_begin; tb < t_end; tb += TP) {
     if (live && tb + tt < t_end) {
       const Node<Real> *nd[kIlp];
@@ -84,8 +88,10 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
       for (int i = 0; i < kIlp; ++i) {
         r_abs[j * LDR + tt + i * TC] = ht_abs(r[i].margin);
         r_key[j * LDR + tt + i * TC] = KeyT(r[i].key);
-        if (RECORD && tb + tt + i * TC < t_end)
+        if (RECORD && tb + tt + i * TC < t_end) {
           rec.put((long long)(tb + tt + i * TC) * d.S + s, r[i].key, r[i].vertex, r[i].ord, r[i].margin);
+          margin_bound.take(r[i].margin);
+        }
       }
     }
     __syncthreads();
@@ -180,6 +186,7 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
     }
     __syncthreads();
   }
+  if (RECORD) bound_publish(margin_bound_value<Real>(margin_bound.bits), rec.bound, (blockIdx.y * gridDim.x + blockIdx.x) % unsigned(kBoundSlots));
 }
 
 
@@ -207,7 +214,10 @@ static inline long long quads_per_tree(int depth) {
 }
 
 __global__ __launch_bounds__(256) void pack_quads_kernel(const float *__restrict__ thr, const int64_t *__restrict__ ord,
-                                                         QuadNode *__restrict__ quads, int T, int V, int NQ, int F) {
+                                                         QuadNode *__restrict__ quads, int T, int V, int NQ, int F,
+                                                         unsigned long long *zero_slots) {
+  if (zero_slots && blockIdx.x == 0)
+    for (int k = threadIdx.x; k < kBoundSlots; k += 256) zero_slots[k] = 0ull;
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (long long)T * NQ) return;
   const int t = int(i / NQ), q = int(i - (long long)t * NQ);
@@ -355,6 +365,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
   const int t_begin = blockIdx.y * trees_per_block;
   const int t_end = min(d.T, t_begin + trees_per_block);
   const uint32_t TM = uint32_t(d.T) * uint32_t(d.M);
+  MarginBits margin_bound;  // RECORD: bound on the |margin| this lane recorded
 
   for (int tb = t_begin + wave * TPW; tb < t_end; tb += kWaves * TPW) {
     // ---- walk: this lane's sample through trees tb + slot + i * SLOTS
@@ -426,10 +437,14 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
       }
 #pragma unroll
       for (int i = 0; i < kRowIlp; ++i) {
-        p_abs[j * LDP + slot + i * SLOTS] = ht_abs(r[i].margin);
+        const Real a = ht_abs(r[i].margin);
+        p_abs[j * LDP + slot + i * SLOTS] = a;
         p_key[j * LDP + slot + i * SLOTS] = uint16_t(r[i].key);
         if (RECORD && live && tb + slot + i * SLOTS < t_end)
           rec.put((long long)(tb + slot + i * SLOTS) * d.S + s, r[i].key, r[i].vertex, r[i].ord, r[i].margin);
+        // (surplus slots re-walk an existing tree and dead lanes a zero row of the tile: their margins may join the
+        // bound, which then costs no predicate)
+        if (RECORD) margin_bound.take_abs(a);
       }
     }
     // the parked results are read by other lanes of this wavefront only
@@ -515,6 +530,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
     // requests in order
     __builtin_amdgcn_wave_barrier();
   }
+  if (RECORD) bound_publish(margin_bound_value<Real>(margin_bound.bits), rec.bound, (blockIdx.y * gridDim.x + blockIdx.x) % unsigned(kBoundSlots));
 }
 
 template <typename Real>
@@ -690,11 +706,12 @@ size_t packed_nodes_bytes(const ForestDims &d) {
 }
 
 template <typename Real>
-int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *dst, hipStream_t stream) {
+int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *dst, hipStream_t stream,
+               unsigned long long *zero_slots) {
   const long long n = (long long)d.T * d.V;
   if (n == 0) return HT_OK;
   hipLaunchKernelGGL(pack_nodes_kernel<Real>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, thr, ord,
-                     static_cast<Node<Real> *>(dst), n, d.F);
+                     static_cast<Node<Real> *>(dst), n, d.F, zero_slots);
   HT_LAUNCH_CHECK("pack vertices");
   return HT_OK;
 }
@@ -772,6 +789,8 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the forward pass.");
   ImageStore img{};
   if (image) img = *image;
+  // the walk records' bound slots are cleared by whichever vertex-packing pre-pass runs below
+  unsigned long long *slots = records ? records_bound_slots<Real>(d, records) : nullptr;
   if (img.nd && d.K == 1)
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: an image result needs inner data positions (inData of 3 or more dimensions).");
   if (rows_ok<Real>(d)) {
@@ -800,17 +819,17 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
         const int NQ = int(quads_per_tree(d.depth));
         const long long n = (long long)d.T * NQ;
         hipLaunchKernelGGL(pack_quads_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, thr, ord,
-                           static_cast<QuadNode *>(ws), d.T, d.V, NQ, d.F);
+                           static_cast<QuadNode *>(ws), d.T, d.V, NQ, d.F, slots);
         HT_LAUNCH_CHECK("pack two-level vertices");
         return dispatch_rows<Real, false, true>(d, x, ws, w, wpitch, out, records, stream);
       }
     }
-    int rc = pack_nodes<Real>(d, thr, ord, ws, stream);
+    int rc = pack_nodes<Real>(d, thr, ord, ws, stream, slots);
     if (rc != HT_OK) return rc;
     return fern ? dispatch_rows<Real, true, false>(d, x, ws, w, wpitch, out, records, stream)
                 : dispatch_rows<Real, false, false>(d, x, ws, w, wpitch, out, records, stream);
   }
-  int rc = pack_nodes<Real>(d, thr, ord, ws, stream);
+  int rc = pack_nodes<Real>(d, thr, ord, ws, stream, slots);
   if (rc != HT_OK) return rc;
   const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
   return fern ? dispatch_forward<Real, true>(d, x, nodes, w, out, records, stream, img)
@@ -819,7 +838,8 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
 
 #define HT_INSTANTIATE(Real)                                                                                          \
   template size_t packed_nodes_bytes<Real>(const ForestDims &);                                                       \
-  template int pack_nodes<Real>(const ForestDims &, const Real *, const int64_t *, void *, hipStream_t);              \
+  template int pack_nodes<Real>(const ForestDims &, const Real *, const int64_t *, void *, hipStream_t,                \
+                                unsigned long long *);                                                                \
   template size_t forest_forward_workspace<Real>(const ForestDims &);                                                 \
   template int forest_forward<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,            \
                                     const Real *, Real *, void *, void *, size_t, hipStream_t, const ImageStore *);
