@@ -250,72 +250,89 @@ constexpr int kTopQuads = 5;  // quads of the first two level pairs (levels 0..3
 // TOP_LDS: top[i] is an LDS copy of the first kTopQuads quads of walk i's tree; levels 0..3 are then read from LDS
 // (the same for all samples of a tree slot: broadcasts), which takes two of the five dependent memory round trips
 // out of a depth-10 walk.
-template <int N, int BT, bool TOP_LDS>
+//
+// The walk is bound by its vector instructions, so a level is kept to the few that the semantics need: the decisions
+// are shifted into `path` through the carry of one add (path = 2 * path + (margin > 0): most significant bit first,
+// which is also the index of the current vertex inside its level), the running minimum is the signed margin itself
+// (compared by magnitude; the root seeds it, so a NaN root sticks as in the reference, HingeTreeCommon.h:157-178),
+// and beside it only the level and ordinal of the minimum are carried, packed in one word. The leaf key (decision of
+// level i in bit i) is the bit reversal of the finished path, the selected vertex is rebuilt from the path and the
+// level. TRACK = false (no walk records wanted) carries |margin| alone: r.margin is then the magnitude, r.vertex and
+// r.ord are 0.
+template <int N, int BT, bool TOP_LDS, bool TRACK>
 __device__ __forceinline__ void walk_quads(int depth, const QuadNode *const (&quads)[N],
                                            const QuadNode *const (&top)[N], const float *xs_j,
                                            WalkResult<float> (&r)[N]) {
-  uint32_t idx[N];
-  float best_abs[N];
-#pragma unroll
-  for (int i = 0; i < N; ++i) {
-    idx[i] = 0;
-    r[i].key = 0;
-    r[i].vertex = 0;
-    r[i].ord = 0;
-    r[i].margin = 0.f;
-    best_abs[i] = 0.f;
-  }
-  uint32_t base = 0, width = 1;  // first quad / number of quads of the current level pair
+  uint32_t path[N], info[N];  // info: ordinal | level << kQuadOrdinalBits of the smallest |margin| so far
+  float best[N];              // TRACK: its signed margin; else its magnitude
   constexpr uint32_t kMask = (1u << kQuadOrdinalBits) - 1;
+#pragma unroll
+  for (int i = 0; i < N; ++i) path[i] = 0, info[i] = 0, best[i] = 0.f;
+  float root[N];
+  uint32_t base = 0, width = 1;  // first quad / number of quads of the current level pair
+  auto take = [&](int i, float m, uint32_t ord, int lvl) {
+    if (TRACK) {
+      const bool closer = ht_abs(m) < ht_abs(best[i]);
+      best[i] = closer ? m : best[i];
+      info[i] = closer ? (ord | (uint32_t(lvl) << kQuadOrdinalBits)) : info[i];
+    } else {
+      best[i] = __builtin_fminf(best[i], ht_abs(m));  // a NaN margin never wins; a NaN root is put back below
+    }
+  };
   for (int lvl = 0; lvl < depth; lvl += 2) {
     QuadNode n[N];
     if (TOP_LDS && lvl < 4) {
 #pragma unroll
-      for (int i = 0; i < N; ++i) n[i] = top[i][base + idx[i]];
+      for (int i = 0; i < N; ++i) n[i] = top[i][base + path[i]];
     } else {
 #pragma unroll
-      for (int i = 0; i < N; ++i) n[i] = quads[i][base + idx[i]];
+      for (int i = 0; i < N; ++i) n[i] = quads[i][base + path[i]];
     }
     float m0[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) m0[i] = xs_j[(n[i].ords & kMask) * BT] - n[i].thr;
-    const uint32_t first = (1u << lvl) - 1u;  // heap index of the level's first vertex
     const bool two = lvl + 1 < depth;
     float m1[N];
-    uint32_t o1[N], b0[N];
+    uint32_t o1[N];
+    bool right0[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      b0[i] = (m0[i] > 0.f) ? 1u : 0u;
-      const float t1 = b0[i] ? n[i].thr_right : n[i].thr_left;
-      o1[i] = (n[i].ords >> (b0[i] ? 2 * kQuadOrdinalBits : kQuadOrdinalBits)) & kMask;
+      right0[i] = m0[i] > 0.f;
+      const float t1 = right0[i] ? n[i].thr_right : n[i].thr_left;
+      o1[i] = (n[i].ords >> (right0[i] ? 2 * kQuadOrdinalBits : kQuadOrdinalBits)) & kMask;
       m1[i] = two ? xs_j[o1[i] * BT] - t1 : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const uint32_t v0 = first + idx[i];
-      const float a0 = ht_abs(m0[i]);
-      if (lvl == 0 || a0 < best_abs[i]) {
-        best_abs[i] = a0;
-        r[i].margin = m0[i];
-        r[i].vertex = v0;
-        r[i].ord = n[i].ords & kMask;
+      if (lvl == 0) {
+        root[i] = m0[i];
+        best[i] = TRACK ? m0[i] : ht_abs(m0[i]);
+        info[i] = n[i].ords & kMask;
+      } else {
+        take(i, m0[i], n[i].ords & kMask, lvl);
       }
-      r[i].key |= b0[i] << lvl;
+      path[i] = path[i] + path[i] + (right0[i] ? 1u : 0u);
       if (two) {
-        const uint32_t b1 = (m1[i] > 0.f) ? 1u : 0u;
-        const float a1 = ht_abs(m1[i]);
-        if (a1 < best_abs[i]) {
-          best_abs[i] = a1;
-          r[i].margin = m1[i];
-          r[i].vertex = 2u * v0 + 1u + b0[i];
-          r[i].ord = o1[i];
-        }
-        r[i].key |= b1 << (lvl + 1);
-        idx[i] = 4u * idx[i] + 2u * b0[i] + b1;
+        take(i, m1[i], o1[i], lvl + 1);
+        path[i] = path[i] + path[i] + ((m1[i] > 0.f) ? 1u : 0u);
       }
     }
     base += width;
     width *= 4u;
+  }
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    r[i].key = __brev(path[i]) >> (32 - depth);
+    if (TRACK) {
+      const uint32_t lvl = info[i] >> kQuadOrdinalBits;
+      r[i].vertex = ((1u << lvl) - 1u) + (path[i] >> (uint32_t(depth) - lvl));
+      r[i].ord = info[i] & kMask;
+      r[i].margin = best[i];
+    } else {
+      r[i].vertex = 0;
+      r[i].ord = 0;
+      r[i].margin = (root[i] != root[i]) ? root[i] : best[i];
+    }
   }
 }
 
@@ -367,6 +384,36 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
   const uint32_t TM = uint32_t(d.T) * uint32_t(d.M);
   MarginBits margin_bound;  // RECORD: bound on the |margin| this lane recorded
 
+  // Output phase, lane constants of burst slot q for `un` slots per burst and u vectors per sample: where the parked
+  // walk result of the vector's pair lies, the vector's column in the leaf table of the step's first tree, and its
+  // offset in the output from the step's first element.
+  auto burst_constants = [&](auto un_tag, int u_per_sample, FastDiv by_u, uint32_t *park, uint32_t *wcol,
+                             uint32_t *off) {
+#pragma unroll
+    for (int q = 0; q < decltype(un_tag)::value; ++q) {
+      const int u = lane + q * kWave;
+      const int jj = by_u.div(u);
+      const int e = (u - jj * u_per_sample) * GW;
+      const int tt = div_m.div(e), m = e - tt * d.M;
+      park[q] = uint32_t(jj * LDP + tt);
+      wcol[q] = uint32_t(tt) * uint32_t(d.L) * uint32_t(wpitch) + uint32_t(m);
+      off[q] = uint32_t(jj) * TM + uint32_t(e);
+    }
+  };
+  // ... prepared once for the complete steps of a complete tile
+  uint32_t full_park[kRowUnroll], full_wcol[kRowUnroll], full_off[kRowUnroll];
+  int full_un = 0;
+  {
+    const int u_full = TPW * d.M / GW, total_full = BT * u_full;
+    if (n_live == BT) {
+      if (total_full % (kWave * kRowUnroll) == 0 && (kWave * kRowUnroll) % u_full == 0) full_un = kRowUnroll;
+    }
+#pragma unroll
+    for (int q = 0; q < kRowUnroll; ++q) full_park[q] = full_wcol[q] = full_off[q] = 0;
+    if (full_un == kRowUnroll)
+      burst_constants(std::integral_constant<int, kRowUnroll>{}, u_full, div_u_full, full_park, full_wcol, full_off);
+  }
+
   for (int tb = t_begin + wave * TPW; tb < t_end; tb += kWaves * TPW) {
     // ---- walk: this lane's sample through trees tb + slot + i * SLOTS
     {
@@ -395,12 +442,12 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
           const QuadNode *top[kRowIlp];
 #pragma unroll
           for (int i = 0; i < kRowIlp; ++i) top[i] = stage + (slot + i * SLOTS) * kTopQuads;
-          walk_quads<kRowIlp, BT, true>(d.depth, qn, top, xs_j, r);
+          walk_quads<kRowIlp, BT, true, RECORD>(d.depth, qn, top, xs_j, r);
           // every lane has read its quads before any lane overwrites them with results
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
           __builtin_amdgcn_wave_barrier();
         } else {
-          walk_quads<kRowIlp, BT, false>(d.depth, qn, qn, xs_j, r);
+          walk_quads<kRowIlp, BT, false, RECORD>(d.depth, qn, qn, xs_j, r);
         }
       } else {
         const Node<Real> *all = static_cast<const Node<Real> *>(vertices);
@@ -460,34 +507,30 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
     const int total = n_live * U;
     Real *obase = out + ((long long)s0 * d.T + tb) * d.M;
     const Real *wbase = w + (long long)tb * d.L * wpitch;  // wpitch: elements between leaf rows (M, or padded)
-    constexpr int kBurst = kWave * kRowUnroll;  // vectors a wavefront handles per iteration
-    if (total % kBurst == 0 && kBurst % U == 0) {
-      // Whole bursts, and a burst is a whole number of samples: which tree and output a lane serves in slot q of a
-      // burst is the same in every burst, so the divisions are done once per step and a burst only advances the
-      // sample (complete tiles of the benchmark shapes: 32 samples x 8 trees x 10 outputs = 4 bursts of 8 samples).
-      uint32_t park[kRowUnroll], wcol[kRowUnroll], off[kRowUnroll];
+    // Whole bursts, and a burst is a whole number of samples: which tree and output a lane serves in slot q of a
+    // burst is the same in every burst, so the divisions are done once (complete tiles of the benchmark shapes: 32
+    // samples x 8 trees x 10 outputs = 4 bursts of 5 vectors per lane, 8 samples each) and a burst only advances the
+    // sample. For complete steps of a complete tile the lane constants were even prepared before the loop over the
+    // steps. (A four-vector burst for one output per leaf, whose step is 256 vectors, was measured slower than the
+    // general loop below: ferns 0.464 -> 0.485 ms.)
+    auto bursts = [&](auto un_tag, const uint32_t *park0, const uint32_t *wcol0, const uint32_t *off0) {
+      constexpr int UN = decltype(un_tag)::value;
+      constexpr int kBurst = kWave * UN;  // vectors a wavefront handles per iteration
+      uint32_t park[UN], wcol[UN], off[UN];
 #pragma unroll
-      for (int q = 0; q < kRowUnroll; ++q) {
-        const int u = lane + q * kWave;
-        const int jj = div_u.div(u);
-        const int e = (u - jj * U) * GW;
-        const int tt = div_m.div(e), m = e - tt * d.M;
-        park[q] = uint32_t(jj * LDP + tt);
-        wcol[q] = uint32_t(tt) * uint32_t(d.L) * uint32_t(wpitch) + uint32_t(m);
-        off[q] = uint32_t(jj) * TM + uint32_t(e);
-      }
+      for (int q = 0; q < UN; ++q) park[q] = park0[q], wcol[q] = wcol0[q], off[q] = off0[q];
       const uint32_t park_step = uint32_t(kBurst / U) * LDP, off_step = uint32_t(kBurst / U) * TM;
       for (int burst = 0; burst < total; burst += kBurst) {
-        Real a[kRowUnroll];
-        Vec wv[kRowUnroll];
+        Real a[UN];
+        Vec wv[UN];
 #pragma unroll
-        for (int q = 0; q < kRowUnroll; ++q) {
+        for (int q = 0; q < UN; ++q) {
           const uint32_t key = p_key[park[q]];
           a[q] = p_abs[park[q]];
           wv[q] = *reinterpret_cast<const Vec *>(wbase + key * uint32_t(wpitch) + wcol[q]);
         }
 #pragma unroll
-        for (int q = 0; q < kRowUnroll; ++q) {
+        for (int q = 0; q < UN; ++q) {
           Vec o;
 #pragma unroll
           for (int i = 0; i < GW; ++i) o[i] = a[q] * wv[q][i];
@@ -496,6 +539,13 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
           off[q] += off_step;
         }
       }
+    };
+    if (full_un != 0 && nt == TPW) {
+      bursts(std::integral_constant<int, kRowUnroll>{}, full_park, full_wcol, full_off);
+    } else if (total % (kWave * kRowUnroll) == 0 && (kWave * kRowUnroll) % U == 0) {
+      uint32_t park[kRowUnroll], wcol[kRowUnroll], off[kRowUnroll];
+      burst_constants(std::integral_constant<int, kRowUnroll>{}, U, div_u, park, wcol, off);
+      bursts(std::integral_constant<int, kRowUnroll>{}, park, wcol, off);
     } else {
       for (int u0 = lane; u0 < total; u0 += kWave * kRowUnroll) {
         Real a[kRowUnroll];
