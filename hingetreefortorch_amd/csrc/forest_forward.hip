@@ -336,6 +336,63 @@ __device__ __forceinline__ void walk_quads(int depth, const QuadNode *const (&qu
   }
 }
 
+// N interleaved fern walks whose vertices are staged in LDS level major: walk i's vertex of level l is
+// mine[l * TPW + i * STRIDE]. Like walk_quads the loop carries the path (decisions, most significant bit first), the
+// signed margin of the smallest |margin| so far (seeded by level 0, strict '<' afterwards: HingeTreeCommon.h:72-91) and
+// one word holding that level and its ordinal; TRACK = false carries |margin| alone. A fern's selected vertex is its
+// level.
+template <typename Real, int N, int BT, int STRIDE, int TPW, bool TRACK>
+__device__ __forceinline__ void walk_ferns_staged(int depth, const Node<Real> *mine, const Real *xs_j,
+                                                  WalkResult<Real> (&r)[N]) {
+  constexpr int kLevelShift = 24;  // ordinals index a tile in LDS: far below 2^24
+  uint32_t path[N], info[N];
+  Real best[N], root[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) path[i] = 0, info[i] = 0, best[i] = Real(0), root[i] = Real(0);
+  // (Issuing the reads of several levels together -- a fern's vertices do not depend on the path -- was measured and
+  // gained nothing: 0.470 against 0.471 ms for the fern benchmark's forward.)
+  auto level = [&](int lvl, auto first_tag) {
+    constexpr bool FIRST = decltype(first_tag)::value;
+    Node<Real> n[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) n[i] = mine[lvl * TPW + i * STRIDE];
+    Real m[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) m[i] = xs_j[int(n[i].ord) * BT] - n[i].thr;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      if (FIRST) {
+        root[i] = m[i];
+        best[i] = TRACK ? m[i] : ht_abs(m[i]);
+        info[i] = uint32_t(n[i].ord);
+      } else if (TRACK) {
+        const bool closer = ht_abs(m[i]) < ht_abs(best[i]);
+        best[i] = closer ? m[i] : best[i];
+        info[i] = closer ? (uint32_t(n[i].ord) | (uint32_t(lvl) << kLevelShift)) : info[i];
+      } else {
+        const Real a = ht_abs(m[i]);
+        best[i] = (a < best[i]) ? a : best[i];  // a NaN margin never wins; a NaN root is put back below
+      }
+      path[i] = path[i] + path[i] + ((m[i] > Real(0)) ? 1u : 0u);
+    }
+  };
+  level(0, std::true_type{});
+  for (int lvl = 1; lvl < depth; ++lvl) level(lvl, std::false_type{});
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    r[i].key = __brev(path[i]) >> (32 - depth);
+    if (TRACK) {
+      r[i].vertex = info[i] >> kLevelShift;
+      r[i].ord = info[i] & ((1u << kLevelShift) - 1u);
+      r[i].margin = best[i];
+    } else {
+      r[i].vertex = 0;
+      r[i].ord = 0;
+      r[i].margin = (root[i] != root[i]) ? root[i] : best[i];
+    }
+  }
+}
+
 constexpr int kRowIlp = 4;     // trees walked concurrently per lane
 constexpr int kRowUnroll = 5;  // output vectors per lane whose weight gathers are in flight together
 
@@ -460,16 +517,15 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
           Node<Real> *stage = reinterpret_cast<Node<Real> *>(p_abs);
           if (size_t(TPW) * d.depth * sizeof(Node<Real>) <= size_t(BT) * LDP * sizeof(Real)) {
             staged = true;
+            // level major, [level][fern]: the ferns of a lane's kRowIlp walks then lie a compile-time distance apart
             for (int i = lane; i < TPW * d.depth; i += kWave) {
-              const int tt = i / d.depth, lv = i - tt * d.depth;
+              const int lv = i / TPW, tt = i - lv * TPW;
               stage[i] = all[(long long)min(tb + tt, t_end - 1) * d.V + lv];
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            walk_many_fn<Real, true, kRowIlp>(
-                d.depth, [&](int i, uint32_t at) { return stage[(slot + i * SLOTS) * d.depth + at]; },
-                [&](int, int f) { return xs_j[f * BT]; }, r);
+            walk_ferns_staged<Real, kRowIlp, BT, SLOTS, TPW, RECORD>(d.depth, stage + slot, xs_j, r);
             // every lane has read its vertices before any lane overwrites them with results
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
