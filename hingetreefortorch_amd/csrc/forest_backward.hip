@@ -116,33 +116,71 @@ int dispatch_records(const ForestDims &d, const Real *x, const Node<Real> *nodes
 // which leaves >= 61 - ceil(log2(count)) bits below the largest term (an fp32 running sum keeps 24). Non-finite
 // bounds (inf / NaN in the inputs) cannot be represented: the header then routes the affected gradients to the
 // sequential owner-computes kernels further down, on the device, without a host round trip.
+//
+// Sampled bound (large upstream gradients on the lean tree kernel). A pass over the whole upstream gradient just for
+// max|g| costs half as much again as the tree kernel that follows it. So max|g| is taken over a fixed 1/64 sample
+// (whole 1 KB runs, their position inside each 64 KB advancing from run to run so that every column is met), the
+// scale is chosen kSampleGuard times more generous than that sample asks for (10 of the spare bits), and the tree
+// kernel, which sees every term anyway, keeps the largest |term| it accumulated. A check kernel then compares: if no
+// term exceeded what the scale allows, the sums are exact sums of correctly rounded terms and stand; otherwise (a
+// gradient with outliers more than kSampleGuard times the sample's largest value, or zero wherever it was sampled) the
+// scale is chosen again from the true largest term and the tree kernel runs a second time -- all decided on the device
+// and by the data alone, so the result stays bit reproducible.
 struct DetHeader {
   unsigned long long max_g, max_a, max_c;  // bit patterns of non-negative doubles (ordered like the values)
   double scale_w, inv_scale_w, scale_c, inv_scale_c;
   int fallback_w, fallback_c;
+  int redo_w;  // sampled bound exceeded: the second run of the tree kernel is wanted
 };
+constexpr double kSampleGuard = 1024.0;
+constexpr int kSampleEvery = 64;                       // one run in 64 is read
+constexpr size_t kSampleMinBytes = size_t(64) << 20;   // below that the full pass costs a few microseconds
 // The bound on |c| is taken by the tree kernels as they store c (one running maximum per lane, one atomic per
 // wavefront): the atomics go to kDetSlots slots behind the header, spread by workgroup, because thousands of atomics
 // on ONE address serialise in L2 for longer than a pass over c takes; the scale kernel folds the slots.
+// A second set of slots takes the largest |term| of dW the same way, a third the sample of max|g| (sampled bound).
 constexpr int kDetSlots = 4096;
-constexpr size_t kDetHeaderBytes = 256 + size_t(kDetSlots) * sizeof(unsigned long long);
+constexpr int kDetFoldThreads = 1024;
+constexpr size_t kDetHeaderBytes = 256 + 3 * size_t(kDetSlots) * sizeof(unsigned long long);
 __device__ __forceinline__ unsigned long long *det_slots(DetHeader *h) {
   return reinterpret_cast<unsigned long long *>(reinterpret_cast<unsigned char *>(h) + 256);
+}
+__device__ __forceinline__ unsigned long long *det_term_slots(DetHeader *h) { return det_slots(h) + kDetSlots; }
+__device__ __forceinline__ unsigned long long *det_g_slots(DetHeader *h) { return det_slots(h) + 2 * kDetSlots; }
+
+// Largest of n slots (bit patterns of non-negative doubles order like the values), by a workgroup of kDetFoldThreads
+// threads; every thread receives it.
+__device__ inline unsigned long long det_fold(const unsigned long long *slots, int n) {
+  __shared__ unsigned long long part[kDetFoldThreads / kWave];
+  unsigned long long m = 0ull;
+  for (int i = threadIdx.x; i < n; i += kDetFoldThreads) m = max(m, slots[i]);
+  for (int off = 32; off > 0; off >>= 1) m = max(m, (unsigned long long)__shfl_xor((long long)m, off, kWave));
+  __syncthreads();  // a previous fold's readers are done with part[]
+  if ((threadIdx.x & (kWave - 1)) == 0) part[threadIdx.x / kWave] = m;
+  __syncthreads();
+  m = 0ull;
+  for (int i = 0; i < kDetFoldThreads / kWave; ++i) m = max(m, part[i]);
+  return m;
 }
 
 __global__ __launch_bounds__(256) void det_init_kernel(DetHeader *h) {
   if (threadIdx.x == 0) {
     h->max_g = h->max_a = h->max_c = 0ull;
     h->scale_w = h->inv_scale_w = h->scale_c = h->inv_scale_c = 1.0;
-    h->fallback_w = h->fallback_c = 0;
+    h->fallback_w = h->fallback_c = h->redo_w = 0;
   }
-  for (int i = threadIdx.x; i < kDetSlots; i += 256) det_slots(h)[i] = 0ull;
+  for (int i = threadIdx.x; i < 3 * kDetSlots; i += 256) det_slots(h)[i] = 0ull;
 }
 
 // A lane's bound on |c| (bound_take, records.hpp) over the wavefront into the workgroup's slot.
 template <typename Real>
 __device__ __forceinline__ void publish_c_bound(Real m, const DetHeader *hdr) {
   bound_publish(double(m), det_slots(const_cast<DetHeader *>(hdr)),
+                (blockIdx.y * gridDim.x + blockIdx.x) % unsigned(kDetSlots));
+}
+// A lane's bound on the |term| it added to dW (MarginBits, records.hpp), likewise.
+__device__ __forceinline__ void publish_term_bound(MarginBits m, const DetHeader *hdr) {
+  bound_publish(margin_bound_value<float>(m.bits), det_term_slots(const_cast<DetHeader *>(hdr)),
                 (blockIdx.y * gridDim.x + blockIdx.x) % unsigned(kDetSlots));
 }
 
@@ -186,6 +224,40 @@ __global__ __launch_bounds__(kAbsmaxThreads) void absmax_kernel(const Real *__re
   }
 }
 
+// The same over a sample: of every kSampleEvery consecutive 1 KB runs (64 x 16 bytes, one load of a wavefront) one is
+// read, run k of the sample at position (37 k mod kSampleEvery) of its 64 KB, so that the sample meets every column of
+// any row length. p is 16-byte aligned.
+template <typename Real>
+__global__ __launch_bounds__(kAbsmaxThreads) void absmax_sample_kernel(const Real *__restrict__ p, long long runs,
+                                                                       unsigned long long *slots) {
+  constexpr int VEC = 16 / sizeof(Real);
+  typedef Real Vec __attribute__((ext_vector_type(VEC)));
+  const Vec *pv = reinterpret_cast<const Vec *>(p);
+  const int lane = threadIdx.x & (kWave - 1);
+  const long long wave = ((long long)blockIdx.x * kAbsmaxThreads + threadIdx.x) / kWave;
+  const long long waves = (long long)gridDim.x * (kAbsmaxThreads / kWave);
+  Real m = Real(0);
+  for (long long k = wave; k < runs; k += waves) {
+    const long long run = k * kSampleEvery + ((k * 37) & (kSampleEvery - 1));
+    const Vec v = pv[run * kWave + lane];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) bound_take(m, v[e]);
+  }
+  double md = double(m);
+  for (int off = 32; off > 0; off >>= 1) {
+    const double o = __shfl_xor(md, off, kWave);
+    if (!(o <= md)) md = o;
+  }
+  __shared__ double part[kAbsmaxThreads / kWave];
+  if (lane == 0) part[threadIdx.x / kWave] = md;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int i = 1; i < kAbsmaxThreads / kWave; ++i)
+      if (!(part[i] <= md)) md = part[i];
+    if (md > 0.0) atomicMax(slots + blockIdx.x % unsigned(kDetSlots), (unsigned long long)__double_as_longlong(md));
+  }
+}
+
 __device__ inline void det_pick_scale(double bound, double count, double *scale, double *inv, int *fallback) {
   if (!(bound < double(INFINITY))) {
     *fallback = 1;
@@ -208,27 +280,50 @@ __device__ inline void det_pick_scale(double bound, double count, double *scale,
   *inv = ldexp(1.0, -k);
 }
 
-__global__ __launch_bounds__(kWave) void det_scale_kernel(DetHeader *h, int which, double count, bool fold_slots,
-                                                          const unsigned long long *margin_slots) {
-  if (which == 0 && margin_slots) {
-    unsigned long long m = 0ull;
-    for (int i = threadIdx.x; i < kBoundSlots; i += kWave) m = max(m, margin_slots[i]);
-    for (int off = 32; off > 0; off >>= 1) m = max(m, (unsigned long long)__shfl_xor((long long)m, off, kWave));
-    if (threadIdx.x == 0) h->max_a = m;
+// which = 0: scale of dW from max|g| (measured by a full pass, or folded here from the sample's slots) x max|margin|
+// (folded from the slots that came with the records) x guard; which = 1: scale of dThr / dX from max|c| (folded from
+// the slots the tree kernel filled).
+__global__ __launch_bounds__(kDetFoldThreads) void det_scale_kernel(DetHeader *h, int which, double count,
+                                                                    bool fold_slots,
+                                                                    const unsigned long long *margin_slots,
+                                                                    double guard, bool sampled) {
+  if (which == 0) {
+    const unsigned long long a = margin_slots ? det_fold(margin_slots, kBoundSlots) : 0ull;
+    const unsigned long long g = sampled ? det_fold(det_g_slots(h), kDetSlots) : 0ull;
+    if (threadIdx.x == 0) {
+      if (margin_slots) h->max_a = a;
+      if (sampled) h->max_g = g;
+    }
   }
   if (which == 1 && fold_slots) {
-    // bit patterns of non-negative doubles order like the values
-    unsigned long long m = 0ull;
-    for (int i = threadIdx.x; i < kDetSlots; i += kWave) m = max(m, det_slots(h)[i]);
-    for (int off = 32; off > 0; off >>= 1) m = max(m, (unsigned long long)__shfl_xor((long long)m, off, kWave));
-    if (threadIdx.x == 0) h->max_c = m;
+    const unsigned long long c = det_fold(det_slots(h), kDetSlots);
+    if (threadIdx.x == 0) h->max_c = c;
   }
   if (threadIdx.x != 0) return;
   if (which == 0)
-    det_pick_scale(__longlong_as_double((long long)h->max_g) * __longlong_as_double((long long)h->max_a), count,
-                   &h->scale_w, &h->inv_scale_w, &h->fallback_w);
+    det_pick_scale(guard * __longlong_as_double((long long)h->max_g) * __longlong_as_double((long long)h->max_a),
+                   count, &h->scale_w, &h->inv_scale_w, &h->fallback_w);
   else
     det_pick_scale(__longlong_as_double((long long)h->max_c), count, &h->scale_c, &h->inv_scale_c, &h->fallback_c);
+}
+
+// Sampled bound: did every term the tree kernel accumulated stay inside what the scale of dW was chosen for? If not,
+// the scale is chosen again from the true largest term and the second run of the tree kernel is switched on (a
+// non-finite term routes dW to the sequential kernel instead, like a non-finite bound does).
+__global__ __launch_bounds__(kDetFoldThreads) void det_verify_kernel(DetHeader *h, double count, double guard) {
+  const unsigned long long m = det_fold(det_term_slots(h), kDetSlots);
+  if (threadIdx.x != 0 || h->fallback_w) return;
+  const double largest = __longlong_as_double((long long)m);
+  const double allowed = guard * __longlong_as_double((long long)h->max_g) * __longlong_as_double((long long)h->max_a);
+  if (largest <= allowed) return;
+  det_pick_scale(largest, count, &h->scale_w, &h->inv_scale_w, &h->fallback_w);
+  h->redo_w = h->fallback_w ? 0 : 1;
+}
+
+// Clears n 64-bit words if *flag is set.
+__global__ __launch_bounds__(256) void zero_if_kernel(unsigned long long *p, long long n, const int *flag) {
+  if (!*flag) return;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) p[i] = 0ull;
 }
 
 __device__ __forceinline__ unsigned long long to_fixed(double v, double scale) {
@@ -544,7 +639,8 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
                                                                    const DetHeader *hdr, int log2_tb,
                                                                    long long part_size, bool need_c, bool dw_atomic,
                                                                    int num_groups, float *dthr_fold,
-                                                                   uint32_t thr_lds_offset, uint32_t w_lds_offset) {
+                                                                   uint32_t thr_lds_offset, uint32_t w_lds_offset,
+                                                                   bool second_run) {
   static_assert(!WLDS || M == 1, "leaf weights are staged in LDS for single-output leaves only");
   typedef LeanSplit<M> Split;
   constexpr int P = Split::P, VE = Split::VE, ROUNDS = Split::ROUNDS, SHIFT = Split::SHIFT;
@@ -561,11 +657,13 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
   float *w_lds = reinterpret_cast<float *>(smem + w_lds_offset);  // WLDS: the group's leaf weights
   double scale = 1.0, inv_scale = 1.0;
   if (FIXED) {
+    if (second_run && !hdr->redo_w) return;  // the sampled bound held (see DetHeader)
     if (hdr->fallback_w) dw = nullptr;
     scale = hdr->scale_w;
     inv_scale = hdr->inv_scale_w;
     if (!dw && !need_c) return;
   }
+  MarginBits term_bound;  // FIXED: largest |term| this lane added to dW
   const int TB = 1 << log2_tb;
   const int group = xcd_tree_group(blockIdx.x, num_groups);
   if (group < 0) return;
@@ -692,6 +790,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
         for (int i = 0; i < ROUNDS; ++i) {
           if (i < Split::BASE || i < my_cnt) {
             const float term = ht_abs(st.mg[u]) * g[i];
+            if (FIXED) term_bound.take(term);
             if (FIXED)
               atomicAdd(reinterpret_cast<unsigned long long *>(cell) + i, to_fixed(double(term), scale));
             else
@@ -788,6 +887,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
             for (int i = 0; i < ROUNDS; ++i) {
               if (i < Split::BASE || i < my_cnt) {
                 const float term = ht_abs(mg_u) * g[i];
+                if (FIXED) term_bound.take(term);
                 if (FIXED)
                   atomicAdd(reinterpret_cast<unsigned long long *>(cell) + i, to_fixed(double(term), scale));
                 else
@@ -893,6 +993,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     compute(st, sblk, have, on, std::false_type{});
   }
   if (FIXED && need_c) publish_c_bound(c_bound, hdr);
+  if (FIXED && dw && !second_run) publish_term_bound(term_bound, hdr);
   if (dw || dthr_fold) __syncthreads();
   if (dthr_fold) {
     float *dst = dthr_fold + (long long)t0 * d.V;
@@ -1665,11 +1766,24 @@ static bool wide_rows_ok(const ForestDims &d, const TreePlan &p) {
   return d.M % 4 == 0 && P4 >= 4 && P4 <= kWave && (P4 & (P4 - 1)) == 0 && (long long)p.TB * d.L * d.M < (1ll << 31);
 }
 
+// Shapes of tree_lean_kernel (float, compact records): contiguous rows of 1 or 10 outputs, a power-of-two tree group,
+// 32-bit offsets inside a block and a group.
+static bool lean_tree_ok(const ForestDims &d, const TreePlan &p, int *log2_tb_out) {
+  int log2_tb = 0;
+  while ((1 << (log2_tb + 1)) <= p.TB) ++log2_tb;
+  if (log2_tb_out) *log2_tb_out = log2_tb;
+  return d.K == 1 && (1 << log2_tb) == p.TB && p.TB <= 16 && (long long)kWave * d.T * d.M < (1ll << 31) &&
+         (long long)p.TB * d.L * d.M < (1ll << 31) && (d.M == 10 || d.M == 1);
+}
+
 // gout_image: the upstream gradient is stored as the image of the tile geometry (only tree_wide_kernel reads it so).
+// second_run: the repeat of the lean kernel after a sampled bound was exceeded (see DetHeader); it does nothing
+// unless the header asks for it.
 template <typename Real, bool COMPACT, bool FIXED>
 int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, const Real *gout,
                        Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
-                       bool need_c, Real *dthr, bool *dthr_done, hipStream_t stream, const ImageStore *gout_image) {
+                       bool need_c, Real *dthr, bool *dthr_done, hipStream_t stream, const ImageStore *gout_image,
+                       bool second_run = false) {
   *dthr_done = false;
   if constexpr (std::is_same<Real, float>::value && COMPACT) {
     if (gout_image != nullptr &&
@@ -1681,12 +1795,8 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
       return fail(HT_ERR_RUNTIME, "Error: this shape cannot read the upstream gradient as an image.");
   }
   if constexpr (std::is_same<Real, float>::value && COMPACT) {
-    // the specialised kernel: contiguous rows, a power-of-two tree group, 32-bit offsets inside a block and a group
     int log2_tb = 0;
-    while ((1 << (log2_tb + 1)) <= p.TB) ++log2_tb;
-    const bool fits = d.K == 1 && (1 << log2_tb) == p.TB && p.TB <= 16 &&
-                      (long long)kWave * d.T * d.M < (1ll << 31) && (long long)p.TB * d.L * d.M < (1ll << 31);
-    if (fits && (d.M == 10 || d.M == 1)) {
+    if (lean_tree_ok(d, p, &log2_tb)) {
       // dThr rides along where its fp64 table fits behind the leaf accumulators (atomic mode: the fixed-point scale of
       // c is only known once every c exists)
       const size_t acc_lds = dw ? size_t(p.TB) * d.L * d.M * sizeof(double) : 0;
@@ -1709,15 +1819,15 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
       if (d.M == 10)
         hipLaunchKernelGGL((tree_lean_kernel<10, FIXED, false>), grid, dim3(kForestThreads), lds, stream, d, w, gout,
                            rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
-                           uint32_t(thr_off), uint32_t(w_off));
+                           uint32_t(thr_off), uint32_t(w_off), second_run);
       else if (stage_w)
         hipLaunchKernelGGL((tree_lean_kernel<1, FIXED, true>), grid, dim3(kForestThreads), lds, stream, d, w, gout,
                            rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
-                           uint32_t(thr_off), uint32_t(w_off));
+                           uint32_t(thr_off), uint32_t(w_off), second_run);
       else
         hipLaunchKernelGGL((tree_lean_kernel<1, FIXED, false>), grid, dim3(kForestThreads), lds, stream, d, w, gout,
                            rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
-                           uint32_t(thr_off), uint32_t(w_off));
+                           uint32_t(thr_off), uint32_t(w_off), second_run);
       HT_LAUNCH_CHECK("forest backward (trees)");
       return HT_OK;
     }
@@ -1851,6 +1961,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
 
   DetHeader *hdr = nullptr;
   unsigned long long *dw_fixed = nullptr, *dthr_fixed = nullptr;
+  bool sampled = false;  // the scale of dW rests on a sample of the upstream gradient (see DetHeader)
   if (FIXED) {
     const FixedLayout lay = fixed_layout(d, dthr != nullptr, dw != nullptr, kLean && d.K == 1);
     unsigned char *base = static_cast<unsigned char *>(fixed_ws);
@@ -1860,10 +1971,21 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
     hipLaunchKernelGGL(det_init_kernel, dim3(1), dim3(256), 0, stream, hdr);
     HT_LAUNCH_CHECK("forest backward (deterministic header)");
     if (dw) {
-      if ((rc = launch_absmax<Real>(gout, pairs * d.M, &hdr->max_g, stream)) != HT_OK) return rc;
+      sampled = kLean && lean_tree_ok(d, plan, nullptr) && reinterpret_cast<uintptr_t>(gout) % 16 == 0 &&
+                size_t(pairs) * d.M * sizeof(Real) >= kSampleMinBytes;
+      if (sampled) {
+        const long long runs = pairs * d.M / (16 / (long long)sizeof(Real)) / kWave / kSampleEvery;
+        long long blocks = (runs + kAbsmaxThreads / kWave - 1) / (kAbsmaxThreads / kWave);
+        if (blocks > 8 * kNumCUs) blocks = 8 * kNumCUs;
+        hipLaunchKernelGGL((absmax_sample_kernel<Real>), dim3((unsigned)blocks), dim3(kAbsmaxThreads), 0, stream, gout,
+                           runs, (unsigned long long *)(reinterpret_cast<unsigned char *>(hdr) + 256) + 2 * kDetSlots);
+        HT_LAUNCH_CHECK("forest backward (sampled magnitude bound)");
+      } else if ((rc = launch_absmax<Real>(gout, pairs * d.M, &hdr->max_g, stream)) != HT_OK) {
+        return rc;
+      }
       // (the bound on |margin| came with the records)
-      hipLaunchKernelGGL(det_scale_kernel, dim3(1), dim3(kWave), 0, stream, hdr, 0, double(d.S), false,
-                         (const unsigned long long *)rec.bound);
+      hipLaunchKernelGGL(det_scale_kernel, dim3(1), dim3(kDetFoldThreads), 0, stream, hdr, 0, double(d.S), false,
+                         (const unsigned long long *)rec.bound, sampled ? kSampleGuard : 1.0, sampled);
       HT_LAUNCH_CHECK("forest backward (dW scale)");
       if (plan.parts > 1 && (rc = zero_fill(dw_fixed, size_t(d.T) * d.L * d.M * 8, stream)) != HT_OK) return rc;
     }
@@ -1876,6 +1998,20 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
   if (rc != HT_OK) return rc;
 
   if (FIXED) {
+    if (dw && sampled) {
+      hipLaunchKernelGGL(det_verify_kernel, dim3(1), dim3(kDetFoldThreads), 0, stream, hdr, double(d.S), kSampleGuard);
+      HT_LAUNCH_CHECK("forest backward (dW bound check)");
+      if (plan.parts > 1) {
+        const long long n = (long long)d.T * d.L * d.M;
+        hipLaunchKernelGGL(zero_if_kernel, dim3((unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096)), dim3(256),
+                           0, stream, dw_fixed, n, (const int *)&hdr->redo_w);
+        HT_LAUNCH_CHECK("forest backward (dW second run, clear)");
+      }
+      bool ignored = false;
+      rc = launch_tree_kernel<Real, COMPACT, FIXED>(d, plan, w, gout, rec, dw, dw_fixed, hdr, false, (Real *)nullptr,
+                                                    &ignored, stream, gout_image, true);
+      if (rc != HT_OK) return rc;
+    }
     if (dw) {
       if (plan.parts > 1) {
         const long long n = (long long)d.T * d.L * d.M;
@@ -1899,8 +2035,8 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
     }
     if (need_c) {
       // the tree kernel left its bound on |c| in the header's slots
-      hipLaunchKernelGGL(det_scale_kernel, dim3(1), dim3(kWave), 0, stream, hdr, 1,
-                         double(d.S > d.T ? d.S : (long long)d.T), true, (const unsigned long long *)nullptr);
+      hipLaunchKernelGGL(det_scale_kernel, dim3(1), dim3(kDetFoldThreads), 0, stream, hdr, 1,
+                         double(d.S > d.T ? d.S : (long long)d.T), true, (const unsigned long long *)nullptr, 1.0, false);
       HT_LAUNCH_CHECK("forest backward (c scale)");
     }
   }
