@@ -105,3 +105,21 @@ def test_inf_outside_the_sample(dev):
     fin = torch.isfinite(rdthr)
     assert torch.equal(fin, torch.isfinite(dthr))
     assert rel_err(torch.where(fin, dthr, 0), torch.where(fin, rdthr, 0)) <= 1e-5
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+def test_float64_precision_at_a_large_batch(dev, fern):
+    """float64 data, 65 536 samples: the fixed-point cells keep 61 - 16 = 45 bits below the largest possible term, so
+    a cell's rounding error is at most 2^-46 of that term per sample -- 2^-30 of it if all 65 536 roundings of a cell
+    pointed the same way, about 2^-38 as a random walk. The serial float64 loop of the reference keeps 53 bits; the bar
+    here is therefore 1e-10 of the largest entry, not the 1e-12 of the small float64 cases."""
+    x, thr, ordn, w, gout = make_forest(65536, 8, [], 8, 3, [2], fern, torch.float64, seed=5)
+    ref = ho.backward(x, thr, ordn, w, gout, fern=fern)
+    gx, gthr, gord, gw, gg = [t.to(dev) for t in (x, thr, ordn, w, gout)]
+    fn = getattr(ops, ("fern_" if fern else "tree_") + "backward_deterministic")
+    runs = [fn(gx, True, gthr, True, gord, False, gw, True, gg) for _ in range(2)]
+    for a, b in zip(runs[0], runs[1]):
+        assert (a is None and b is None) or torch.equal(a, b)
+    dx, dthr, _, dw = runs[0]
+    for got, want in zip((dx, dthr, dw), ref):
+        assert rel_err(got.cpu(), want) <= 1e-10
