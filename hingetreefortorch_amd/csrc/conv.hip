@@ -553,7 +553,9 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
 // positions x C walks), which is what the second walk of the two-kernel form is traded for; workgroups start at
 // different out channels so that those atomics spread over all trees' addresses. NT = 512: the larger tile halves the
 // flushes and the tree staging per walk, and one workgroup fills a CU's wavefront slots the way two smaller ones do.
-template <typename Real, bool FERN, int NT>
+// M1: one output per leaf, known at compile time (no loop over outputs; the position's upstream gradient is loaded once
+// per out channel instead of once per walk).
+template <typename Real, bool FERN, int NT, bool M1>
 __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, ConvLds lay, int C, int Cout, int depth,
                                                                  int V, int L, int M, int j_per,
                                                                  const Real *__restrict__ x,
@@ -573,7 +575,13 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
   const long long b = blockIdx.z;
   int *special = reinterpret_cast<int *>(smem + lay.flag);
   const int LM = L * M;
-  load_conv_tile<Real>(tile, x, g, C, b, tyi, txi, special);
+  // single-output float trees walk by the sign bit where the data allow it (walk_paths_plain_tracked)
+  constexpr bool kLeanWalk = M1 && std::is_same<Real, float>::value;
+  if (kLeanWalk) {
+    if (threadIdx.x == 0) *special = 0;
+    __syncthreads();
+  }
+  load_conv_tile<Real, kLeanWalk>(tile, x, g, C, b, tyi, txi, special);
   for (int i = threadIdx.x; i < C * g.TSZ; i += NT) acc[i] = 0.0;
   for (int i = threadIdx.x; i < C * LM; i += NT) acc_w[i] = 0.0;
   for (int i = threadIdx.x; i < C * V; i += NT) acc_t[i] = 0.0;
@@ -611,10 +619,45 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
           }
         }
     }
-    stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
+    stage_conv_trees<Real, kLeanWalk>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
     __syncthreads();
     if (!live) continue;
     const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+    const Real g_one = M1 ? gp[0] : Real(0);
+    if constexpr (kLeanWalk) {
+      if (*special == 0) {
+        for (int c = 0; c < C; c += kConvIlp) {
+          TrackedPath st[kConvIlp];
+          const Node<float> *nd[kConvIlp];
+          const float *px[kConvIlp];
+          int ch[kConvIlp];
+#pragma unroll
+          for (int i = 0; i < kConvIlp; ++i) {
+            int ci = min(c + i, C - 1) + skew;
+            ci = ci >= C ? ci - C : ci;
+            ch[i] = ci;
+            nd[i] = nodes + ci * V - (FERN ? 0 : 1);  // trees: addressed by the 1-based heap index
+            px[i] = mine + ci * g.TSZ;
+          }
+          walk_paths_plain_tracked<FERN, kConvIlp>(
+              depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, st);
+#pragma unroll
+          for (int i = 0; i < kConvIlp; ++i) {
+            if (c + i >= C) break;
+            const float t = st[i].t;  // thr - x at the selected vertex: margin = -t
+            const int cell = ch[i] * L + int(st[i].key(depth));
+            if (dw) atomicAdd(acc_w + cell, double(ht_abs(t) * g_one));
+            // sign(margin) * (w * g): the product with the sign bit of t flipped in, zero where the margin is zero
+            const float wg = wl[cell] * g_one;
+            const float cs = t == 0.f ? 0.f
+                                      : __uint_as_float(__float_as_uint(wg) ^ (~__float_as_uint(t) & 0x80000000u));
+            if (dthr) atomicAdd(acc_t + ch[i] * V + int(st[i].template vertex<FERN>(depth)), -double(cs));
+            atomicAdd(acc + (px[i] - tile) + int(st[i].ordinal()), double(cs));
+          }
+        }
+        continue;
+      }
+    }
     for (int c = 0; c < C; c += kConvIlp) {
       WalkResult<Real> r[kConvIlp];
       const Node<Real> *nd[kConvIlp];
@@ -633,12 +676,17 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
       for (int i = 0; i < kConvIlp; ++i) {
         if (c + i >= C) break;
         const Real a = ht_abs(r[i].margin);
-        const int cell = (ch[i] * L + int(r[i].key)) * M;
+        const int cell = (ch[i] * L + int(r[i].key)) * (M1 ? 1 : M);
         Real cs = Real(0);
-        for (int m = 0; m < M; ++m) {
-          const Real gv = gp[m];
-          cs += wl[cell + m] * gv;
-          if (dw) atomicAdd(acc_w + cell + m, double(a * gv));
+        if (M1) {
+          cs += wl[cell] * g_one;
+          if (dw) atomicAdd(acc_w + cell, double(a * g_one));
+        } else {
+          for (int m = 0; m < M; ++m) {
+            const Real gv = gp[m];
+            cs += wl[cell + m] * gv;
+            if (dw) atomicAdd(acc_w + cell + m, double(a * gv));
+          }
         }
         cs = ht_sign(r[i].margin) * cs;
         if (dthr) atomicAdd(acc_t + ch[i] * V + int(r[i].vertex), -double(cs));
@@ -803,11 +851,18 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
     if (lay.total > kConvTiledLdsMax || tiles > 0x7fffffffLL) continue;
     const int j_per = conv_j_per(tiles * s.B, int(s.Cout));
     const dim3 grid((unsigned)tiles, (unsigned)((s.Cout + j_per - 1) / j_per), (unsigned)s.B);
-    auto kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvWideThreads>
-                       : conv_tiled_backward_kernel<Real, false, kConvWideThreads>;
+    auto kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvWideThreads, false>
+                       : conv_tiled_backward_kernel<Real, false, kConvWideThreads, false>;
     if (threads == kConvThreads)
-      kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvThreads>
-                    : conv_tiled_backward_kernel<Real, false, kConvThreads>;
+      kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvThreads, false>
+                    : conv_tiled_backward_kernel<Real, false, kConvThreads, false>;
+    if (s.M == 1) {
+      kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvWideThreads, true>
+                    : conv_tiled_backward_kernel<Real, false, kConvWideThreads, true>;
+      if (threads == kConvThreads)
+        kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvThreads, true>
+                      : conv_tiled_backward_kernel<Real, false, kConvThreads, true>;
+    }
     HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(lay.total)));
     hipLaunchKernelGGL(kernel, grid, dim3(threads), lay.total, stream, t, lay, int(s.C), int(s.Cout), int(s.depth), V,

@@ -102,21 +102,24 @@ __device__ __forceinline__ void walk_many(int depth, const Node<Real> *const (&n
 // instruction count is what matters). The decisions are collected most significant bit first in `path` -- which is
 // also the index of the current vertex inside its level, so the heap index needs no separate update -- and the leaf
 // key (decision of level i in bit i) is the bit reversal of the finished path. TRACK = false skips the selected
-// vertex / ordinal / signed margin (forward pass): r.margin then holds |margin|.
+// vertex / ordinal / signed margin (forward pass): r.margin then holds |margin|. TRACK = true carries the signed
+// margin of the selected vertex as the running minimum (compared by magnitude) and beside it ONE word, level << 26 |
+// ordinal (ordinals below 2^26, depth at most 32), from which the selected vertex is rebuilt once the path is
+// complete: two selects per level instead of four.
+constexpr int kPathLevelShift = 26;
 template <typename Real, bool FERN, bool TRACK, int N, typename NodeFn, typename FeatureFn>
 __device__ __forceinline__ void walk_paths(int depth, NodeFn node, FeatureFn feature, WalkResult<Real> (&r)[N]) {
-  uint32_t path[N];
-  Real best_abs[N];
+  uint32_t path[N], info[N];
+  Real best[N];  // TRACK: signed margin of the selected vertex; else its magnitude
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     path[i] = 0;
-    best_abs[i] = Real(0);
-    r[i].vertex = 0;
-    r[i].ord = 0;
-    r[i].margin = Real(0);
+    info[i] = 0;
+    best[i] = Real(0);
   }
   for (int lvl = 0; lvl < depth; ++lvl) {
     const uint32_t first = FERN ? uint32_t(lvl) : (1u << lvl) - 1u;  // wave uniform
+    const uint32_t lvl_tag = uint32_t(lvl) << kPathLevelShift;        // wave uniform
     Node<Real> n[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) n[i] = node(i, FERN ? first : first + path[i]);
@@ -125,14 +128,14 @@ __device__ __forceinline__ void walk_paths(int depth, NodeFn node, FeatureFn fea
     for (int i = 0; i < N; ++i) m[i] = feature(i, int(n[i].ord)) - n[i].thr;
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const Real a = ht_abs(m[i]);
-      if (lvl == 0 || a < best_abs[i]) {
-        best_abs[i] = a;
-        if (TRACK) {
-          r[i].margin = m[i];
-          r[i].vertex = FERN ? first : first + path[i];
-          r[i].ord = uint32_t(n[i].ord);
+      if (TRACK) {
+        if (lvl == 0 || ht_abs(m[i]) < ht_abs(best[i])) {
+          best[i] = m[i];
+          info[i] = lvl_tag | uint32_t(n[i].ord);
         }
+      } else {
+        const Real a = ht_abs(m[i]);
+        if (lvl == 0 || a < best[i]) best[i] = a;
       }
       path[i] = path[i] + path[i] + ((m[i] > Real(0)) ? 1u : 0u);
     }
@@ -140,7 +143,16 @@ __device__ __forceinline__ void walk_paths(int depth, NodeFn node, FeatureFn fea
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     r[i].key = __brev(path[i]) >> (32 - depth);
-    if (!TRACK) r[i].margin = best_abs[i];
+    r[i].margin = best[i];
+    if (TRACK) {
+      const uint32_t lvl = info[i] >> kPathLevelShift;
+      r[i].ord = info[i] & ((1u << kPathLevelShift) - 1u);
+      // the path's leading `lvl` bits are the index of the selected vertex inside its level
+      r[i].vertex = FERN ? lvl : ((1u << lvl) - 1u) + (lvl == 0 ? 0u : path[i] >> (uint32_t(depth) - lvl));
+    } else {
+      r[i].vertex = 0;
+      r[i].ord = 0;
+    }
   }
 }
 
@@ -198,6 +210,54 @@ __device__ __forceinline__ void walk_paths_plain(int depth, NodeFn node, Feature
       r[i].vertex = 0;
       r[i].ord = 0;
       r[i].margin = best_abs[i];
+    }
+  }
+}
+
+// walk_paths_plain for the backward pass, without the second read of the selected vertex: beside the path the walk
+// carries t = thr - x of the selected vertex (the signed margin is -t, its magnitude |t|) and one word, level << 26 |
+// ordinal (see walk_paths). The path is kept as a 1-based heap index (root = 1, child = 2 i + decision), so that
+// the address of the next vertex is one shift-add: for trees node(i, at) is called with that 1-based index (the
+// caller passes a table pointer moved back by one vertex), for ferns with the level. At the end heap = 2^depth + path:
+//   leaf key            brev(heap) >> (32 - depth)           (the marker bit falls off)
+//   selected vertex     (heap >> (depth - level)) - 1        (0-based heap index; ferns: the level itself)
+struct TrackedPath {
+  uint32_t heap;
+  float t;
+  uint32_t info;
+  __device__ __forceinline__ uint32_t key(int depth) const { return __brev(heap) >> (32 - depth); }
+  __device__ __forceinline__ uint32_t level() const { return info >> kPathLevelShift; }
+  __device__ __forceinline__ uint32_t ordinal() const { return info & ((1u << kPathLevelShift) - 1u); }
+  template <bool FERN>
+  __device__ __forceinline__ uint32_t vertex(int depth) const {
+    return FERN ? level() : (heap >> (uint32_t(depth) - level())) - 1u;
+  }
+};
+template <bool FERN, int N, typename NodeFn, typename FeatureFn>
+__device__ __forceinline__ void walk_paths_plain_tracked(int depth, NodeFn node, FeatureFn feature,
+                                                         TrackedPath (&r)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const Node<float> n = node(i, FERN ? 0u : 1u);
+    const float t = n.thr - feature(i, int(n.ord));
+    r[i].heap = __builtin_amdgcn_alignbit(1u, __float_as_uint(t), 31);  // 2 | sign(t)
+    r[i].t = t;
+    r[i].info = uint32_t(n.ord);
+  }
+  for (int lvl = 1; lvl < depth; ++lvl) {
+    const uint32_t lvl_tag = uint32_t(lvl) << kPathLevelShift;  // wave uniform
+    Node<float> n[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) n[i] = node(i, FERN ? uint32_t(lvl) : r[i].heap);
+    float t[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) t[i] = n[i].thr - feature(i, int(n[i].ord));
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const bool closer = ht_abs(t[i]) < ht_abs(r[i].t);
+      r[i].t = closer ? t[i] : r[i].t;
+      r[i].info = closer ? (lvl_tag | uint32_t(n[i].ord)) : r[i].info;
+      r[i].heap = __builtin_amdgcn_alignbit(r[i].heap, __float_as_uint(t[i]), 31);  // (heap << 1) | sign(t)
     }
   }
 }
