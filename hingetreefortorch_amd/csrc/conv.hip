@@ -237,12 +237,15 @@ static bool make_tile(const ConvGeom &g, ConvTile *t, int threads = kConvThreads
 
 // Cooperative load of the input region of tile (tyi, txi) of image b, all channels: a thread owns one or two cells of
 // the region and copies them channel by channel (the coordinate arithmetic is done once per cell, not per element).
+// c0 / count: the window of channels to load (all of them by default); plane c0 + k goes to tile plane k.
 template <typename Real, bool CHECK = false>
 __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restrict__ x, const ConvTile &g, int C,
-                                               long long b, int tyi, int txi, int *special) {
+                                               long long b, int tyi, int txi, int *special, int c0 = 0,
+                                               int count = -1) {
   const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
   const long long chan = (long long)g.H * g.W;
-  const Real *img = x + b * C * chan;
+  const Real *img = x + (b * C + c0) * chan;
+  if (count >= 0) C = count;
   for (int e = threadIdx.x; e < g.TSZ; e += int(blockDim.x)) {
     const int iy = e / g.IW, ix = e - iy * g.IW;
     const int gy = iy0 + iy, gx = ix0 + ix;
@@ -264,11 +267,14 @@ __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restric
 }
 
 // Trees (and optionally leaf weights) of out channel j into LDS.
+// c0 / count: the window of channels whose trees are staged (all of them by default).
 template <typename Real, bool CHECK = false>
 __device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, const ConvTile &g, int C, int V, int LM,
                                                  int j, const Real *__restrict__ thr, const int64_t *__restrict__ ord,
-                                                 const Real *__restrict__ w, int *special) {
-  const long long first = (long long)j * C * V;
+                                                 const Real *__restrict__ w, int *special, int c0 = 0, int count = -1) {
+  const long long tree0 = (long long)j * C + c0;
+  if (count >= 0) C = count;
+  const long long first = tree0 * V;
   for (int i = threadIdx.x; i < C * V; i += int(blockDim.x)) {
     const int tap = clamp_ordinal(ord[first + i], g.taps);
     const int ky = tap / g.kw, kx = tap - ky * g.kw;
@@ -279,7 +285,7 @@ __device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, co
     if (CHECK && !plain_threshold(n.thr)) *special = 1;
   }
   if (wl) {
-    const long long wfirst = (long long)j * C * LM;
+    const long long wfirst = tree0 * LM;
     for (int i = threadIdx.x; i < C * LM; i += int(blockDim.x)) wl[i] = w[wfirst + i];
   }
 }
@@ -548,16 +554,18 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
 }
 
 // All three gradients from ONE walk per (position, out channel, channel), for callers that want dX together with dThr
-// or dW: tile-stationary like the dX kernel, with the fp64 tables of the current out channel's C trees beside the dX
-// image. The tree tables are flushed to memory with atomics after each out channel (C * (V + L * M) cells per NT
+// or dW: tile-stationary like the dX kernel, with the fp64 tables of the current out channel's trees beside the dX
+// image. A workgroup serves a window of c_per channels (its tile planes, dX image and trees): with all 16 channels of
+// the benchmark shape one workgroup fills the LDS and a SIMD holds two wavefronts, with 8 it holds four, which hides
+// the chains of dependent LDS reads that a walk is (2.74 -> 2.47 ms). The tree tables are flushed to memory with atomics after each out channel (C * (V + L * M) cells per NT
 // positions x C walks), which is what the second walk of the two-kernel form is traded for; workgroups start at
 // different out channels so that those atomics spread over all trees' addresses. NT = 512: the larger tile halves the
 // flushes and the tree staging per walk, and one workgroup fills a CU's wavefront slots the way two smaller ones do.
 // M1: one output per leaf, known at compile time (no loop over outputs; the position's upstream gradient is loaded once
 // per out channel instead of once per walk).
 template <typename Real, bool FERN, int NT, bool M1>
-__global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, ConvLds lay, int C, int Cout, int depth,
-                                                                 int V, int L, int M, int j_per,
+__global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, ConvLds lay, int C_all, int c_per, int Cout,
+                                                                 int depth, int V, int L, int M, int j_per,
                                                                  const Real *__restrict__ x,
                                                                  const Real *__restrict__ thr,
                                                                  const int64_t *__restrict__ ord,
@@ -573,6 +581,11 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
   double *acc_t = reinterpret_cast<double *>(smem + lay.acc_t);
   const int tyi = blockIdx.x / g.tiles_x, txi = blockIdx.x - tyi * g.tiles_x;
   const long long b = blockIdx.z;
+  // blockIdx.y = (block of out channels, window of channels): a workgroup holds the tile planes, the dX image and the
+  // trees of c_per channels only, so that several workgroups fit a CU
+  const int c_blocks = (C_all + c_per - 1) / c_per;
+  const int c0 = int(blockIdx.y % unsigned(c_blocks)) * c_per, j_block = int(blockIdx.y / unsigned(c_blocks));
+  const int C = min(c_per, C_all - c0);
   int *special = reinterpret_cast<int *>(smem + lay.flag);
   const int LM = L * M;
   // single-output float trees walk by the sign bit where the data allow it (walk_paths_plain_tracked)
@@ -581,7 +594,7 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
     if (threadIdx.x == 0) *special = 0;
     __syncthreads();
   }
-  load_conv_tile<Real, kLeanWalk>(tile, x, g, C, b, tyi, txi, special);
+  load_conv_tile<Real, kLeanWalk>(tile, x, g, C_all, b, tyi, txi, special, c0, C);
   for (int i = threadIdx.x; i < C * g.TSZ; i += NT) acc[i] = 0.0;
   for (int i = threadIdx.x; i < C * LM; i += NT) acc_w[i] = 0.0;
   for (int i = threadIdx.x; i < C * V; i += NT) acc_t[i] = 0.0;
@@ -594,7 +607,7 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
   // min(C, 64) trees' tables and dX planes, so the atomics of one instruction rarely meet on one address.
   const int lane = int(threadIdx.x & 63u);
   const int skew = ((lane & 31) + (lane >> 5) * (C >> 1)) % C;
-  const int j_begin = blockIdx.y * j_per, j_count = min(Cout, j_begin + j_per) - j_begin;
+  const int j_begin = j_block * j_per, j_count = min(Cout, j_begin + j_per) - j_begin;
   const int rot = int((blockIdx.x * 7u + blockIdx.z * 13u) % unsigned(j_count));
   for (int jj = 0; jj < j_count; ++jj) {
     const int j = j_begin + (jj + rot >= j_count ? jj + rot - j_count : jj + rot);
@@ -606,7 +619,7 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
         for (int i = threadIdx.x; i < C * LM; i += NT) {
           const double v = acc_w[i];
           if (v != 0.0) {
-            atomicAdd(dw + (long long)jp * C * LM + i, Real(v));
+            atomicAdd(dw + ((long long)jp * C_all + c0) * LM + i, Real(v));
             acc_w[i] = 0.0;
           }
         }
@@ -614,12 +627,12 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
         for (int i = threadIdx.x; i < C * V; i += NT) {
           const double v = acc_t[i];
           if (v != 0.0) {
-            atomicAdd(dthr + (long long)jp * C * V + i, Real(v));
+            atomicAdd(dthr + ((long long)jp * C_all + c0) * V + i, Real(v));
             acc_t[i] = 0.0;
           }
         }
     }
-    stage_conv_trees<Real, kLeanWalk>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
+    stage_conv_trees<Real, kLeanWalk>(nodes, wl, g, C_all, V, LM, j, thr, ord, w, special, c0, C);
     __syncthreads();
     if (!live) continue;
     const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
@@ -699,10 +712,10 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
     const int jp = j_begin + (j_count - 1 + rot >= j_count ? rot - 1 : j_count - 1 + rot);
     if (dw)
       for (int i = threadIdx.x; i < C * LM; i += NT)
-        if (acc_w[i] != 0.0) atomicAdd(dw + (long long)jp * C * LM + i, Real(acc_w[i]));
+        if (acc_w[i] != 0.0) atomicAdd(dw + ((long long)jp * C_all + c0) * LM + i, Real(acc_w[i]));
     if (dthr)
       for (int i = threadIdx.x; i < C * V; i += NT)
-        if (acc_t[i] != 0.0) atomicAdd(dthr + (long long)jp * C * V + i, Real(acc_t[i]));
+        if (acc_t[i] != 0.0) atomicAdd(dthr + ((long long)jp * C_all + c0) * V + i, Real(acc_t[i]));
   }
   const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
   for (int i = threadIdx.x; i < C * g.TSZ; i += NT) {
@@ -711,7 +724,7 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
     const int c = i / g.TSZ, r = i - c * g.TSZ;
     const int iy = r / g.IW, ix = r - iy * g.IW;
     const int gy = iy0 + iy, gx = ix0 + ix;
-    if (gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) atomicAdd(dx + ((b * C + c) * g.H + gy) * (long long)g.W + gx, Real(v));
+    if (gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) atomicAdd(dx + ((b * C_all + c0 + c) * g.H + gy) * (long long)g.W + gx, Real(v));
   }
 }
 
@@ -846,11 +859,21 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
   for (int threads : {kConvWideThreads, kConvThreads}) {
     if (!(dx && (dthr || dw)) || !make_tile(g, &t, threads)) continue;
     const int LM = L * int(s.M);
-    const ConvLds lay = conv_lds_layout<Real>(t, int(s.C), V, LM, true, true, true);
+    // channels per workgroup: all of them if that leaves room for a second workgroup on the CU, else a half or a
+    // quarter (each window reads the tile's upstream gradient again, which is small beside the walks)
+    int c_per = int(s.C);
+    ConvLds lay = conv_lds_layout<Real>(t, c_per, V, LM, true, true, true);
+    while (lay.total > kConvTiledLdsMax / 2 && c_per >= 16) {  // (at least 8 channels: the lanes' skew spreads over them)
+      c_per = (c_per + 1) / 2;
+      lay = conv_lds_layout<Real>(t, c_per, V, LM, true, true, true);
+    }
     const long long tiles = (long long)t.tiles_y * t.tiles_x;
     if (lay.total > kConvTiledLdsMax || tiles > 0x7fffffffLL) continue;
-    const int j_per = conv_j_per(tiles * s.B, int(s.Cout));
-    const dim3 grid((unsigned)tiles, (unsigned)((s.Cout + j_per - 1) / j_per), (unsigned)s.B);
+    const int c_blocks = (int(s.C) + c_per - 1) / c_per;
+    const int j_per = conv_j_per(tiles * s.B * c_blocks, int(s.Cout));
+    const long long grid_y = (long long)((s.Cout + j_per - 1) / j_per) * c_blocks;
+    if (grid_y > 65535) continue;
+    const dim3 grid((unsigned)tiles, (unsigned)grid_y, (unsigned)s.B);
     auto kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvWideThreads, false>
                        : conv_tiled_backward_kernel<Real, false, kConvWideThreads, false>;
     if (threads == kConvThreads)
@@ -865,8 +888,8 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
     }
     HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(lay.total)));
-    hipLaunchKernelGGL(kernel, grid, dim3(threads), lay.total, stream, t, lay, int(s.C), int(s.Cout), int(s.depth), V,
-                       L, int(s.M), j_per, x, thr, ord, w, gout, dx, dthr, dw);
+    hipLaunchKernelGGL(kernel, grid, dim3(threads), lay.total, stream, t, lay, int(s.C), c_per, int(s.Cout),
+                       int(s.depth), V, L, int(s.M), j_per, x, thr, ord, w, gout, dx, dthr, dw);
     HT_LAUNCH_CHECK("conv backward (one walk, tiled)");
     return HT_OK;
   }

@@ -24,6 +24,8 @@ CASES = [
     (1, 1, 2, [30, 30], 12, [], [5, 5], [1, 1], [2, 2], [1, 1]),       # deep trees: accumulators leave LDS
     (1, 24, 3, [21, 40], 3, [], [3, 3], [1, 1], [1, 1], [1, 1]),       # many channels: the one-walk backward's narrow tile
     (2, 40, 2, [9, 33], 2, [], [3, 3], [1, 1], [1, 1], [1, 1]),        # more channels than any tile holds in LDS
+    (1, 19, 3, [21, 40], 5, [], [3, 3], [1, 1], [1, 1], [1, 1]),       # one-walk backward in two uneven channel windows
+    (2, 35, 2, [18, 33], 4, [2], [3, 3], [1, 1], [1, 1], [1, 1]),      # ... in several, more than one output per leaf
 ]
 
 
