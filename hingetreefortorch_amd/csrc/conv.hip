@@ -321,12 +321,26 @@ static ConvLds conv_lds_layout(const ConvTile &t, int C, int V, int LM, bool dx_
 template <typename Real, bool FERN, bool TRACK>
 __device__ __forceinline__ void conv_walks(bool plain, int depth, const Node<Real> *const (&nd)[kConvIlp],
                                            const Real *const (&px)[kConvIlp], WalkResult<Real> (&r)[kConvIlp]) {
-  // (the backward kernels are bound by LDS traffic, and the short form reads the selected vertex a second time:
-  // measured slower there, so they keep the general walk)
-  if constexpr (std::is_same<Real, float>::value && !TRACK) {
+  if constexpr (std::is_same<Real, float>::value) {
     if (plain) {
-      walk_paths_plain<FERN, TRACK, kConvIlp>(
-          depth, [&](int i, uint32_t at) { return nd[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
+      const Node<float> *nd1[kConvIlp];  // trees: addressed by the 1-based heap index
+#pragma unroll
+      for (int i = 0; i < kConvIlp; ++i) nd1[i] = nd[i] - (FERN ? 0 : 1);
+      if constexpr (TRACK) {
+        TrackedPath st[kConvIlp];
+        walk_paths_plain_tracked<FERN, kConvIlp>(
+            depth, [&](int i, uint32_t at) { return nd1[i][at]; }, [&](int i, int off) { return px[i][off]; }, st);
+#pragma unroll
+        for (int i = 0; i < kConvIlp; ++i) {
+          r[i].key = st[i].key(depth);
+          r[i].vertex = st[i].template vertex<FERN>(depth);
+          r[i].ord = st[i].ordinal();
+          r[i].margin = 0.f - st[i].t;  // x - thr, exactly; +0.0 where they are equal
+        }
+      } else {
+        walk_paths_plain<FERN, kConvIlp>(
+            depth, [&](int i, uint32_t at) { return nd1[i][at]; }, [&](int i, int off) { return px[i][off]; }, r);
+      }
       return;
     }
   }
@@ -422,7 +436,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_dx_kernel(ConvTile g,
   int *special = reinterpret_cast<int *>(smem + lay.flag);
   if (threadIdx.x == 0) *special = 0;
   __syncthreads();
-  load_conv_tile<Real>(tile, x, g, C, b, tyi, txi, special);
+  load_conv_tile<Real, true>(tile, x, g, C, b, tyi, txi, special);
   for (int i = threadIdx.x; i < C * g.TSZ; i += kConvThreads) acc[i] = 0.0;
   const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
   const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
@@ -433,7 +447,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_dx_kernel(ConvTile g,
   const int j_begin = blockIdx.y * j_per, j_end = min(Cout, j_begin + j_per);
   for (int j = j_begin; j < j_end; ++j) {
     __syncthreads();
-    stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
+    stage_conv_trees<Real, true>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
     __syncthreads();
     if (!live) continue;
     const bool plain = *special == 0;
@@ -494,7 +508,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
   int *special = reinterpret_cast<int *>(smem + lay.flag);
   if (threadIdx.x == 0) *special = 0;
   __syncthreads();
-  stage_conv_trees<Real>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
+  stage_conv_trees<Real, true>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
   for (int i = threadIdx.x; i < C * LM; i += kConvThreads) acc_w[i] = 0.0;
   for (int i = threadIdx.x; i < C * V; i += kConvThreads) acc_t[i] = 0.0;
   const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
@@ -506,7 +520,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
     const int t = int(it - b * tiles);
     const int tyi = t / g.tiles_x, txi = t - tyi * g.tiles_x;
     __syncthreads();  // the previous tile is no longer read (first pass: the staged trees are complete)
-    load_conv_tile<Real>(tile, x, g, C, b, tyi, txi, special);
+    load_conv_tile<Real, true>(tile, x, g, C, b, tyi, txi, special);
     __syncthreads();
     const bool plain = *special == 0;
     const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;

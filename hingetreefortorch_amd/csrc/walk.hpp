@@ -156,69 +156,52 @@ __device__ __forceinline__ void walk_paths(int depth, NodeFn node, FeatureFn fea
   }
 }
 
-// walk_paths for float data known to be "plain": every feature and threshold finite and no threshold equal to -0.0.
-// Then t = thr - x carries everything the walk needs -- |t| is |margin| and the sign bit of t is the decision
-// (x > thr  <=>  t < 0; t is +0.0 whenever x == thr, and never NaN) -- so a level costs one subtraction, one funnel
-// shift that appends the sign bit to the path, and the minimum tracking. With TRACK only the level of the smallest
-// |margin| is carried through the loop (first level wins ties, as in the reference); its vertex is rebuilt from the
-// finished path and read once more for the signed margin and the ordinal.
-template <bool FERN, bool TRACK, int N, typename NodeFn, typename FeatureFn>
+// walk_paths for the forward pass over float data known to be "plain": every feature and threshold finite and no
+// threshold equal to -0.0. Then t = thr - x carries everything the walk needs -- |t| is |margin| and the sign bit of t
+// is the decision (x > thr  <=>  t < 0; t is +0.0 whenever x == thr, and never NaN) -- so a level costs one
+// subtraction, one funnel shift that appends the sign bit to the path, and one minimum. The path is kept as a 1-based
+// heap index (root = 1, child = 2 i + decision), so that the address of the next vertex is one shift-add: for trees
+// node(i, at) is called with that 1-based index (the caller passes a table pointer moved back by one vertex), for
+// ferns with the level. At the end heap = 2^depth + path and the leaf key is brev(heap) >> (32 - depth): the marker
+// bit falls off. r.margin holds |margin|.
+template <bool FERN, int N, typename NodeFn, typename FeatureFn>
 __device__ __forceinline__ void walk_paths_plain(int depth, NodeFn node, FeatureFn feature, WalkResult<float> (&r)[N]) {
-  uint32_t path[N];
+  uint32_t heap[N];
   float best_abs[N];
-  uint32_t best_lvl[N];
 #pragma unroll
   for (int i = 0; i < N; ++i) {
-    const Node<float> n = node(i, 0u);
+    const Node<float> n = node(i, FERN ? 0u : 1u);
     const float t = n.thr - feature(i, int(n.ord));
-    path[i] = __float_as_uint(t) >> 31;
+    heap[i] = __builtin_amdgcn_alignbit(1u, __float_as_uint(t), 31);  // 2 | sign(t)
     best_abs[i] = ht_abs(t);
-    best_lvl[i] = 0;
   }
   for (int lvl = 1; lvl < depth; ++lvl) {
-    const uint32_t first = FERN ? uint32_t(lvl) : (1u << lvl) - 1u;  // wave uniform
     Node<float> n[N];
 #pragma unroll
-    for (int i = 0; i < N; ++i) n[i] = node(i, FERN ? first : first + path[i]);
+    for (int i = 0; i < N; ++i) n[i] = node(i, FERN ? uint32_t(lvl) : heap[i]);
     float t[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) t[i] = n[i].thr - feature(i, int(n[i].ord));
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const float a = ht_abs(t[i]);
-      if (TRACK) {
-        const bool closer = a < best_abs[i];
-        best_abs[i] = closer ? a : best_abs[i];
-        best_lvl[i] = closer ? uint32_t(lvl) : best_lvl[i];
-      } else {
-        best_abs[i] = __builtin_fminf(best_abs[i], a);
-      }
-      path[i] = __builtin_amdgcn_alignbit(path[i], __float_as_uint(t[i]), 31);  // (path << 1) | sign(t)
+      // min of two non-negative, never-NaN values as the median with zero: one instruction, where fminf would first
+      // quiet its operands
+      best_abs[i] = __builtin_amdgcn_fmed3f(best_abs[i], ht_abs(t[i]), 0.f);
+      heap[i] = __builtin_amdgcn_alignbit(heap[i], __float_as_uint(t[i]), 31);  // (heap << 1) | sign(t)
     }
   }
 #pragma unroll
   for (int i = 0; i < N; ++i) {
-    r[i].key = __brev(path[i]) >> (32 - depth);
-    if (TRACK) {
-      const uint32_t lvl = best_lvl[i];
-      const uint32_t vertex = FERN ? lvl : ((1u << lvl) - 1u) + (path[i] >> (uint32_t(depth) - lvl));
-      const Node<float> n = node(i, vertex);
-      r[i].vertex = vertex;
-      r[i].ord = uint32_t(n.ord);
-      r[i].margin = feature(i, int(n.ord)) - n.thr;
-    } else {
-      r[i].vertex = 0;
-      r[i].ord = 0;
-      r[i].margin = best_abs[i];
-    }
+    r[i].key = __brev(heap[i]) >> (32 - depth);
+    r[i].vertex = 0;
+    r[i].ord = 0;
+    r[i].margin = best_abs[i];
   }
 }
 
-// walk_paths_plain for the backward pass, without the second read of the selected vertex: beside the path the walk
-// carries t = thr - x of the selected vertex (the signed margin is -t, its magnitude |t|) and one word, level << 26 |
-// ordinal (see walk_paths). The path is kept as a 1-based heap index (root = 1, child = 2 i + decision), so that
-// the address of the next vertex is one shift-add: for trees node(i, at) is called with that 1-based index (the
-// caller passes a table pointer moved back by one vertex), for ferns with the level. At the end heap = 2^depth + path:
+// walk_paths_plain for the backward pass: beside the path the walk carries t = thr - x of the selected vertex (the
+// signed margin is -t, its magnitude |t|) and one word, level << 26 | ordinal (see walk_paths). Same 1-based heap
+// index and the same contract for node(i, at) as walk_paths_plain. At the end heap = 2^depth + path:
 //   leaf key            brev(heap) >> (32 - depth)           (the marker bit falls off)
 //   selected vertex     (heap >> (depth - level)) - 1        (0-based heap index; ferns: the level itself)
 struct TrackedPath {

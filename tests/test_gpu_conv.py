@@ -121,3 +121,8 @@ def test_conv_special_values(dev, special, fern):
     rdx, rdthr, rdw = ho.conv_backward(x, thr, ordn, w, gout, *args, fern=fern)
     dx, dthr, _, dw = getattr(ops, pre + "backward")(d[0], True, d[1], True, d[2], False, d[3], True, gout.to(dev), *args)
     assert rel_err(dx.cpu(), rdx) <= 1e-5 and rel_err(dthr.cpu(), rdthr) <= 1e-5 and rel_err(dw.cpu(), rdw) <= 1e-5
+    # the single-purpose kernels (dX alone; the tree gradients alone) choose between the two walks as well
+    dx, _, _, _ = getattr(ops, pre + "backward")(d[0], True, d[1], False, d[2], False, d[3], False, gout.to(dev), *args)
+    assert rel_err(dx.cpu(), rdx) <= 1e-5
+    _, dthr, _, dw = getattr(ops, pre + "backward")(d[0], False, d[1], True, d[2], False, d[3], True, gout.to(dev), *args)
+    assert rel_err(dthr.cpu(), rdthr) <= 1e-5 and rel_err(dw.cpu(), rdw) <= 1e-5
