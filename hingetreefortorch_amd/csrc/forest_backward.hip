@@ -664,6 +664,16 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
     if (!dw && !need_c) return;
   }
   MarginBits term_bound;  // FIXED: largest |term| this lane added to dW
+  // A leaf's accumulators are M cells of 8 bytes. One atomic instruction touches the same element of different
+  // leaves, so with M = 2^Z * odd its cells would fall on 32 / 2^Z of the LDS's 32 bank pairs only. The low Z bits of
+  // a cell's index inside its row are therefore XORed with Z bits of the leaf key (bits that do not enter M * key
+  // mod 32), which spreads them over all pairs; rows begin at multiples of 2^Z, so a cell stays inside its row. The
+  // swizzle of a pair travels in the upper half of its `rel` word (offsets inside a group's table stay below 2^16
+  // whenever the table exists).
+  constexpr int Z = (M % 2) ? 0 : ((M % 4) ? 1 : ((M % 8) ? 2 : ((M % 16) ? 3 : 4)));
+  constexpr uint32_t kSwizzleMask = (1u << Z) - 1u;
+  auto swizzle_of = [&](uint32_t key) -> uint32_t { return Z == 0 ? 0u : (key >> (5 - Z)) & kSwizzleMask; };
+  auto pack_rel = [&](uint32_t r, uint32_t key) -> uint32_t { return (Z != 0 && dw) ? (r | (swizzle_of(key) << 16)) : r; };
   const int TB = 1 << log2_tb;
   const int group = xcd_tree_group(blockIdx.x, num_groups);
   if (group < 0) return;
@@ -766,12 +776,13 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
       constexpr int u = decltype(u_tag)::value;
       const uint32_t key = uint32_t(group_bcast<P, u>(int(st.a_r))) & key_mask;
       st.mg[u] = __int_as_float(group_bcast<P, u>(__float_as_int(st.mg_r)));
-      st.rel[u] = woff + key * M;
+      const uint32_t r = woff + key * M;
+      st.rel[u] = pack_rel(r, key);
       if (need_c) {
         if constexpr (WLDS) {
-          st.wv[u] = Float4U{w_lds[on[u] ? st.rel[u] : 0u], 0.f, 0.f, 0.f};
+          st.wv[u] = Float4U{w_lds[on[u] ? r : 0u], 0.f, 0.f, 0.f};
         } else {
-          st.wv[u] = load_chunk(wbase + (on[u] ? st.rel[u] : uint32_t(e0)), false);
+          st.wv[u] = load_chunk(wbase + (on[u] ? r : uint32_t(e0)), false);
         }
       }
     });
@@ -785,16 +796,17 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
       float g[ROUNDS];
       own_elements(st.gv[u], g);
       if (dw && (FULL || on[u])) {
-        Acc *cell = acc + (st.rel[u] - e0 + my_begin);
+        const uint32_t row = (Z != 0 ? (st.rel[u] & 0xFFFFu) : st.rel[u]) - e0, swz = Z != 0 ? st.rel[u] >> 16 : 0u;
 #pragma unroll
         for (int i = 0; i < ROUNDS; ++i) {
           if (i < Split::BASE || i < my_cnt) {
             const float term = ht_abs(st.mg[u]) * g[i];
+            Acc *cell = acc + (row + ((uint32_t(my_begin) + i) ^ swz));
             if (FIXED) term_bound.take(term);
             if (FIXED)
-              atomicAdd(reinterpret_cast<unsigned long long *>(cell) + i, to_fixed(double(term), scale));
+              atomicAdd(reinterpret_cast<unsigned long long *>(cell), to_fixed(double(term), scale));
             else
-              atomicAdd(reinterpret_cast<double *>(cell) + i, double(term));
+              atomicAdd(reinterpret_cast<double *>(cell), double(term));
           }
         }
       }
@@ -862,12 +874,13 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
         static_for<P>([&](auto u_tag) {
           constexpr int u = decltype(u_tag)::value;
           const uint32_t key = uint32_t(group_bcast<P, u>(int(a_k))) & key_mask;
-          ld.rel[u] = woff + key * M;
+          const uint32_t r = woff + key * M;
+          ld.rel[u] = pack_rel(r, key);
           if (need_c) {
             if constexpr (WLDS) {
-              ld.wv[u] = Float4U{w_lds[ld.rel[u]], 0.f, 0.f, 0.f};
+              ld.wv[u] = Float4U{w_lds[r], 0.f, 0.f, 0.f};
             } else {
-              ld.wv[u] = load_chunk(wbase + ld.rel[u], false);
+              ld.wv[u] = load_chunk(wbase + r, false);
             }
           }
         });
@@ -882,16 +895,17 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
           float g[ROUNDS];
           own_elements(ld.gv[u], g);
           if (dw) {
-            Acc *cell = acc + (ld.rel[u] - e0 + my_begin);
+            const uint32_t row = (Z != 0 ? (ld.rel[u] & 0xFFFFu) : ld.rel[u]) - e0, swz = Z != 0 ? ld.rel[u] >> 16 : 0u;
 #pragma unroll
             for (int i = 0; i < ROUNDS; ++i) {
               if (i < Split::BASE || i < my_cnt) {
                 const float term = ht_abs(mg_u) * g[i];
+                Acc *cell = acc + (row + ((uint32_t(my_begin) + i) ^ swz));
                 if (FIXED) term_bound.take(term);
                 if (FIXED)
-                  atomicAdd(reinterpret_cast<unsigned long long *>(cell) + i, to_fixed(double(term), scale));
+                  atomicAdd(reinterpret_cast<unsigned long long *>(cell), to_fixed(double(term), scale));
                 else
-                  atomicAdd(reinterpret_cast<double *>(cell) + i, double(term));
+                  atomicAdd(reinterpret_cast<double *>(cell), double(term));
               }
             }
           }
@@ -1009,21 +1023,31 @@ __global__ __launch_bounds__(kForestThreads) void tree_lean_kernel(ForestDims d,
   if (dw) {
     float *dst = dw + (long long)t0 * LM;
     const uint32_t n = uint32_t(nt) * LM;
+    // element i of the table sits in cell at(i) (see the swizzle above)
+    auto at = [&](uint32_t i) -> uint32_t {
+      if (Z == 0) return i;
+      const uint32_t row = i / uint32_t(M), m = i - row * uint32_t(M);
+      return i - m + (m ^ swizzle_of(row & uint32_t(d.L - 1)));
+    };
     if (FIXED) {
       const unsigned long long *q = reinterpret_cast<const unsigned long long *>(acc);
       if (dw_atomic) {
-        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads)
-          if (q[i] != 0ull) atomicAdd(dw_fixed + (long long)t0 * LM + i, q[i]);
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) {
+          const unsigned long long v = q[at(i)];
+          if (v != 0ull) atomicAdd(dw_fixed + (long long)t0 * LM + i, v);
+        }
       } else {
-        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = from_fixed<float>(q[i], inv_scale);
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = from_fixed<float>(q[at(i)], inv_scale);
       }
     } else {
       const double *q = reinterpret_cast<const double *>(acc);
       if (dw_atomic) {
-        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads)
-          if (q[i] != 0.0) atomicAdd(dst + i, float(q[i]));
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) {
+          const double v = q[at(i)];
+          if (v != 0.0) atomicAdd(dst + i, float(v));
+        }
       } else {
-        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = float(q[i]);
+        for (uint32_t i = threadIdx.x; i < n; i += kForestThreads) dst[i] = float(q[at(i)]);
       }
     }
   }
@@ -1670,6 +1694,7 @@ __global__ __launch_bounds__(kWave) void det_tree_kernel(ForestDims d, const Rea
 // ---------------------------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------------------------
+constexpr int kLeanMaxOutputs = 16;  // tree_lean_kernel: at most four lanes of four values per pair
 struct TreePlan {
   int TB;               // trees per workgroup
   int groups, parts;    // grid
@@ -1692,19 +1717,22 @@ static bool plan_trees(const ForestDims &d, bool need_dw, bool lean, TreePlan *p
     tb = int(size_t(kLdsBytes) / per_tree);
   }
   if (w_tree != 0) {
-    // room for the staged weights and the vertex table of the group as well; the lean kernel wants a power of two
+    // room for the staged weights and the vertex table of the group as well
     const size_t all = (need_dw ? per_tree : 0) + w_tree + size_t(d.V) * sizeof(double);
     int fit = int(size_t(kLdsBytes - 64) / all);
     if (fit < 1) fit = 1;
     if (tb > fit) tb = fit;
-    while (tb & (tb - 1)) tb &= tb - 1;
   }
   if (tb > kMaxGroupTrees) tb = kMaxGroupTrees;
   if (tb > d.T) tb = d.T;
-  // Keep at least ~one workgroup per CU by shrinking the groups before splitting the samples -- except for
-  // single-output leaves, where a group reads only 4 * TB bytes of every 128-byte line of upstream gradients it
+  // the lean kernel (see lean_tree_ok) wants a power of two
+  const bool pow2 = lean && d.M <= kLeanMaxOutputs;
+  if (pow2)
+    while (tb & (tb - 1)) tb &= tb - 1;
+  // Keep at least ~one workgroup per CU by shrinking the groups before splitting the samples -- except for leaves
+  // with few outputs, where a group reads only 4 * M * TB bytes of every 128-byte line of upstream gradients it
   // requests: there wide groups matter more, and the samples are split instead.
-  const bool keep = w_tree != 0;
+  const bool keep = w_tree != 0 || (pow2 && d.M <= 4);
   while (!keep && tb > 4 && (d.T + tb - 1) / tb < kNumCUs) tb = (tb + 1) / 2;
   p->TB = tb;
   p->groups = (d.T + tb - 1) / tb;
@@ -1766,14 +1794,14 @@ static bool wide_rows_ok(const ForestDims &d, const TreePlan &p) {
   return d.M % 4 == 0 && P4 >= 4 && P4 <= kWave && (P4 & (P4 - 1)) == 0 && (long long)p.TB * d.L * d.M < (1ll << 31);
 }
 
-// Shapes of tree_lean_kernel (float, compact records): contiguous rows of 1 or 10 outputs, a power-of-two tree group,
+// Shapes of tree_lean_kernel (float, compact records): contiguous rows of up to 16 outputs, a power-of-two tree group,
 // 32-bit offsets inside a block and a group.
 static bool lean_tree_ok(const ForestDims &d, const TreePlan &p, int *log2_tb_out) {
   int log2_tb = 0;
   while ((1 << (log2_tb + 1)) <= p.TB) ++log2_tb;
   if (log2_tb_out) *log2_tb_out = log2_tb;
   return d.K == 1 && (1 << log2_tb) == p.TB && p.TB <= 16 && (long long)kWave * d.T * d.M < (1ll << 31) &&
-         (long long)p.TB * d.L * d.M < (1ll << 31) && (d.M == 10 || d.M == 1);
+         (long long)p.TB * d.L * d.M < (1ll << 31) && d.M >= 1 && d.M <= kLeanMaxOutputs;
 }
 
 // gout_image: the upstream gradient is stored as the image of the tile geometry (only tree_wide_kernel reads it so).
@@ -1810,24 +1838,28 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
       if (lds < p.lds) lds = p.lds;
       float *dthr_fold = fold ? dthr : nullptr;
       *dthr_done = fold;
-      const void *fn = d.M == 10 ? (const void *)tree_lean_kernel<10, FIXED, false>
-                                 : (stage_w ? (const void *)tree_lean_kernel<1, FIXED, true>
-                                            : (const void *)tree_lean_kernel<1, FIXED, false>);
-      HT_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
       const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
       const dim3 grid((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts);
-      if (d.M == 10)
-        hipLaunchKernelGGL((tree_lean_kernel<10, FIXED, false>), grid, dim3(kForestThreads), lds, stream, d, w, gout,
-                           rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
-                           uint32_t(thr_off), uint32_t(w_off), second_run);
-      else if (stage_w)
-        hipLaunchKernelGGL((tree_lean_kernel<1, FIXED, true>), grid, dim3(kForestThreads), lds, stream, d, w, gout,
-                           rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
-                           uint32_t(thr_off), uint32_t(w_off), second_run);
-      else
-        hipLaunchKernelGGL((tree_lean_kernel<1, FIXED, false>), grid, dim3(kForestThreads), lds, stream, d, w, gout,
-                           rec, dw, dw_fixed, hdr, log2_tb, p.part_size, need_c, p.parts > 1, p.groups, dthr_fold,
-                           uint32_t(thr_off), uint32_t(w_off), second_run);
+#define HT_LEAN_LAUNCH(MM, WLDS_)                                                                                     \
+  {                                                                                                                   \
+    auto kernel = tree_lean_kernel<MM, FIXED, WLDS_>;                                                                 \
+    HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                                          \
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));                          \
+    hipLaunchKernelGGL(kernel, grid, dim3(kForestThreads), lds, stream, d, w, gout, rec, dw, dw_fixed, hdr, log2_tb,  \
+                       p.part_size, need_c, p.parts > 1, p.groups, dthr_fold, uint32_t(thr_off), uint32_t(w_off),     \
+                       second_run);                                                                                   \
+  }
+#define HT_LEAN(MM) \
+  case MM: HT_LEAN_LAUNCH(MM, false) break;
+      switch (d.M) {
+        case 1:
+          if (stage_w) HT_LEAN_LAUNCH(1, true) else HT_LEAN_LAUNCH(1, false)
+          break;
+        HT_LEAN(2) HT_LEAN(3) HT_LEAN(4) HT_LEAN(5) HT_LEAN(6) HT_LEAN(7) HT_LEAN(8) HT_LEAN(9) HT_LEAN(10)
+        HT_LEAN(11) HT_LEAN(12) HT_LEAN(13) HT_LEAN(14) HT_LEAN(15) HT_LEAN(16)
+      }
+#undef HT_LEAN
+#undef HT_LEAN_LAUNCH
       HT_LAUNCH_CHECK("forest backward (trees)");
       return HT_OK;
     }

@@ -130,6 +130,32 @@ def test_backward_deterministic(dev, case, dtype, fern):
         assert torch.equal(dw.cpu(), rdw)
 
 
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("B", [4100, 4099], ids=["aligned", "ragged"])
+@pytest.mark.parametrize("M", list(range(1, 17)))
+def test_backward_row_widths(dev, M, B, fern):
+    """Every row width the specialised tree kernel is instantiated for (1 to 16 outputs per leaf: one, two or four
+    lanes per pair, rows that end inside a 16-byte chunk, swizzled accumulator rows for even widths), on a problem
+    large enough for the staged backward, with a sample count that is and is not a multiple of four (superblocks vs.
+    single blocks and the incomplete tail); training path and stateless path, both modes."""
+    x, thr, ordn, w, gout = make_forest(B, 24, [], 70, 5, [M], fern, torch.float32, seed=M)
+    (rdx, rdthr, rdw), slack, exact = _reference_gradients(x, thr, ordn, w, gout, fern)
+    gx, gthr, gord, gw, gg = _gpu(dev, x, thr, ordn, w, gout)
+    pre = "fern_" if fern else "tree_"
+    _, rec = getattr(ops, pre + "forward_records")(gx, gthr, gord, gw)
+    results = [getattr(ops, pre + "backward")(gx, True, gthr, True, gord, False, gw, True, gg),
+               getattr(ops, pre + "backward_deterministic")(gx, True, gthr, True, gord, False, gw, True, gg),
+               getattr(ops, pre + "backward_records")(rec, False, gx, True, gthr, True, gord, False, gw, True, gg),
+               getattr(ops, pre + "backward_records")(rec, True, gx, True, gthr, True, gord, False, gw, True, gg)]
+    assert torch.equal(results[1][3], results[3][3]) and torch.equal(results[1][0], results[3][0])
+    for dx, dthr, _, dw in results:
+        assert rel_err(dx.cpu(), rdx) <= 1e-5 + slack[0]
+        assert rel_err(dthr.cpu(), rdthr) <= 1e-5 + slack[1]
+        assert rel_err(dw.cpu(), rdw) <= 1e-5 + slack[2]
+        for got, want in zip((dx, dthr, dw), exact):
+            assert rel_err(got.cpu().double(), want.double()) <= 1e-5
+
+
 def _same_or_nan(a, b):
     return bool(((a == b) | (a.isnan() & b.isnan())).all())
 
