@@ -401,7 +401,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
                                                               Records<Real, COMPACT> rec, Real *dw,
                                                               unsigned long long *dw_fixed, const DetHeader *hdr,
                                                               int TB, long long part_size, bool need_c,
-                                                              bool dw_atomic, int P, int num_groups) {
+                                                              bool dw_atomic, int P, int num_groups, int slices) {
   constexpr int VE = 16 / sizeof(Real);  // elements per 16-byte chunk
   typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -413,13 +413,25 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
     inv_scale = hdr->inv_scale_w;
     if (!dw && !need_c) return;
   }
-  const int group = xcd_tree_group(blockIdx.x, num_groups);
+  int group = xcd_tree_group(blockIdx.x, num_groups);
   if (group < 0) return;
+  // slices > 1 (one tree per group; its leaf table does not fit LDS): `slices` consecutive groups serve the same tree,
+  // each accumulating the leaves [leaf_begin, leaf_begin + leaves) only. Every slice streams all records and gradient
+  // rows of the tree (the loads go out before the keys are known; loading a slice's own rows only, once the keys are
+  // there, was measured slower: the chain record -> row costs more than the L2 traffic it saves); c is computed by
+  // the first slice.
+  const int slice = group % slices;
+  group /= slices;
+  const int leaves = d.L / slices;
+  const uint32_t leaf_begin = uint32_t(slice) * uint32_t(leaves);
+  if (slice != 0) need_c = false;
+  if (!dw && !need_c) return;
   const int t0 = group * TB;
   const int nt = min(TB, d.T - t0);
   const long long LM = (long long)d.L * d.M;
+  const long long acc_cells = (long long)nt * leaves * d.M;  // (nt == 1 whenever slices > 1)
   if (dw) {
-    for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) acc[i] = Acc(0);
+    for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads) acc[i] = Acc(0);
     __syncthreads();
   }
   const long long s_begin = (long long)blockIdx.y * part_size;
@@ -512,6 +524,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
     Chunk cur;
     prefetch(c, cur);
     uint32_t rel[U];
+    bool in_slice[U];
     Real mg[U];
     Real wv[U][VE];
 #pragma unroll
@@ -520,10 +533,13 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
       mg[u] = __shfl(cur.mg_r, cur.src[u], kWave);
       rel[u] = (uint32_t(cur.tq_of[u]) * d.L + key) * d.M + e0;
       if (need_c) load_chunk(wbase + rel[u], wv[u]);
+      // the pair's accumulator row: this slice's leaves only, counted from the slice's first leaf
+      in_slice[u] = cur.on[u] && key - leaf_begin < uint32_t(leaves);
+      rel[u] -= leaf_begin * uint32_t(d.M);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      if (dw && cur.on[u]) {
+      if (dw && in_slice[u]) {
         const Real a = ht_abs(mg[u]);
         Acc *cell = acc + rel[u];
 #pragma unroll
@@ -559,22 +575,23 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
   if (FIXED && need_c) publish_c_bound(c_bound, hdr);
   if (dw) {
     __syncthreads();
-    Real *dst = dw + (long long)t0 * LM;
+    const long long first = (long long)t0 * LM + (long long)leaf_begin * d.M;
+    Real *dst = dw + first;
     if (FIXED) {
       const unsigned long long *q = reinterpret_cast<const unsigned long long *>(acc);
       if (dw_atomic) {
-        for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads)
-          if (q[i] != 0ull) atomicAdd(dw_fixed + (long long)t0 * LM + i, q[i]);
+        for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads)
+          if (q[i] != 0ull) atomicAdd(dw_fixed + first + i, q[i]);
       } else {
-        for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) dst[i] = from_fixed<Real>(q[i], inv_scale);
+        for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads) dst[i] = from_fixed<Real>(q[i], inv_scale);
       }
     } else {
       const double *q = reinterpret_cast<const double *>(acc);
       if (dw_atomic) {
-        for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads)
+        for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads)
           if (q[i] != 0.0) atomicAdd(dst + i, Real(q[i]));
       } else {
-        for (long long i = threadIdx.x; i < nt * LM; i += kForestThreads) dst[i] = Real(q[i]);
+        for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads) dst[i] = Real(q[i]);
       }
     }
   }
@@ -1697,10 +1714,12 @@ __global__ __launch_bounds__(kWave) void det_tree_kernel(ForestDims d, const Rea
 constexpr int kLeanMaxOutputs = 16;  // tree_lean_kernel: at most four lanes of four values per pair
 struct TreePlan {
   int TB;               // trees per workgroup
-  int groups, parts;    // grid
+  int groups, parts;    // grid (groups counts tree groups x leaf slices)
   long long part_size;  // samples per part
   size_t lds;
+  int slices;           // > 1: a tree's leaf table is split over that many workgroups (generic tree kernel only)
 };
+constexpr int kMaxLeafSlices = 1024;
 
 // Single-output leaf tables (M == 1, 4 bytes per leaf) are small enough to sit in LDS next to the accumulators of the
 // lean tree kernel; its leaf-weight gathers then never leave the CU.
@@ -1712,8 +1731,29 @@ static bool plan_trees(const ForestDims &d, bool need_dw, bool lean, TreePlan *p
   const size_t per_tree = size_t(d.L) * d.M * sizeof(double);
   const size_t w_tree = staged_weights_per_tree(d, lean);
   int tb = 4;
+  p->slices = 1;
   if (need_dw) {
-    if (per_tree > size_t(kLdsBytes)) return false;
+    if (per_tree > size_t(kLdsBytes)) {
+      // one tree's table is too large: slices of its leaves (a power of two of them, like the leaves), one tree at a time
+      int slices = 2;
+      while (per_tree / slices > size_t(kLdsBytes) && slices < d.L) slices *= 2;
+      if (per_tree / slices > size_t(kLdsBytes) || slices > kMaxLeafSlices || slices > d.L) return false;
+      p->slices = slices;
+      p->TB = 1;
+      p->groups = d.T * slices;
+      p->parts = 1;
+      p->part_size = d.S;
+      if (p->groups < kNumCUs) {
+        long long parts = (kNumCUs + p->groups - 1) / p->groups;
+        const long long max_parts = (d.S + 4 * kForestThreads - 1) / (4 * kForestThreads);
+        if (parts > max_parts) parts = max_parts;
+        if (parts < 1) parts = 1;
+        p->part_size = (d.S + parts - 1) / parts;
+        p->parts = int((d.S + p->part_size - 1) / p->part_size);
+      }
+      p->lds = per_tree / slices;
+      return true;
+    }
     tb = int(size_t(kLdsBytes) / per_tree);
   }
   if (w_tree != 0) {
@@ -1783,7 +1823,8 @@ int launch_tree_kernel_u(const ForestDims &d, const TreePlan &p, int P, const Re
                                    int(p.lds)));
   const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
   hipLaunchKernelGGL(kernel, dim3((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts), dim3(kForestThreads), p.lds,
-                     stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB, p.part_size, need_c, p.parts > 1, P, p.groups);
+                     stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB, p.part_size, need_c, p.parts > 1, P, p.groups,
+                     p.slices);
   HT_LAUNCH_CHECK("forest backward (trees)");
   return HT_OK;
 }
@@ -1791,7 +1832,8 @@ int launch_tree_kernel_u(const ForestDims &d, const TreePlan &p, int P, const Re
 // Shapes of tree_wide_kernel: M = 4 * P with P a power of two from 4 to 64, leaf offsets of a tree group in 32 bits.
 static bool wide_rows_ok(const ForestDims &d, const TreePlan &p) {
   const int P4 = d.M / 4;
-  return d.M % 4 == 0 && P4 >= 4 && P4 <= kWave && (P4 & (P4 - 1)) == 0 && (long long)p.TB * d.L * d.M < (1ll << 31);
+  return p.slices == 1 && d.M % 4 == 0 && P4 >= 4 && P4 <= kWave && (P4 & (P4 - 1)) == 0 &&
+         (long long)p.TB * d.L * d.M < (1ll << 31);
 }
 
 // Shapes of tree_lean_kernel (float, compact records): contiguous rows of up to 16 outputs, a power-of-two tree group,
@@ -1800,7 +1842,7 @@ static bool lean_tree_ok(const ForestDims &d, const TreePlan &p, int *log2_tb_ou
   int log2_tb = 0;
   while ((1 << (log2_tb + 1)) <= p.TB) ++log2_tb;
   if (log2_tb_out) *log2_tb_out = log2_tb;
-  return d.K == 1 && (1 << log2_tb) == p.TB && p.TB <= 16 && (long long)kWave * d.T * d.M < (1ll << 31) &&
+  return p.slices == 1 && d.K == 1 && (1 << log2_tb) == p.TB && p.TB <= 16 && (long long)kWave * d.T * d.M < (1ll << 31) &&
          (long long)p.TB * d.L * d.M < (1ll << 31) && d.M >= 1 && d.M <= kLeanMaxOutputs;
 }
 
@@ -1930,7 +1972,10 @@ bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw, bool fixed) {
   // the gradient rows of one 64-sample step with 32-bit offsets
   if ((d.M + 16 / int(sizeof(Real)) - 1) / (16 / int(sizeof(Real))) > kWave) return false;
   if ((long long)d.T * d.M * kWave >= (1ll << 31)) return false;
-  if (need_dw && size_t(d.L) * d.M * sizeof(double) > size_t(kLdsBytes)) return false;
+  // (a leaf table beyond LDS is accumulated in slices of its leaves, each at least one leaf row)
+  if (need_dw && size_t(d.L) * d.M * sizeof(double) > size_t(kLdsBytes) * kMaxLeafSlices) return false;
+  if (need_dw && size_t(d.M) * sizeof(double) > size_t(kLdsBytes)) return false;
+  if ((long long)d.L * d.M >= (1ll << 31)) return false;
   if (size_t(d.V) * sizeof(double) > size_t(kLdsBytes)) return false;
   // (atomic mode serves a feature space too wide for the dX tile with one global atomic per pair instead)
   if (need_dx && fixed && pick_dx_tile(d.F, sizeof(unsigned long long)) == 0) return false;

@@ -44,6 +44,12 @@ CASES = [
     (3, 30, [70, 33], 50, 5, [8, 8]),      # the segmentation head's shape in small
     (2500, 11, [], 110, 2, [128]),
     (1300, 8, [], 210, 2, [256]),
+    # one tree's leaf table beyond LDS (1024 leaves x 24 outputs, 8192 x 6, 2048 x 3 x 7 with inner positions): the
+    # staged backward accumulates it in slices of its leaves
+    (600, 30, [], 500, 10, [24]),
+    (2000, 16, [], 140, 13, [6]),
+    (90, 12, [33], 100, 11, [3, 7]),
+    (640, 16, [], 420, 10, [8, 8]),        # ... on the wide-row kernel (64 outputs per leaf, four slices)
 ]
 
 
