@@ -1252,11 +1252,13 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
   }
 }
 
-// dThr[t, v] = sum over samples with selected vertex v of -c. One workgroup per tree (x sample parts).
+// dThr[t, v] = sum over samples with selected vertex v of -c. One workgroup per tree (x sample parts); where a tree's
+// vertex table does not fit LDS (depth 15 and more), `vslices` workgroups per tree, each owning a range of vertices
+// and passing over all of the tree's records.
 template <typename Real, bool COMPACT, bool FIXED>
 __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dthr,
                                                    unsigned long long *dthr_fixed, const DetHeader *hdr,
-                                                   long long part_size, bool use_atomic) {
+                                                   long long part_size, bool use_atomic, int vslices) {
   typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
   extern __shared__ __align__(16) unsigned char smem[];
   Acc *acc = reinterpret_cast<Acc *>(smem);  // fp64 / int64: fast LDS atomics, and the root vertex is a hot spot
@@ -1266,8 +1268,11 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
     scale = hdr->scale_c;
     inv_scale = hdr->inv_scale_c;
   }
-  const int t = blockIdx.x;
-  for (int i = threadIdx.x; i < d.V; i += 256) acc[i] = Acc(0);
+  const int t = int(blockIdx.x) / vslices, vslice = int(blockIdx.x) - t * vslices;
+  const int per_slice = (d.V + vslices - 1) / vslices;
+  const uint32_t v_begin = uint32_t(vslice) * uint32_t(per_slice);
+  const int nv = max(0, min(per_slice, d.V - int(v_begin)));  // this workgroup's vertices [v_begin, v_begin + nv)
+  for (int i = threadIdx.x; i < nv; i += 256) acc[i] = Acc(0);
   __syncthreads();
   const long long s_begin = (long long)blockIdx.y * part_size;
   const long long s_end = min(d.S, s_begin + part_size);
@@ -1285,11 +1290,12 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
       val = to_fixed(-double(c), scale);
     else
       val = -double(c);
+    if (v - v_begin >= uint32_t(nv)) return;  // another slice's vertex
     if (v < uint32_t(kTop)) {
 #pragma unroll
       for (int k = 0; k < kTop; ++k) top[k] += v == uint32_t(k) ? val : Acc(0);
     } else {
-      atomicAdd(acc + v, val);
+      atomicAdd(acc + (v - v_begin), val);
     }
   };
   for (long long s0 = s_begin + threadIdx.x; s0 < s_end; s0 += 256 * kBatch) {
@@ -1313,15 +1319,15 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
   for (int k = 0; k < kTop; ++k) {
     Acc sum = top[k];
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, kWave);
-    if ((threadIdx.x & (kWave - 1)) == 0 && k < d.V) atomicAdd(acc + k, sum);
+    if ((threadIdx.x & (kWave - 1)) == 0 && vslice == 0 && k < nv) atomicAdd(acc + k, sum);
   }
   __syncthreads();
-  Real *dst = dthr + (long long)t * d.V;
-  for (int i = threadIdx.x; i < d.V; i += 256) {
+  Real *dst = dthr + (long long)t * d.V + v_begin;
+  for (int i = threadIdx.x; i < nv; i += 256) {
     if (FIXED) {
       const unsigned long long q = reinterpret_cast<const unsigned long long *>(acc)[i];
       if (use_atomic) {
-        if (q != 0ull) atomicAdd(dthr_fixed + (long long)t * d.V + i, q);
+        if (q != 0ull) atomicAdd(dthr_fixed + (long long)t * d.V + v_begin + i, q);
       } else {
         dst[i] = from_fixed<Real>(q, inv_scale);
       }
@@ -1976,7 +1982,8 @@ bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw, bool fixed) {
   if (need_dw && size_t(d.L) * d.M * sizeof(double) > size_t(kLdsBytes) * kMaxLeafSlices) return false;
   if (need_dw && size_t(d.M) * sizeof(double) > size_t(kLdsBytes)) return false;
   if ((long long)d.L * d.M >= (1ll << 31)) return false;
-  if (size_t(d.V) * sizeof(double) > size_t(kLdsBytes)) return false;
+  // (a vertex table beyond LDS is accumulated in slices of its vertices)
+  if (size_t(d.V) * sizeof(double) > size_t(kLdsBytes) * 64) return false;
   // (atomic mode serves a feature space too wide for the dX tile with one global atomic per pair instead)
   if (need_dx && fixed && pick_dx_tile(d.F, sizeof(unsigned long long)) == 0) return false;
   return true;
@@ -2119,8 +2126,14 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
   }
 
   if (dthr && !dthr_done) {
-    hipLaunchKernelGGL((dthr_kernel<Real, COMPACT, FIXED>), dim3((unsigned)d.T, (unsigned)dthr_gy), dim3(256),
-                       size_t(d.V) * sizeof(double), stream, d, rec, dthr, dthr_fixed, hdr, dthr_part, dthr_gy > 1);
+    const int vslices = int((size_t(d.V) * sizeof(double) + size_t(kLdsBytes) - 1) / size_t(kLdsBytes));
+    const size_t thr_lds = size_t((d.V + vslices - 1) / vslices) * sizeof(double);
+    if ((long long)d.T * vslices > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many trees for one launch.");
+    auto thr_kernel = dthr_kernel<Real, COMPACT, FIXED>;
+    HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(thr_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(thr_lds)));
+    hipLaunchKernelGGL(thr_kernel, dim3((unsigned)(d.T * vslices), (unsigned)dthr_gy), dim3(256), thr_lds, stream, d,
+                       rec, dthr, dthr_fixed, hdr, dthr_part, dthr_gy > 1, vslices);
     HT_LAUNCH_CHECK("forest backward (dThr)");
     if (FIXED) {
       if (dthr_gy > 1) {
@@ -2130,11 +2143,16 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
         HT_LAUNCH_CHECK("forest backward (dThr conversion)");
       }
       const size_t need = size_t(d.V) * sizeof(Real);
-      auto kernel = det_tree_kernel<Real, true, COMPACT>;
-      HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(need)));
-      hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, dthr,
-                         (Real *)nullptr, &hdr->fallback_c);
+      if (need <= size_t(kLdsBytes) / 3) {
+        auto kernel = det_tree_kernel<Real, true, COMPACT>;
+        HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(need)));
+        hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, dthr,
+                           (Real *)nullptr, &hdr->fallback_c);
+      } else {
+        hipLaunchKernelGGL((det_tree_kernel<Real, false, COMPACT>), dim3((unsigned)d.T), dim3(kWave), 0, stream, d, w,
+                           gout, rec, dthr, (Real *)nullptr, &hdr->fallback_c);
+      }
       HT_LAUNCH_CHECK("forest backward (dThr fallback)");
     }
   }

@@ -49,7 +49,10 @@ CASES = [
     (600, 30, [], 500, 10, [24]),
     (2000, 16, [], 140, 13, [6]),
     (90, 12, [33], 100, 11, [3, 7]),
-    (640, 16, [], 420, 10, [8, 8]),        # ... on the wide-row kernel (64 outputs per leaf, four slices)
+    (640, 16, [], 420, 10, [8, 8]),        # ... 64 outputs per leaf, four slices
+    # depth 15 and 16: the vertex table of a tree is beyond LDS as well (dThr in slices of the vertices)
+    (2100, 20, [], 130, 15, [2]),
+    (4200, 12, [], 64, 16, []),
 ]
 
 
