@@ -1344,9 +1344,11 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
 
 // dX: sample tile x all trees. LDS accumulator [F][BT+1] (the pad keeps the transposing write-out conflict free).
 // FIXED: 64-bit fixed-point cells; dX is cleared beforehand and left alone when the header asks for the fallback.
+// A feature space too wide for the tile is served in windows of f_per features (blockIdx.y): every window passes
+// over all records of the tile's samples and keeps the terms whose ordinal falls inside it.
 template <typename Real, int BT, bool COMPACT, bool FIXED>
 __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dx,
-                                                            const DetHeader *hdr) {
+                                                            const DetHeader *hdr, int f_per) {
   typedef typename std::conditional<FIXED, unsigned long long, Real>::type Acc;
   constexpr int NT = kForestThreads;
   constexpr int TC = NT / BT;
@@ -1359,7 +1361,9 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
     scale = hdr->scale_c;
     inv_scale = hdr->inv_scale_c;
   }
-  for (int i = threadIdx.x; i < d.F * LD; i += NT) acc[i] = Acc(0);
+  const uint32_t f_begin = blockIdx.y * uint32_t(f_per);
+  const uint32_t nf = uint32_t(min(f_per, d.F - int(f_begin)));  // this workgroup's features [f_begin, f_begin + nf)
+  for (int i = threadIdx.x; i < int(nf) * LD; i += NT) acc[i] = Acc(0);
   __syncthreads();
   const long long s0 = (long long)blockIdx.x * BT;
   const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
@@ -1396,7 +1400,8 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
             if (t0 + i * TCQ >= d.T) break;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              const uint32_t o = av[i][e] >> rec.oshift;
+              const uint32_t o = (av[i][e] >> rec.oshift) - f_begin;
+              if (o >= nf) continue;
               if (FIXED)
                 atomicAdd(reinterpret_cast<unsigned long long *>(acc) + o * LD + jq + e,
                           to_fixed(double(cv[i][e]), scale));
@@ -1418,12 +1423,13 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
       for (int i = 0; i < kBatch; ++i) {
         const int t = min(t0 + i * TC, d.T - 1);
         const long long at = (long long)t * d.S + s;
-        o[i] = rec.ord(at);
+        o[i] = rec.ord(at) - f_begin;
         cv[i] = __builtin_nontemporal_load(rec.c + at);
       }
 #pragma unroll
       for (int i = 0; i < kBatch; ++i) {
         if (t0 + i * TC >= d.T) break;
+        if (o[i] >= nf) continue;
         if (FIXED)
           atomicAdd(reinterpret_cast<unsigned long long *>(acc) + o[i] * LD + j, to_fixed(double(cv[i]), scale));
         else
@@ -1440,29 +1446,16 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
     // dx[s, 0..F) is a contiguous row: a wavefront per sample, lanes along the features
     const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
     for (int jj = wv; jj < BT && s0 + jj < d.S; jj += NT / kWave) {
-      Real *row = dx + (s0 + jj) * d.F;
-      for (int f = lane; f < d.F; f += kWave) row[f] = cell(f, jj);
+      Real *row = dx + (s0 + jj) * d.F + f_begin;
+      for (int f = lane; f < int(nf); f += kWave) row[f] = cell(f, jj);
     }
   } else {
     // dx[b, f, k]: consecutive samples of a tile are consecutive k (within one b)
-    for (int i = threadIdx.x; i < d.F * BT; i += NT) {
+    for (int i = threadIdx.x; i < int(nf) * BT; i += NT) {
       const int f = i / BT, jj = i - f * BT;
       const long long ss = s0 + jj;
-      if (ss < d.S) dx[(ss / d.K) * d.FK + (long long)f * d.K + (ss % d.K)] = cell(f, jj);
+      if (ss < d.S) dx[(ss / d.K) * d.FK + (long long)(f_begin + f) * d.K + (ss % d.K)] = cell(f, jj);
     }
-  }
-}
-
-// dX for feature spaces too wide for an LDS tile (atomic mode): one global atomic per (tree, sample) pair straight
-// into the pre-cleared dX. With F in the thousands two pairs of one sample rarely meet, so the atomics do not
-// contend; the pair count, not the feature count, sets the cost.
-template <typename Real, bool COMPACT>
-__global__ __launch_bounds__(256) void dx_scatter_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dx) {
-  const long long pairs = (long long)d.T * d.S;
-  for (long long at = (long long)blockIdx.x * 256 + threadIdx.x; at < pairs; at += (long long)gridDim.x * 256) {
-    const long long s = at % d.S;
-    const Real c = rec.c[at];
-    if (c != Real(0)) atomicAdd(dx + (s / d.K) * d.FK + (long long)rec.ord(at) * d.K + (s % d.K), c);
   }
 }
 
@@ -1952,13 +1945,18 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
 
 template <typename Real, int BT, bool COMPACT, bool FIXED>
 int launch_dx(const ForestDims &d, Records<Real, COMPACT> rec, Real *dx, const DetHeader *hdr, hipStream_t stream) {
-  const size_t lds = size_t(d.F) * (BT + 1) * (FIXED ? sizeof(unsigned long long) : sizeof(Real));
+  const size_t cell = (BT + 1) * (FIXED ? sizeof(unsigned long long) : sizeof(Real));  // bytes per feature
+  int f_per = d.F;  // features per workgroup: all of them, or as many as LDS holds
+  if (size_t(f_per) * cell > size_t(kLdsBytes)) f_per = int(size_t(kLdsBytes) / cell);
+  const int windows = (d.F + f_per - 1) / f_per;
+  const size_t lds = size_t(f_per) * cell;
   const long long tiles = (d.S + BT - 1) / BT;
-  if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
+  if (tiles > 0x7fffffffLL || windows > 65535) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
   auto kernel = dx_kernel<Real, BT, COMPACT, FIXED>;
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kForestThreads), lds, stream, d, rec, dx, hdr);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)windows), dim3(kForestThreads), lds, stream, d, rec, dx, hdr,
+                     f_per);
   HT_LAUNCH_CHECK("forest backward (dX)");
   return HT_OK;
 }
@@ -1984,8 +1982,8 @@ bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw, bool fixed) {
   if ((long long)d.L * d.M >= (1ll << 31)) return false;
   // (a vertex table beyond LDS is accumulated in slices of its vertices)
   if (size_t(d.V) * sizeof(double) > size_t(kLdsBytes) * 64) return false;
-  // (atomic mode serves a feature space too wide for the dX tile with one global atomic per pair instead)
-  if (need_dx && fixed && pick_dx_tile(d.F, sizeof(unsigned long long)) == 0) return false;
+  // (dX of a feature space too wide for the tile: windows of features, at most 65535 of them)
+  if (need_dx && (long long)d.F * 9 * 8 > (long long)kLdsBytes * 65535) return false;
   return true;
 }
 
@@ -2162,14 +2160,9 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
       case 32: rc = launch_dx<Real, 32, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
       case 16: rc = launch_dx<Real, 16, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
       case 8: rc = launch_dx<Real, 8, COMPACT, FIXED>(d, rec, dx, hdr, stream); break;
-      default: {  // no tile fits (atomic mode only, see staged_ok); dX was cleared by the caller
-        const long long pairs = (long long)d.T * d.S;
-        long long blocks = (pairs + 255) / 256;
-        if (blocks > 16 * kNumCUs) blocks = 16 * kNumCUs;
-        hipLaunchKernelGGL((dx_scatter_kernel<Real, COMPACT>), dim3((unsigned)blocks), dim3(256), 0, stream, d, rec, dx);
-        HT_LAUNCH_CHECK("forest backward (dX, scattered)");
+      default:  // no tile holds all features: windows of features on the smallest tile
+        rc = launch_dx<Real, 8, COMPACT, FIXED>(d, rec, dx, hdr, stream);
         break;
-      }
     }
     if (rc != HT_OK) return rc;
     if (FIXED) {
@@ -2273,7 +2266,7 @@ template <typename Real>
 int clear_gradients(const ForestDims &d, Route route, Real *dx, Real *dthr, Real *dw, hipStream_t stream, bool *done) {
   int rc;
   const bool empty = is_empty(d);
-  const bool clear_dx = route != Route::kStaged || empty || pick_dx_tile(d.F, sizeof(Real)) == 0;
+  const bool clear_dx = route != Route::kStaged || empty;
   if (dx && clear_dx && (rc = zero_fill(dx, size_t(d.S) * d.F * sizeof(Real), stream)) != HT_OK) return rc;
   // The staged atomic route stores dW and dThr from its LDS tables (every cell, by the workgroup that owns the tree)
   // unless the samples are split over several workgroups, whose shares then meet in atomics on the cleared buffers.

@@ -3,7 +3,7 @@
 Bars: leaf keys, selected ordinals, signed margins and forward outputs bit-exact; gradients within 1e-5 (fp32,
 relative to the largest reference entry of the tensor; the summation order differs from the serial CPU loop) and
 1e-12 (fp64); deterministic mode bit-identical run to run (fixed-point accumulation), and where it has to use its
-sequential kernels (accumulators that do not fit on chip, non-finite magnitudes) dX / dW bit-identical to the CPU order.
+sequential kernels (non-finite magnitudes) dX / dW bit-identical to the CPU order.
 """
 import itertools
 
@@ -26,7 +26,7 @@ CASES = [
     (19, 13, [3, 2], 6, 4, [2, 3]),
     (5, 7, [70], 3, 5, [4]),
     (130, 300, [], 35, 10, [3]),
-    (4, 5000, [], 3, 4, [2]),              # feature count too large for an LDS tile of 8 float64 rows
+    (4, 5000, [], 3, 4, [2]),              # feature count too large for an LDS tile of 8 rows: dX in feature windows
     # large enough (>= 2^18 sample x tree pairs) for the staged backward: records -> trees -> dThr -> dX
     (2048, 40, [], 130, 6, [10]),
     (300, 17, [10], 90, 5, [3]),           # inner data dims, odd extra outputs
@@ -133,10 +133,6 @@ def test_backward_deterministic(dev, case, dtype, fern):
     assert rel_err(dthr.cpu(), rdthr) <= tol + slack[1]
     for got, want in zip((dx, dthr, dw), exact):
         assert rel_err(got.cpu().double(), want.double()) <= tol
-    if F == 5000:
-        # too wide for an on-chip dX tile: the sequential kernels add dX and dW terms in the CPU loop's order
-        assert torch.equal(dx.cpu(), rdx)
-        assert torch.equal(dw.cpu(), rdw)
 
 
 @pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
