@@ -350,10 +350,15 @@ __device__ __forceinline__ void conv_walks(bool plain, int depth, const Node<Rea
 
 // MREG = outputs per leaf kept in registers per pass over the channels (1, 4 or 16: the smallest that holds M, so the
 // common single-output case carries no per-output loop at all).
+// Channel windows: where the tile planes and the staged trees of all C channels would leave room for one workgroup per
+// CU only (many channels, deep trees, many outputs per leaf), the workgroup takes c_per channels at a time -- loads
+// their planes, then for every out channel stages their trees and adds their terms to what the earlier windows left
+// in `out`. The terms of a position are still added one by one in ascending channel order to the same running value
+// (it merely passes through memory between windows), so the result is bit for bit the one of a single pass.
 template <typename Real, bool FERN, int MREG>
-__global__ __launch_bounds__(kConvThreads) void conv_tiled_forward_kernel(ConvTile g, ConvLds lay, int C, int Cout,
-                                                                          int depth, int V, int L, int M, int j_per,
-                                                                          const Real *__restrict__ x,
+__global__ __launch_bounds__(kConvThreads) void conv_tiled_forward_kernel(ConvTile g, ConvLds lay, int C_all, int c_per,
+                                                                          int Cout, int depth, int V, int L, int M,
+                                                                          int j_per, const Real *__restrict__ x,
                                                                           const Real *__restrict__ thr,
                                                                           const int64_t *__restrict__ ord,
                                                                           const Real *__restrict__ w,
@@ -366,51 +371,54 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_forward_kernel(ConvTi
   const long long b = blockIdx.z;
   int *special = reinterpret_cast<int *>(smem + lay.flag);
   if (threadIdx.x == 0) *special = 0;
-  __syncthreads();
-  load_conv_tile<Real, true>(tile, x, g, C, b, tyi, txi, special);
   const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
   const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
   const bool live = oy < g.OH && ox < g.OW;
   const Real *mine = tile + ty * g.sy * g.IW + tx * g.sx;
   const int LM = L * M;
   const int j_begin = blockIdx.y * j_per, j_end = min(Cout, j_begin + j_per);
-  for (int j = j_begin; j < j_end; ++j) {
-    __syncthreads();  // the tile is complete / the previous out channel's trees are no longer read
-    stage_conv_trees<Real, true>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
-    __syncthreads();
-    if (!live) continue;
-    const bool plain = *special == 0;
-    Real *o = out + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
-    for (int m0 = 0; m0 < M; m0 += MREG) {
-      const int mc = min(MREG, M - m0);
-      Real acc[MREG];
+  for (int c0 = 0; c0 < C_all; c0 += c_per) {
+    const int C = min(c_per, C_all - c0);
+    __syncthreads();  // the flag is cleared / the previous window's planes and trees are no longer read
+    load_conv_tile<Real, true>(tile, x, g, C_all, b, tyi, txi, special, c0, C);
+    for (int j = j_begin; j < j_end; ++j) {
+      __syncthreads();  // the planes are complete / the previous out channel's trees are no longer read
+      stage_conv_trees<Real, true>(nodes, wl, g, C_all, V, LM, j, thr, ord, w, special, c0, C);
+      __syncthreads();
+      if (!live) continue;
+      const bool plain = *special == 0;
+      Real *o = out + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+      for (int m0 = 0; m0 < M; m0 += MREG) {
+        const int mc = min(MREG, M - m0);
+        Real acc[MREG];
 #pragma unroll
-      for (int m = 0; m < MREG; ++m) acc[m] = Real(0);
-      for (int c = 0; c < C; c += kConvIlp) {
-        // several channels' walks interleaved; their terms are still added in ascending channel order
-        WalkResult<Real> r[kConvIlp];
-        const Node<Real> *nd[kConvIlp];
-        const Real *px[kConvIlp];
+        for (int m = 0; m < MREG; ++m) acc[m] = (c0 == 0 || (MREG != 1 && m >= mc)) ? Real(0) : o[m0 + m];
+        for (int c = 0; c < C; c += kConvIlp) {
+          // several channels' walks interleaved; their terms are still added in ascending channel order
+          WalkResult<Real> r[kConvIlp];
+          const Node<Real> *nd[kConvIlp];
+          const Real *px[kConvIlp];
 #pragma unroll
-        for (int i = 0; i < kConvIlp; ++i) {
-          const int ci = min(c + i, C - 1);  // surplus slots re-walk the last channel, unused
-          nd[i] = nodes + ci * V;
-          px[i] = mine + ci * g.TSZ;
+          for (int i = 0; i < kConvIlp; ++i) {
+            const int ci = min(c + i, C - 1);  // surplus slots re-walk the last channel, unused
+            nd[i] = nodes + ci * V;
+            px[i] = mine + ci * g.TSZ;
+          }
+          conv_walks<Real, FERN, false>(plain, depth, nd, px, r);
+#pragma unroll
+          for (int i = 0; i < kConvIlp; ++i) {
+            if (c + i >= C) break;
+            const Real a = r[i].margin;  // |margin|
+            const Real *row = wl + ((c + i) * L + r[i].key) * M + m0;
+#pragma unroll
+            for (int m = 0; m < MREG; ++m)
+              if (MREG == 1 || m < mc) acc[m] = acc[m] + row[m] * a;
+          }
         }
-        conv_walks<Real, FERN, false>(plain, depth, nd, px, r);
 #pragma unroll
-        for (int i = 0; i < kConvIlp; ++i) {
-          if (c + i >= C) break;
-          const Real a = r[i].margin;  // |margin|
-          const Real *row = wl + ((c + i) * L + r[i].key) * M + m0;
-#pragma unroll
-          for (int m = 0; m < MREG; ++m)
-            if (MREG == 1 || m < mc) acc[m] = acc[m] + row[m] * a;
-        }
+        for (int m = 0; m < MREG; ++m)
+          if (MREG == 1 || m < mc) o[m0 + m] = acc[m];
       }
-#pragma unroll
-      for (int m = 0; m < MREG; ++m)
-        if (MREG == 1 || m < mc) o[m0 + m] = acc[m];
     }
   }
 }
@@ -813,7 +821,16 @@ int conv_forward(const ht_conv_shape &s, const Real *x, const Real *thr, const i
   ConvTile t;
   if (make_tile(g, &t)) {
     const int LM = L * int(s.M);
-    const ConvLds lay = conv_lds_layout<Real>(t, int(s.C), V, LM, false, false, true);
+    // channels per window: all of them while four workgroups still fit a CU, else halved (not below four channels:
+    // every window re-stages its trees per out channel and passes the running sums through memory). Trees of more
+    // than 255 vertices are not split into windows: staging them costs more than a tile of positions gets out of
+    // them, and where they do not fit at once the kernel below, which reads vertices through the caches, is faster.
+    int c_per = int(s.C);
+    ConvLds lay = conv_lds_layout<Real>(t, c_per, V, LM, false, false, true);
+    while (V <= 255 && lay.total > kConvTiledLdsMax / 4 && c_per >= 8) {
+      c_per = (c_per + 1) / 2;
+      lay = conv_lds_layout<Real>(t, c_per, V, LM, false, false, true);
+    }
     if (lay.total <= kConvTiledLdsMax && (long long)t.tiles_y * t.tiles_x <= 0x7fffffffLL) {
       const long long tiles = (long long)t.tiles_y * t.tiles_x;
       const int j_per = conv_j_per(tiles * s.B, int(s.Cout));
@@ -823,7 +840,7 @@ int conv_forward(const ht_conv_shape &s, const Real *x, const Real *thr, const i
       else if (s.M <= 4) kernel = fern ? conv_tiled_forward_kernel<Real, true, 4> : conv_tiled_forward_kernel<Real, false, 4>;
       HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, int(lay.total)));
-      hipLaunchKernelGGL(kernel, tgrid, dim3(kConvThreads), lay.total, stream, t, lay, int(s.C), int(s.Cout),
+      hipLaunchKernelGGL(kernel, tgrid, dim3(kConvThreads), lay.total, stream, t, lay, int(s.C), c_per, int(s.Cout),
                          int(s.depth), V, L, int(s.M), j_per, x, thr, ord, w, out);
       HT_LAUNCH_CHECK("conv forward (tiled)");
       return HT_OK;
@@ -878,6 +895,10 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
     int c_per = int(s.C);
     ConvLds lay = conv_lds_layout<Real>(t, c_per, V, LM, true, true, true);
     while (lay.total > kConvTiledLdsMax / 2 && c_per >= 16) {  // (at least 8 channels: the lanes' skew spreads over them)
+      c_per = (c_per + 1) / 2;
+      lay = conv_lds_layout<Real>(t, c_per, V, LM, true, true, true);
+    }
+    while (lay.total > kConvTiledLdsMax && c_per > 1) {  // ... unless nothing larger fits at all (deep trees)
       c_per = (c_per + 1) / 2;
       lay = conv_lds_layout<Real>(t, c_per, V, LM, true, true, true);
     }

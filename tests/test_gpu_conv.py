@@ -26,6 +26,9 @@ CASES = [
     (2, 40, 2, [9, 33], 2, [], [3, 3], [1, 1], [1, 1], [1, 1]),        # more channels than any tile holds in LDS
     (1, 19, 3, [21, 40], 5, [], [3, 3], [1, 1], [1, 1], [1, 1]),       # one-walk backward in two uneven channel windows
     (2, 35, 2, [18, 33], 4, [2], [3, 3], [1, 1], [1, 1], [1, 1]),      # ... in several, more than one output per leaf
+    (1, 70, 3, [20, 37], 6, [], [3, 3], [1, 1], [1, 1], [1, 1]),       # forward in channel windows (running sums pass through `out`)
+    (1, 21, 2, [23, 35], 5, [5], [3, 3], [2, 1], [1, 1], [1, 1]),      # ... with several outputs per leaf and a stride
+    (1, 6, 3, [24, 40], 10, [], [3, 3], [1, 1], [1, 1], [1, 1]),       # deep trees: the one-walk backward in windows of few channels
 ]
 
 
