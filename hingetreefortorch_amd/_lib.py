@@ -70,6 +70,7 @@ SIGNATURES = {
     "ht_contract": (_I, [ctypes.POINTER(TileShape), _P, _P, _P]),
     "ht_expand": (_I, [ctypes.POINTER(TileShape), _P, _P, _P]),
     "ht_projection_workspace": (_SZ, [ctypes.c_int64]),
+    "ht_projection_backward_workspace": (_SZ, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]),
     "ht_projection_forward": (_I, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _P, _P, ctypes.c_double, _P, _P, _P,
                                    _P, _P, _SZ, _P]),
     "ht_projection_backward": (_I, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _P, _P, _P, _P, _P, _P, _P, _P,

@@ -489,6 +489,9 @@ int ht_expand(const ht_tile_shape *s, const void *tiles, void *image, void *stre
 }
 
 size_t ht_projection_workspace(int64_t N) { return N < 0 ? 0 : projection_workspace(N); }
+size_t ht_projection_backward_workspace(int64_t B, int64_t K, int64_t N) {
+  return (B < 0 || K < 0 || N < 0) ? 0 : projection_backward_workspace(B, K, N);
+}
 
 int ht_projection_forward(int64_t B, int64_t K, int64_t N, const float *x, const float *lin, double eps, float *zhat,
                           float *mean, float *rstd, float *var, void *workspace, size_t workspace_bytes, void *stream) {
@@ -506,7 +509,7 @@ int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, cons
   if (B < 0 || K < 0 || N < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
   if (B > 0 && N > 0 && (!zhat || !rstd || !g || !workspace || (dlin && !x) || (dx && !lin)))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
-  if (workspace_bytes < projection_workspace(N))
+  if (workspace_bytes < projection_backward_workspace(B, K, N))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the projection.");
   return projection_backward(B, K, N, x, lin, zhat, rstd, g, dlin, dx, workspace, static_cast<hipStream_t>(stream));
 }

@@ -163,6 +163,7 @@ int tile_expand(const ht_tile_shape *s, const void *in, void *out, hipStream_t s
 
 // Dense projection + batch normalisation in front of a forest (projection.hip), fp32.
 size_t projection_workspace(long long N);
+size_t projection_backward_workspace(long long B, long long K, long long N);
 int projection_forward(long long B, long long K, long long N, const float *x, const float *lin, double eps,
                        float *zhat, float *mean, float *rstd, float *var, void *ws, hipStream_t stream);
 int projection_backward(long long B, long long K, long long N, const float *x, const float *lin, const float *zhat,

@@ -135,7 +135,8 @@ struct GemmArgs {
   long long lda, ldb, ldc, stride_a, stride_b, stride_c;
   int n_i, n_j, n_r, batches;
   int tiles_i, tiles_j, rows_per_xcd;  // result tiles, and how many tile rows each of the 8 L2 domains takes
-  int splits;                          // > 1: blockIdx.y takes a share of the reduction and adds into a zeroed C
+  int splits;                          // > 1: blockIdx.y takes a share of the reduction and adds into a zeroed C ...
+  long long split_stride;              // ... or, if not 0, stores its share at C + blockIdx.y * split_stride
   bool vec_a, vec_b;
   double *stats;
   const float *bias_i, *bias_j;
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
   const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wavefront's 64 x 64 corner
   const int lr = lane & 31, lk = lane >> 5;
   const float *A = g.A, *B = g.B;
-  float *C = g.C;
+  float *C = g.C + (long long)blockIdx.y * g.split_stride;
   if (!SUM_BATCHES) {
     A += (long long)blockIdx.z * g.stride_a;
     B += (long long)blockIdx.z * g.stride_b;
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
           float v = acc[a][b][e];
           if (g.bias_i && first) v += g.bias_i[i];
           v += bj;
-          if (g.splits > 1)
+          if (g.splits > 1 && g.split_stride == 0)
             atomicAdd(C + (long long)i * g.ldc + j, v);
           else
             C[(long long)i * g.ldc + j] = v;
@@ -394,6 +395,16 @@ __global__ __launch_bounds__(256) void bn_backward_apply_kernel(float *g, const 
 
 constexpr long long kMaxGridZ = 65535;  // limit of gridDim.z
 
+// dst[i] = shares[0][i] + shares[1][i] + ... in that order (n elements per share).
+__global__ __launch_bounds__(256) void sum_shares_kernel(const float *__restrict__ shares, int count, long long n,
+                                                         float *dst) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    float v = shares[i];
+    for (int s = 1; s < count; ++s) v += shares[(long long)s * n + i];
+    dst[i] = v;
+  }
+}
+
 bool aligned16(const void *p, long long ld, long long stride) {
   return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0 && stride % 4 == 0;
 }
@@ -402,7 +413,7 @@ template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS, bool SUM_BATCHES>
 int launch_gemm_batched(const float *A, long long lda, long long stride_a, const float *B, long long ldb,
                         long long stride_b, float *C, long long ldc, long long stride_c, long long n_i, long long n_j,
                         long long n_r, long long batches, double *stats, const float *bias_i, const float *bias_j,
-                        hipStream_t stream, bool allow_split = false) {
+                        hipStream_t stream, bool allow_split = false, float *partials = nullptr, int ordered_splits = 0) {
   if (n_i <= 0 || n_j <= 0 || batches <= 0) return HT_OK;
   if (!SUM_BATCHES && batches > kMaxGridZ) {
     // one result per batch rides on blockIdx.z: longer batch lists go out in several launches
@@ -434,7 +445,24 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
   // would leave most of the device idle: the reduction is then split over blockIdx.y and the shares are added into
   // the zeroed result with float atomics (a few thousand elements times the number of shares).
   g.splits = 1;
+  g.split_stride = 0;
   const long long all_steps = SUM_BATCHES ? per_batch * batches : per_batch;
+  if (ordered_splits > 1 && partials != nullptr && !STATS && ldc == n_j && batches == 1 && !bias_i && !bias_j) {
+    // reproducible form of the split: every share stores its partial result, and the shares are added in a fixed order
+    g.splits = ordered_splits;
+    g.split_stride = n_i * n_j;
+    g.C = partials;
+    hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES>),
+                       dim3((unsigned)slots, (unsigned)g.splits, 1u), dim3(kGemmThreads), 0, stream, g);
+    HT_LAUNCH_CHECK("matrix product (matrix cores, split reduction)");
+    const long long chunk = (all_steps + g.splits - 1) / g.splits;
+    const int filled = int((all_steps + chunk - 1) / chunk);  // shares that had steps to do (the others wrote nothing)
+    const long long n = n_i * n_j;
+    hipLaunchKernelGGL(sum_shares_kernel, dim3((unsigned)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192)), dim3(256), 0,
+                       stream, partials, filled, n, C);
+    HT_LAUNCH_CHECK("matrix product (sum of the shares)");
+    return HT_OK;
+  }
   if (allow_split && !STATS && ldc == n_j && (SUM_BATCHES || batches == 1) && gi * gj < kNumCUs && all_steps >= 64) {
     long long want = (2 * kNumCUs + gi * gj - 1) / (gi * gj);
     if (want > all_steps / 16) want = all_steps / 16;
@@ -473,6 +501,28 @@ int gemm_tile_map(int tiles_i, int tiles_j, int *tile_i, int *tile_j) {
 
 size_t projection_workspace(long long N) { return align_up(size_t(2) * size_t(N) * sizeof(double), 256); }
 
+// Shares of the reduction of a product with rows x cols results over `red` terms (1: no split). Few result tiles and
+// a long reduction only.
+int reduction_shares(long long rows, long long cols, long long red) {
+  const long long tiles = ((rows + kTile - 1) / kTile) * ((cols + kTile - 1) / kTile), steps = (red + kRed - 1) / kRed;
+  if (tiles <= 0 || tiles >= kNumCUs / 2 || steps < 64) return 1;
+  long long want = (2 * kNumCUs + tiles - 1) / tiles;
+  if (want > steps / 16) want = steps / 16;
+  return want > 1 ? int(want) : 1;
+}
+// dLin [N x K] reduces over the batch, dX [B x K] over the N columns; the two products run one after the other and
+// share the area for their partial results.
+size_t shares_bytes(long long B, long long K, long long N) {
+  const int s_lin = reduction_shares(N, K, B), s_x = reduction_shares(B, K, N);
+  const size_t lin = s_lin > 1 ? size_t(s_lin) * size_t(N) * size_t(K) * sizeof(float) : 0;
+  const size_t dx = s_x > 1 ? size_t(s_x) * size_t(B) * size_t(K) * sizeof(float) : 0;
+  return lin > dx ? lin : dx;
+}
+
+size_t projection_backward_workspace(long long B, long long K, long long N) {
+  return projection_workspace(N) + shares_bytes(B, K, N);
+}
+
 // zhat [B x N] = normalised (x [B x K] * lin [N x K]^T); mean, rstd, var [N] out; ws: projection_workspace(N).
 int projection_forward(long long B, long long K, long long N, const float *x, const float *lin, double eps,
                        float *zhat, float *mean, float *rstd, float *var, void *ws, hipStream_t stream) {
@@ -506,10 +556,20 @@ int projection_backward(long long B, long long K, long long N, const float *x, c
   HT_LAUNCH_CHECK("batch-norm backward (sums)");
   hipLaunchKernelGGL(bn_backward_apply_kernel, grid, dim3(256), 0, stream, g, zhat, B, int(N), rstd, sums);
   HT_LAUNCH_CHECK("batch-norm backward");
-  // dlin[n, k] = sum_b g[b, n] * x[b, k]: both operands row contiguous, reduction over the batch
-  if (dlin && (rc = launch_gemm<false, false, false>(g, N, x, K, dlin, K, N, K, B, nullptr, stream)) != HT_OK) return rc;
-  // dx[b, k] = sum_n g[b, n] * lin[n, k]: g has the reduction index n contiguous, lin the row index k
-  if (dx && (rc = launch_gemm<true, false, false>(g, N, lin, K, dx, K, B, K, N, nullptr, stream)) != HT_OK) return rc;
+  // dlin[n, k] = sum_b g[b, n] * x[b, k]: both operands row contiguous, reduction over the batch. A small layer under a
+  // large batch has a handful of result tiles and a long reduction: it is then split over workgroups whose shares are
+  // summed in a fixed order (reproducible, unlike a split that meets in atomics).
+  float *partials = reinterpret_cast<float *>(static_cast<unsigned char *>(ws) + projection_workspace(N));
+  if (dlin && (rc = launch_gemm_batched<false, false, false, false>(g, N, 0, x, K, 0, dlin, K, 0, N, K, B, 1, nullptr,
+                                                                     nullptr, nullptr, stream, false, partials,
+                                                                     reduction_shares(N, K, B))) != HT_OK)
+    return rc;
+  // dx[b, k] = sum_n g[b, n] * lin[n, k]: g has the reduction index n contiguous, lin the row index k (split the same
+  // way where a small batch meets a wide layer)
+  if (dx && (rc = launch_gemm_batched<true, false, false, false>(g, N, 0, lin, K, 0, dx, K, 0, B, K, N, 1, nullptr,
+                                                                  nullptr, nullptr, stream, false, partials,
+                                                                  reduction_shares(B, K, N))) != HT_OK)
+    return rc;
   return HT_OK;
 }
 

@@ -358,7 +358,7 @@ def linear_bn_backward(inData, bInDataGrad, inLinearWeights, bInLinearWeightsGra
     with torch.cuda.device(inData.device):
         dx = torch.empty_like(inData) if bInDataGrad else None
         dlin = torch.empty_like(inLinearWeights) if bInLinearWeightsGrad else None
-        nbytes = lib.ht_projection_workspace(N)
+        nbytes = lib.ht_projection_backward_workspace(B, K, N)
         ws = _workspace(nbytes, inData.device)
         L.check(lib.ht_projection_backward(B, K, N, _ptr(inData), _ptr(inLinearWeights), _ptr(zhat), _ptr(rstd),
                                            _ptr(outDataGrad), _ptr(dlin), _ptr(dx), _ptr(ws), nbytes,

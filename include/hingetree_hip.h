@@ -166,8 +166,11 @@ int ht_conv_backward(const ht_conv_shape *s, const void *x, const void *thr, con
  *             the caller's running statistics; may be NULL).
  *   backward: g [B, N] holds dL/dzhat on entry and is overwritten with dL/dz; dlin [N, K] and dx [B, K] receive the
  *             parameter / input gradients (either may be NULL).
- * workspace: ht_projection_workspace(N) bytes. */
+ * workspace: ht_projection_workspace(N) bytes for the forward pass, ht_projection_backward_workspace(B, K, N) for the
+ * backward pass (a small layer under a large batch splits the batch reduction of dlin over workgroups and sums their
+ * shares in a fixed order, so the result does not depend on scheduling). */
 size_t ht_projection_workspace(int64_t N);
+size_t ht_projection_backward_workspace(int64_t B, int64_t K, int64_t N);
 int ht_projection_forward(int64_t B, int64_t K, int64_t N, const float *x, const float *lin, double eps, float *zhat,
                           float *mean, float *rstd, float *var, void *workspace, size_t workspace_bytes, void *stream);
 int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, const float *lin, const float *zhat,

@@ -55,6 +55,28 @@ def test_projection_forward_backward(dev, shape):
     assert only[0] is None and rel_err(only[1].cpu().double(), rdlin) <= 2e-5 * scale
 
 
+@pytest.mark.parametrize("shape", [(40000, 48, 300), (192, 40, 9000)], ids=["small layer, large batch", "wide layer, small batch"])
+def test_split_reductions(dev, shape):
+    """A small layer under a large batch: dLin has three result tiles and a reduction over 40 000 rows; a wide layer
+    under a small batch: dX has two result tiles and a reduction over 9000 columns. Either reduction is split over
+    workgroups whose shares are summed in a fixed order -- checked against fp64 and for bit-identical repeats."""
+    B, K, N = shape
+    g = torch.Generator().manual_seed(12)
+    x = torch.rand([B, K], generator=g)
+    lin = torch.randn([N, K], generator=g) / K ** 0.5
+    up = torch.randn([B, N], generator=g)
+    zhat, mean, rstd, var = ops.linear_bn_forward(x.to(dev), lin.to(dev), 1e-5)
+    rz, rmean, rrstd, rvar = _reference(x, lin, 1e-5)
+    gd = up.double()
+    dz = rrstd * (gd - gd.mean(0) - rz * (gd * rz).mean(0))
+    rdlin, rdx = dz.t() @ x.double(), dz @ lin.double()
+    runs = [ops.linear_bn_backward(x.to(dev), True, lin.to(dev), True, zhat, rstd, up.to(dev).clone()) for _ in range(2)]
+    assert torch.equal(runs[0][1], runs[1][1]) and torch.equal(runs[0][0], runs[1][0])
+    scale = max(float(rrstd.abs().max()), 1.0)
+    assert rel_err(runs[0][1].cpu().double(), rdlin) <= 2e-5 * scale
+    assert rel_err(runs[0][0].cpu().double(), rdx) <= 2e-5 * scale
+
+
 def test_projection_rejects_bad_input(dev):
     x = torch.rand([4, 3], device=dev)
     lin = torch.rand([5, 2], device=dev)
