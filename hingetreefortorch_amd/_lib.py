@@ -69,6 +69,10 @@ SIGNATURES = {
     "ht_tree_mix_backward_f64": (_I, [ctypes.c_int64] * 4 + [_P, _P, _P, _P, _P, _P]),
     "ht_contract": (_I, [ctypes.POINTER(TileShape), _P, _P, _P]),
     "ht_expand": (_I, [ctypes.POINTER(TileShape), _P, _P, _P]),
+    "ht_tree_mix_backward_workspace": (_SZ, [ctypes.c_int64] * 4),
+    "ht_tree_mix_backward_ws": (_I, [ctypes.c_int64] * 4 + [_P, _P, _P, _P, _P, ctypes.c_int32, _P, _SZ, _P]),
+    "ht_rows_to_planes": (_I, [ctypes.c_int64, ctypes.c_int64, _P, _P, _P]),
+    "ht_planes_to_rows": (_I, [ctypes.c_int64, ctypes.c_int64, _P, _P, _P]),
     "ht_projection_workspace": (_SZ, [ctypes.c_int64]),
     "ht_projection_backward_workspace": (_SZ, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]),
     "ht_projection_forward": (_I, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _P, _P, ctypes.c_double, _P, _P, _P,

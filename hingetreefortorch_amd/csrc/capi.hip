@@ -464,6 +464,31 @@ int ht_tree_mix_backward(int64_t B, int64_t T, int64_t O, int64_t R, const float
   return mix_backward(B, T, O, R, f, lin, g, h, dlin, deterministic != 0, static_cast<hipStream_t>(stream));
 }
 
+size_t ht_tree_mix_backward_workspace(int64_t B, int64_t T, int64_t O, int64_t R) {
+  return (B < 0 || T < 0 || O < 0 || R < 0) ? 0 : mix_backward_workspace(B, T, O, R);
+}
+
+int ht_tree_mix_backward_ws(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin, const float *g,
+                            float *h, float *dlin, int deterministic, void *workspace, size_t workspace_bytes,
+                            void *stream) {
+  if (B < 0 || T < 0 || O < 0 || R < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if (B * O * R > 0 && (!g || (h && !lin) || (dlin && !f))) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return mix_backward(B, T, O, R, f, lin, g, h, dlin, deterministic != 0, static_cast<hipStream_t>(stream), workspace,
+                      workspace_bytes);
+}
+
+int ht_rows_to_planes(int64_t n, int64_t R, const float *rows, float *planes, void *stream) {
+  if (n < 0 || R < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if (n > 0 && R > 0 && (!rows || !planes)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return rows_to_planes(n, R, rows, planes, false, static_cast<hipStream_t>(stream));
+}
+
+int ht_planes_to_rows(int64_t n, int64_t R, const float *planes, float *rows, void *stream) {
+  if (n < 0 || R < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");
+  if (n > 0 && R > 0 && (!rows || !planes)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  return rows_to_planes(n, R, planes, rows, true, static_cast<hipStream_t>(stream));
+}
+
 int ht_tree_mix_forward_f64(int64_t B, int64_t T, int64_t O, int64_t R, const double *f, const double *lin,
                             const double *bias, double *out, void *stream) {
   if (B < 0 || T < 0 || O < 0 || R < 0) return fail(HT_ERR_INVALID_ARGUMENT, "Error: negative tensor size.");

@@ -152,10 +152,12 @@ int mix_backward_f64(long long B, long long T, long long O, long long R, const d
                      const double *g, double *h, double *dlin, hipStream_t stream);
 
 // Linear mix over the tree axis behind a forest (projection.hip), fp32.
+int rows_to_planes(long long n, long long R, const float *rows, float *planes, bool back, hipStream_t stream);
 int mix_forward(long long B, long long T, long long O, long long R, const float *f, const float *lin,
                 const float *bias, float *out, hipStream_t stream);
+size_t mix_backward_workspace(long long B, long long T, long long O, long long R);
 int mix_backward(long long B, long long T, long long O, long long R, const float *f, const float *lin, const float *g,
-                 float *h, float *dlin, bool deterministic, hipStream_t stream);
+                 float *h, float *dlin, bool deterministic, hipStream_t stream, void *ws = nullptr, size_t ws_bytes = 0);
 
 // Tile <-> image permutation (expand.hip).
 int tile_contract(const ht_tile_shape *s, const void *in, void *out, hipStream_t stream);

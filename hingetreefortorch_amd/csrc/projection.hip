@@ -578,6 +578,33 @@ int projection_backward(long long B, long long K, long long N, const float *x, c
 //   forward : out[b, o, r] = bias[o] + sum_t lin[o, t] * f[b, t, r]
 //   backward: h[b, t, r] = sum_o lin[o, t] * g[b, o, r]   (the upstream gradient of the forest)
 //             dlin[o, t] = sum_{b, r} g[b, o, r] * f[b, t, r]
+// rows [n][R] (the R values of a row contiguous) -> planes [R][n], and back. A thread takes a row: its R values are
+// read (written) one after the other -- neighbouring threads' rows are neighbours in memory, so the lines are used
+// whole -- and each plane is written (read) with consecutive threads on consecutive addresses.
+__global__ __launch_bounds__(256) void rows_to_planes_kernel(long long n, int R, const float *__restrict__ rows,
+                                                             float *__restrict__ planes) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    for (int r = 0; r < R; ++r) planes[(long long)r * n + i] = rows[i * R + r];
+}
+__global__ __launch_bounds__(256) void planes_to_rows_kernel(long long n, int R, const float *__restrict__ planes,
+                                                             float *__restrict__ rows) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    for (int r = 0; r < R; ++r) rows[i * R + r] = planes[(long long)r * n + i];
+}
+
+int rows_to_planes(long long n, long long R, const float *rows, float *planes, bool back, hipStream_t stream) {
+  if (n <= 0 || R <= 0) return HT_OK;
+  if (R > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: rows too long for this build.");
+  long long blocks = (n + 255) / 256;
+  if (blocks > 32 * kNumCUs) blocks = 32 * kNumCUs;
+  if (back)
+    hipLaunchKernelGGL(planes_to_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, n, int(R), rows, planes);
+  else
+    hipLaunchKernelGGL(rows_to_planes_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, n, int(R), rows, planes);
+  HT_LAUNCH_CHECK("rows <-> planes");
+  return HT_OK;
+}
+
 int mix_forward(long long B, long long T, long long O, long long R, const float *f, const float *lin,
                 const float *bias, float *out, hipStream_t stream) {
   if (R == 1)  // out [B x O] = f [B x T] * lin [O x T]^T, bias per column
@@ -588,8 +615,15 @@ int mix_forward(long long B, long long T, long long O, long long R, const float 
                                                         nullptr, stream);
 }
 
+// Area for the shares of the reproducible split of dLin's reduction (R == 1: one product reducing over the samples).
+size_t mix_backward_workspace(long long B, long long T, long long O, long long R) {
+  if (R != 1) return 0;
+  const int shares = reduction_shares(O, T, B);
+  return shares > 1 ? size_t(shares) * size_t(O) * size_t(T) * sizeof(float) : 0;
+}
+
 int mix_backward(long long B, long long T, long long O, long long R, const float *f, const float *lin, const float *g,
-                 float *h, float *dlin, bool deterministic, hipStream_t stream) {
+                 float *h, float *dlin, bool deterministic, hipStream_t stream, void *ws, size_t ws_bytes) {
   int rc;
   if (h) {
     if (R == 1)  // h [B x T] = g [B x O] * lin [O x T]
@@ -602,9 +636,14 @@ int mix_backward(long long B, long long T, long long O, long long R, const float
   }
   if (dlin && (B == 0 || R == 0)) return zero_fill(dlin, size_t(O) * size_t(T) * sizeof(float), stream);
   if (dlin) {
-    if (R == 1)  // dlin [O x T] = g^T [O x B] * f [B x T]
+    if (R == 1) {  // dlin [O x T] = g^T [O x B] * f [B x T]
+      // deterministic mode with a workspace: shares of the reduction summed in a fixed order instead of one long pass
+      const bool ordered = deterministic && ws != nullptr && ws_bytes >= mix_backward_workspace(B, T, O, R);
       rc = launch_gemm_batched<false, false, false, false>(g, O, 0, f, T, 0, dlin, T, 0, O, T, B, 1, nullptr, nullptr,
-                                                           nullptr, stream, !deterministic);
+                                                           nullptr, stream, !deterministic,
+                                                           ordered ? static_cast<float *>(ws) : nullptr,
+                                                           ordered ? reduction_shares(O, T, B) : 0);
+    }
     else  // dlin [O x T] = sum_b g_b [O x R] * f_b [T x R]^T
       rc = launch_gemm_batched<true, true, false, true>(g, R, O * R, f, R, T * R, dlin, T, 0, O, T, R, B, nullptr,
                                                         nullptr, nullptr, stream, !deterministic);

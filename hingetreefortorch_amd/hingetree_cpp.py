@@ -143,11 +143,29 @@ def _fused_linear_forward(kind, inData, inThresholds, inOrdinals, inWeights, inL
     else:
         f = _forward(kind, inData, inThresholds, inOrdinals, inWeights)
     B, T, O, R, out_sizes = _mix_sizes(inData, inWeights, inLinearWeights)
+    lib = L.load()
     with torch.cuda.device(inData.device):
         out = torch.empty(out_sizes, dtype=inData.dtype, device=inData.device)
-        mix = L.load().ht_tree_mix_forward if inData.dtype == torch.float32 else L.load().ht_tree_mix_forward_f64
-        L.check(mix(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(inLinearBias), _ptr(out), _stream(inData.device)))
+        stream = _stream(inData.device)
+        if _mix_in_planes(inData.dtype, B, R):
+            # few values per (sample, tree): as planes they are R times as many samples of one product
+            planes = torch.empty(R * B * T, dtype=inData.dtype, device=inData.device)
+            mixed = torch.empty(R * B * O, dtype=inData.dtype, device=inData.device)
+            L.check(lib.ht_rows_to_planes(B * T, R, _ptr(f), _ptr(planes), stream))
+            L.check(lib.ht_tree_mix_forward(R * B, T, O, 1, _ptr(planes), _ptr(inLinearWeights), _ptr(inLinearBias),
+                                            _ptr(mixed), stream))
+            L.check(lib.ht_planes_to_rows(B * O, R, _ptr(mixed), _ptr(out), stream))
+        else:
+            mix = lib.ht_tree_mix_forward if inData.dtype == torch.float32 else lib.ht_tree_mix_forward_f64
+            L.check(mix(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(inLinearBias), _ptr(out), stream))
     return (out, f, records) if keep else out
+
+
+def _mix_in_planes(dtype, B, R):
+    """Whether the float32 mix moves its operands to planes first: with R values per (sample, tree) the product per
+    sample has results of O x R, a sliver of a 128 x 128 matrix-core tile, while the R slices taken as samples make one
+    product of B * R rows."""
+    return dtype == torch.float32 and 1 < R < 128 and B > 1
 
 
 def _fused_linear_backward(kind, mode, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals,
@@ -174,10 +192,29 @@ def _fused_linear_backward(kind, mode, inData, bInDataGrad, inThresholds, bInThr
                         device=inData.device) if need_forest else None
         dlin = torch.empty_like(inLinearWeights) if bInLinearWeightsGrad else None
         if h is not None or dlin is not None:
-            if inData.dtype == torch.float32:
-                L.check(lib.ht_tree_mix_backward(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(outDataGrad), _ptr(h),
-                                                 _ptr(dlin), int(mode == L.HT_BACKWARD_DETERMINISTIC),
-                                                 _stream(inData.device)))
+            if _mix_in_planes(inData.dtype, B, R):
+                stream = _stream(inData.device)
+                dev = inData.device
+                g_planes = torch.empty(R * B * O, dtype=inData.dtype, device=dev)
+                L.check(lib.ht_rows_to_planes(B * O, R, _ptr(outDataGrad), _ptr(g_planes), stream))
+                f_planes = None
+                if dlin is not None:
+                    f_planes = torch.empty(R * B * T, dtype=inData.dtype, device=dev)
+                    L.check(lib.ht_rows_to_planes(B * T, R, _ptr(f), _ptr(f_planes), stream))
+                h_planes = torch.empty(R * B * T, dtype=inData.dtype, device=dev) if h is not None else None
+                nbytes = lib.ht_tree_mix_backward_workspace(R * B, T, O, 1)
+                ws = _workspace(nbytes, dev)
+                L.check(lib.ht_tree_mix_backward_ws(R * B, T, O, 1, _ptr(f_planes), _ptr(inLinearWeights), _ptr(g_planes),
+                                                    _ptr(h_planes), _ptr(dlin), int(mode == L.HT_BACKWARD_DETERMINISTIC),
+                                                    _ptr(ws), nbytes, stream))
+                if h is not None:
+                    L.check(lib.ht_planes_to_rows(B * T, R, _ptr(h_planes), _ptr(h), stream))
+            elif inData.dtype == torch.float32:
+                nbytes = lib.ht_tree_mix_backward_workspace(B, T, O, R)
+                ws = _workspace(nbytes, inData.device)
+                L.check(lib.ht_tree_mix_backward_ws(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(outDataGrad),
+                                                    _ptr(h), _ptr(dlin), int(mode == L.HT_BACKWARD_DETERMINISTIC),
+                                                    _ptr(ws), nbytes, _stream(inData.device)))
             else:  # float64: plain kernels with a fixed summation order in either mode
                 L.check(lib.ht_tree_mix_backward_f64(B, T, O, R, _ptr(f), _ptr(inLinearWeights), _ptr(outDataGrad),
                                                      _ptr(h), _ptr(dlin), _stream(inData.device)))

@@ -200,6 +200,21 @@ int ht_tree_mix_forward(int64_t B, int64_t T, int64_t O, int64_t R, const float 
 int ht_tree_mix_backward(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin, const float *g,
                          float *h, float *dlin, int deterministic, void *stream);
 
+/* ht_tree_mix_backward with a workspace (ht_tree_mix_backward_workspace bytes; may be NULL / 0): in deterministic
+ * mode the reduction of dlin over the samples (R == 1) is then split over workgroups whose shares are summed in a
+ * fixed order, instead of running as one long reproducible pass. No counterpart in the reference. */
+size_t ht_tree_mix_backward_workspace(int64_t B, int64_t T, int64_t O, int64_t R);
+int ht_tree_mix_backward_ws(int64_t B, int64_t T, int64_t O, int64_t R, const float *f, const float *lin, const float *g,
+                            float *h, float *dlin, int deterministic, void *workspace, size_t workspace_bytes,
+                            void *stream);
+
+/* Helpers for the mix with a few values per (sample, tree) (R = 2 ... ~100: extra outputs of a tabular forest), no
+ * counterpart in the reference: rows [n][R] <-> planes [R][n]. With f, g, out and h moved to planes, the R slices are
+ * R times as many samples of an R = 1 problem, and ht_tree_mix_forward / _backward serve them as ONE product with
+ * B * R rows instead of B products whose results fill a sliver of a matrix-core tile each. */
+int ht_rows_to_planes(int64_t n, int64_t R, const float *rows, float *planes, void *stream);
+int ht_planes_to_rows(int64_t n, int64_t R, const float *planes, float *rows, void *stream);
+
 /* The same three products for float64 data (the reference instantiates its fused-linear operators for double as well,
  * hingetree_fused_linear.cpp:798-806,845-853): plain kernels with a fixed summation order, always reproducible. */
 int ht_tree_mix_forward_f64(int64_t B, int64_t T, int64_t O, int64_t R, const double *f, const double *lin,
