@@ -1255,7 +1255,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_wide_kernel(ForestDims d,
 // dThr[t, v] = sum over samples with selected vertex v of -c. One workgroup per tree (x sample parts); where a tree's
 // vertex table does not fit LDS (depth 15 and more), `vslices` workgroups per tree, each owning a range of vertices
 // and passing over all of the tree's records.
-template <typename Real, bool COMPACT, bool FIXED>
+template <typename Real, bool COMPACT, bool FIXED, bool SLICED>
 __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dthr,
                                                    unsigned long long *dthr_fixed, const DetHeader *hdr,
                                                    long long part_size, bool use_atomic, int vslices) {
@@ -1290,7 +1290,7 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
       val = to_fixed(-double(c), scale);
     else
       val = -double(c);
-    if (v - v_begin >= uint32_t(nv)) return;  // another slice's vertex
+    if (SLICED && v - v_begin >= uint32_t(nv)) return;  // another slice's vertex
     if (v < uint32_t(kTop)) {
 #pragma unroll
       for (int k = 0; k < kTop; ++k) top[k] += v == uint32_t(k) ? val : Acc(0);
@@ -1346,7 +1346,7 @@ __global__ __launch_bounds__(256) void dthr_kernel(ForestDims d, Records<Real, C
 // FIXED: 64-bit fixed-point cells; dX is cleared beforehand and left alone when the header asks for the fallback.
 // A feature space too wide for the tile is served in windows of f_per features (blockIdx.y): every window passes
 // over all records of the tile's samples and keeps the terms whose ordinal falls inside it.
-template <typename Real, int BT, bool COMPACT, bool FIXED>
+template <typename Real, int BT, bool COMPACT, bool FIXED, bool WINDOWED>
 __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Records<Real, COMPACT> rec, Real *dx,
                                                             const DetHeader *hdr, int f_per) {
   typedef typename std::conditional<FIXED, unsigned long long, Real>::type Acc;
@@ -1361,8 +1361,8 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
     scale = hdr->scale_c;
     inv_scale = hdr->inv_scale_c;
   }
-  const uint32_t f_begin = blockIdx.y * uint32_t(f_per);
-  const uint32_t nf = uint32_t(min(f_per, d.F - int(f_begin)));  // this workgroup's features [f_begin, f_begin + nf)
+  const uint32_t f_begin = WINDOWED ? blockIdx.y * uint32_t(f_per) : 0u;
+  const uint32_t nf = WINDOWED ? uint32_t(min(f_per, d.F - int(f_begin))) : uint32_t(d.F);  // features [f_begin, f_begin + nf)
   for (int i = threadIdx.x; i < int(nf) * LD; i += NT) acc[i] = Acc(0);
   __syncthreads();
   const long long s0 = (long long)blockIdx.x * BT;
@@ -1401,7 +1401,7 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const uint32_t o = (av[i][e] >> rec.oshift) - f_begin;
-              if (o >= nf) continue;
+              if (WINDOWED && o >= nf) continue;
               if (FIXED)
                 atomicAdd(reinterpret_cast<unsigned long long *>(acc) + o * LD + jq + e,
                           to_fixed(double(cv[i][e]), scale));
@@ -1429,7 +1429,7 @@ __global__ __launch_bounds__(kForestThreads) void dx_kernel(ForestDims d, Record
 #pragma unroll
       for (int i = 0; i < kBatch; ++i) {
         if (t0 + i * TC >= d.T) break;
-        if (o[i] >= nf) continue;
+        if (WINDOWED && o[i] >= nf) continue;
         if (FIXED)
           atomicAdd(reinterpret_cast<unsigned long long *>(acc) + o[i] * LD + j, to_fixed(double(cv[i]), scale));
         else
@@ -1952,7 +1952,11 @@ int launch_dx(const ForestDims &d, Records<Real, COMPACT> rec, Real *dx, const D
   const size_t lds = size_t(f_per) * cell;
   const long long tiles = (d.S + BT - 1) / BT;
   if (tiles > 0x7fffffffLL || windows > 65535) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
-  auto kernel = dx_kernel<Real, BT, COMPACT, FIXED>;
+  auto kernel = dx_kernel<Real, BT, COMPACT, FIXED, false>;
+  if constexpr (BT == 8) {  // (windows are only ever needed on the smallest tile)
+    if (windows > 1) kernel = dx_kernel<Real, BT, COMPACT, FIXED, true>;
+  }
+  if (BT != 8 && windows > 1) return fail(HT_ERR_RUNTIME, "Error: feature windows on a tile other than the smallest.");
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)windows), dim3(kForestThreads), lds, stream, d, rec, dx, hdr,
@@ -2127,7 +2131,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
     const int vslices = int((size_t(d.V) * sizeof(double) + size_t(kLdsBytes) - 1) / size_t(kLdsBytes));
     const size_t thr_lds = size_t((d.V + vslices - 1) / vslices) * sizeof(double);
     if ((long long)d.T * vslices > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many trees for one launch.");
-    auto thr_kernel = dthr_kernel<Real, COMPACT, FIXED>;
+    auto thr_kernel = vslices > 1 ? dthr_kernel<Real, COMPACT, FIXED, true> : dthr_kernel<Real, COMPACT, FIXED, false>;
     HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(thr_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(thr_lds)));
     hipLaunchKernelGGL(thr_kernel, dim3((unsigned)(d.T * vslices), (unsigned)dthr_gy), dim3(256), thr_lds, stream, d,
