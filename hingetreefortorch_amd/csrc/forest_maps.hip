@@ -10,7 +10,8 @@ __global__ __launch_bounds__(kForestThreads) void maps_kernel(ForestDims d, cons
                                                               const Real *__restrict__ thr,
                                                               const int64_t *__restrict__ ord, int64_t *leafmap,
                                                               Real *margins, int64_t *ordinals,
-                                                              unsigned long long *reach, int trees_per_block) {
+                                                              unsigned long long *reach, uint16_t *keys,
+                                                              int trees_per_block) {
   constexpr int NT = kForestThreads;
   constexpr int TC = NT / BT;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -40,13 +41,58 @@ __global__ __launch_bounds__(kForestThreads) void maps_kernel(ForestDims d, cons
     if (leafmap) leafmap[at] = (int64_t)r.key;
     if (margins) margins[at] = r.margin;
     if (ordinals) ordinals[at] = od[r.vertex];
-    if (reach) atomicAdd(reach + (long long)t * d.L + r.key, 1ull);
+    if (keys)
+      keys[(long long)t * d.S + s] = (uint16_t)r.key;
+    else if (reach)
+      atomicAdd(reach + (long long)t * d.L + r.key, 1ull);
   }
+}
+
+// Reachability as a histogram: the walk stores each pair's 16-bit leaf key tree-major, and here one workgroup counts a
+// stretch of one tree's keys in LDS and adds its non-zero counters to the tree's row. A global atomic per pair, the
+// other way to count, runs several times longer once a launch holds millions of pairs.
+constexpr int kReachThreads = 256;
+
+__global__ __launch_bounds__(kReachThreads) void reach_histogram_kernel(const uint16_t *__restrict__ keys, long long S,
+                                                                        int L, long long per_part,
+                                                                        unsigned long long *reach) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint32_t *count = reinterpret_cast<uint32_t *>(smem);
+  for (int l = threadIdx.x; l < L; l += kReachThreads) count[l] = 0u;
+  __syncthreads();
+  const int t = blockIdx.x;
+  const uint16_t *row = keys + (long long)t * S;
+  const long long s0 = (long long)blockIdx.y * per_part;
+  const long long s1 = s0 + per_part < S ? s0 + per_part : S;
+  if ((S & 7) == 0) {  // per_part is a multiple of 8, so every stretch of every tree starts on 16 bytes
+    for (long long s = s0 + threadIdx.x * 8; s < s1; s += kReachThreads * 8) {
+      const uint4 v = *reinterpret_cast<const uint4 *>(row + s);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        atomicAdd(count + (w[i] & 0xffffu), 1u);
+        atomicAdd(count + (w[i] >> 16), 1u);
+      }
+    }
+  } else {
+    for (long long s = s0 + threadIdx.x; s < s1; s += kReachThreads) atomicAdd(count + row[s], 1u);
+  }
+  __syncthreads();
+  unsigned long long *dst = reach + (long long)t * L;
+  for (int l = threadIdx.x; l < L; l += kReachThreads) {
+    const uint32_t c = count[l];
+    if (c) atomicAdd(dst + l, (unsigned long long)c);
+  }
+}
+
+// The histogram needs 16-bit keys and a tree's counters in LDS, and pays off once there are enough pairs.
+inline bool reach_by_histogram(const ForestDims &d) {
+  return d.L <= 65536 && size_t(d.L) * 4 <= kLdsBytes && d.S * (long long)d.T >= (1 << 16);
 }
 
 template <typename Real, bool FERN, int BT, bool XLDS>
 int launch_maps(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap, Real *margins,
-                int64_t *ordinals, int64_t *reach, hipStream_t stream) {
+                int64_t *ordinals, int64_t *reach, uint16_t *keys, hipStream_t stream) {
   constexpr int TC = kForestThreads / BT;
   const size_t lds = XLDS ? size_t(d.F) * BT * sizeof(Real) : 0;
   const long long tiles = (d.S + BT - 1) / BT;
@@ -60,20 +106,21 @@ int launch_maps(const ForestDims &d, const Real *x, const Real *thr, const int64
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    int(lds)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, thr, ord,
-                     leafmap, margins, ordinals, reinterpret_cast<unsigned long long *>(reach), trees_per_block);
+                     leafmap, margins, ordinals, reinterpret_cast<unsigned long long *>(reach), keys,
+                     trees_per_block);
   HT_LAUNCH_CHECK("forest maps");
   return HT_OK;
 }
 
 template <typename Real, bool FERN>
 int dispatch_maps(const ForestDims &d, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap,
-                  Real *margins, int64_t *ordinals, int64_t *reach, hipStream_t stream) {
+                  Real *margins, int64_t *ordinals, int64_t *reach, uint16_t *keys, hipStream_t stream) {
   switch (pick_tile<Real>(d.F, 1024)) {
-    case 64: return launch_maps<Real, FERN, 64, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
-    case 32: return launch_maps<Real, FERN, 32, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
-    case 16: return launch_maps<Real, FERN, 16, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
-    case 8: return launch_maps<Real, FERN, 8, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
-    default: return launch_maps<Real, FERN, 64, false>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
+    case 64: return launch_maps<Real, FERN, 64, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream);
+    case 32: return launch_maps<Real, FERN, 32, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream);
+    case 16: return launch_maps<Real, FERN, 16, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream);
+    case 8: return launch_maps<Real, FERN, 8, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream);
+    default: return launch_maps<Real, FERN, 64, false>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream);
   }
 }
 
@@ -146,19 +193,42 @@ int ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, hipStream_t st
   return HT_OK;
 }
 
+// Bytes that let reachability run as a histogram; the call works without them, slower.
 template <typename Real>
-size_t forest_maps_workspace(const ForestDims &) {
-  return 0;
+size_t forest_maps_workspace(const ForestDims &d) {
+  return reach_by_histogram(d) ? size_t(d.S) * d.T * sizeof(uint16_t) : 0;
 }
 
 template <typename Real>
 int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap,
-                Real *margins, int64_t *ordinals, int64_t *reach, void *, size_t, hipStream_t stream) {
+                Real *margins, int64_t *ordinals, int64_t *reach, void *workspace, size_t workspace_bytes,
+                hipStream_t stream) {
   int rc;
   if (reach && (rc = zero_fill(reach, size_t(d.T) * d.L * sizeof(int64_t), stream)) != HT_OK) return rc;
   if (d.S == 0 || d.T == 0) return HT_OK;
-  return fern ? dispatch_maps<Real, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream)
-              : dispatch_maps<Real, false>(d, x, thr, ord, leafmap, margins, ordinals, reach, stream);
+  uint16_t *keys = nullptr;
+  if (reach && workspace && reach_by_histogram(d) && workspace_bytes >= size_t(d.S) * d.T * sizeof(uint16_t) &&
+      (reinterpret_cast<uintptr_t>(workspace) & 15) == 0)
+    keys = static_cast<uint16_t *>(workspace);
+  rc = fern ? dispatch_maps<Real, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream)
+            : dispatch_maps<Real, false>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream);
+  if (rc != HT_OK || !keys) return rc;
+  // enough workgroups to fill the part, each with a stretch of keys that is worth its counter flush
+  long long parts = (2048 + d.T - 1) / d.T;
+  const long long most = (d.S + 4LL * d.L - 1) / (4LL * d.L);
+  if (parts > most) parts = most;
+  if (parts < 1) parts = 1;
+  if (parts > 65535) parts = 65535;
+  long long per_part = (d.S + parts - 1) / parts;
+  per_part = (per_part + 7) / 8 * 8;
+  parts = (d.S + per_part - 1) / per_part;
+  const size_t lds = size_t(d.L) * 4;
+  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(reach_histogram_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
+  hipLaunchKernelGGL(reach_histogram_kernel, dim3((unsigned)d.T, (unsigned)parts), dim3(kReachThreads), lds, stream,
+                     keys, (long long)d.S, d.L, per_part, reinterpret_cast<unsigned long long *>(reach));
+  HT_LAUNCH_CHECK("reachability histogram");
+  return HT_OK;
 }
 
 template size_t forest_maps_workspace<float>(const ForestDims &);

@@ -605,8 +605,12 @@ def _maps(kind, inData, inThresholds, inOrdinals, inWeights, want):
         margins = torch.empty(map_sizes, dtype=inData.dtype, device=dev) if want == "margin" else None
         ordinals = torch.empty(map_sizes, dtype=torch.int64, device=dev) if want == "margin" else None
         reach = torch.empty(list(inWeights.shape[:2]), dtype=torch.int64, device=dev) if want == "reach" else None
-        L.check(L.load().ht_forest_maps(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals),
-                                        _ptr(leaf), _ptr(margins), _ptr(ordinals), _ptr(reach), None, 0, _stream(dev)))
+        lib = L.load()
+        # only reachability has a use for the workspace (leaf keys for its histogram)
+        nbytes = lib.ht_forest_maps_workspace(ctypes.byref(shape)) if want == "reach" else 0
+        ws = _workspace(nbytes, dev)
+        L.check(lib.ht_forest_maps(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals), _ptr(leaf),
+                                   _ptr(margins), _ptr(ordinals), _ptr(reach), _ptr(ws), nbytes, _stream(dev)))
     if want == "leaf":
         return leaf
     if want == "margin":

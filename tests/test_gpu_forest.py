@@ -341,6 +341,29 @@ EMPTY = {"no samples": (0, 5, [], 3, 2, []), "no inner positions": (4, 5, [0], 3
          "no samples, staged sizes": (0, 64, [], 300, 6, [10])}
 
 
+# B, F, K dims, T, depth: launches with 2^16 (sample, tree) pairs and more count reachability as a histogram of 16-bit
+# leaf keys when a tree's counters fit the LDS (depth <= 15); below that, and at depth 16, by one atomic per pair.
+REACH = [(30000, 12, [], 5, 6), (30001, 12, [], 5, 6), (700, 9, [5, 3], 11, 4), (9000, 20, [], 9, 15),
+         (5000, 20, [], 14, 16), (262144, 4, [], 1, 2), (70000, 6, [], 1, 1)]
+
+
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("case", REACH, ids=[f"r{i}" for i in range(len(REACH))])
+def test_reachability_counts(dev, case, fern):
+    B, F, Kd, T, D = case
+    x, thr, ordn, w, _ = make_forest(B, F, Kd, T, D, [1], fern, torch.float32, seed=11)
+    if case == REACH[5]:
+        thr[:] = 1e9                                    # every sample of the batch in the same leaf of each tree
+    ref_reach = ho.maps(x, thr, ordn, w, fern)[3].to(torch.int64)
+    gx, gthr, gord, gw = _gpu(dev, x, thr, ordn, w)
+    pre = "fern_" if fern else "tree_"
+    for _ in range(2):                                  # the workspace of the first call is reused by the second
+        reach = getattr(ops, pre + "reachability")(gx, gthr, gord, gw)
+        assert reach.dtype == torch.int64 and torch.equal(reach.cpu(), ref_reach)
+    if case == REACH[5]:
+        assert int(reach.max()) == B
+
+
 @pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
 @pytest.mark.parametrize("name", sorted(EMPTY))
 def test_empty_inputs(dev, name, fern):
