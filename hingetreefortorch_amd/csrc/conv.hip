@@ -187,71 +187,118 @@ __global__ __launch_bounds__(kConvThreads) void conv_backward_kernel(ConvGeom g,
 // ---------------------------------------------------------------------------------------------------------------
 // tiled kernels for 1 and 2 spatial dims
 // ---------------------------------------------------------------------------------------------------------------
-// A workgroup of 256 threads owns a TY x TX tile of output positions of one image (one thread per position) and keeps
-// the input region that tile reads -- all C channels, zeros where the region leaves the image -- in LDS. The trees of
-// one out channel (C trees) are staged in LDS as (threshold, tile offset of the tap) pairs, so a walk step is two LDS
-// reads and no address arithmetic beyond one add, and the padding needs no test. Every byte of x is read from memory
-// once per tile instead of once per (out channel, vertex visit).
+// A workgroup owns a TZ x TY x TX tile of output positions of one image (one thread per position; TZ = 1 for 1-d and
+// 2-d data, TY = 1 as well for 1-d) and keeps the input region that tile reads -- all C channels, zeros where the region
+// leaves the image -- in LDS. The trees of one out channel (C trees) are staged in LDS as (threshold, tile offset of the
+// tap) pairs, so a walk step is two LDS reads and no address arithmetic beyond one add, and the padding needs no test.
+// Every byte of x is read from memory once per tile instead of once per (out channel, vertex visit).
 struct ConvTile {
-  int H, W, OH, OW;
-  int kh, kw, sy, sx, py, px, dy, dx;
-  int TY, TX, log2_tx;  // output tile, TY * TX == threads of the workgroup
-  int IH, IW, TSZ;      // input region of a tile, TSZ = IH * IW
-  int tiles_y, tiles_x;
+  int D, H, W, OD, OH, OW;
+  int kd, kh, kw, sz, sy, sx, pz, py, px, dz, dy, dx;
+  int TZ, TY, TX, log2_tx, log2_ty;  // output tile, TZ * TY * TX == threads of the workgroup, powers of two
+  int ID, IH, IW, PL, TSZ;           // input region of a tile: PL = IH * IW cells per slice, TSZ = ID * PL
+  int tiles_z, tiles_y, tiles_x;
   int taps;
+  __host__ __device__ long long tiles() const { return (long long)tiles_z * tiles_y * tiles_x; }
+  __host__ __device__ long long positions() const { return (long long)OD * OH * OW; }
 };
 
 static bool make_tile(const ConvGeom &g, ConvTile *t, int threads = kConvThreads) {
-  if (g.nd > 2) return false;
-  const int a = g.nd == 2 ? 0 : -1;  // index of the row dimension, none for 1-d
-  t->H = a < 0 ? 1 : g.size[0];
-  t->OH = a < 0 ? 1 : g.osz[0];
-  t->kh = a < 0 ? 1 : g.ker[0];
-  t->sy = a < 0 ? 1 : g.str[0];
-  t->py = a < 0 ? 0 : g.pad[0];
-  t->dy = a < 0 ? 1 : g.dil[0];
-  const int c = g.nd - 1;
-  t->W = g.size[c];
-  t->OW = g.osz[c];
-  t->kw = g.ker[c];
-  t->sx = g.str[c];
-  t->px = g.pad[c];
-  t->dx = g.dil[c];
+  // the last dimension is x, the one before it y, the one before that z; missing ones have extent 1
+  int size[3] = {1, 1, 1}, osz[3] = {1, 1, 1}, ker[3] = {1, 1, 1}, str[3] = {1, 1, 1}, pad[3] = {0, 0, 0},
+      dil[3] = {1, 1, 1};
+  for (int dd = 0; dd < g.nd; ++dd) {
+    const int at = 3 - g.nd + dd;
+    size[at] = g.size[dd], osz[at] = g.osz[dd], ker[at] = g.ker[dd];
+    str[at] = g.str[dd], pad[at] = g.pad[dd], dil[at] = g.dil[dd];
+  }
+  t->D = size[0], t->H = size[1], t->W = size[2];
+  t->OD = osz[0], t->OH = osz[1], t->OW = osz[2];
+  t->kd = ker[0], t->kh = ker[1], t->kw = ker[2];
+  t->sz = str[0], t->sy = str[1], t->sx = str[2];
+  t->pz = pad[0], t->py = pad[1], t->px = pad[2];
+  t->dz = dil[0], t->dy = dil[1], t->dx = dil[2];
   int tx = threads;  // widest power-of-two tile row that the output needs
   while (tx > 32 && tx / 2 >= t->OW) tx /= 2;
-  if (t->OH > 1 && tx > 32) tx = 32;
+  if ((t->OH > 1 || t->OD > 1) && tx > 32) tx = 32;
+  int ty = threads / tx;
+  if (t->OD > 1) {
+    // three dimensions: a brick rather than a slab, so that the input region (and the dX image flushed from it) is
+    // a small multiple of the tile
+    while (tx > 16 || (tx > 4 && tx / 2 >= t->OW)) tx /= 2;
+    ty = 8;
+    while (ty > 1 && ty / 2 >= t->OH) ty /= 2;
+    if (threads / (tx * ty) > 8) ty = threads / (tx * 8);  // at most eight slices per brick
+  }
   t->TX = tx;
-  t->TY = threads / tx;
-  t->log2_tx = 0;
+  t->TY = ty;
+  t->TZ = threads / (tx * ty);
+  t->log2_tx = t->log2_ty = 0;
   while ((1 << t->log2_tx) < tx) ++t->log2_tx;
+  while ((1 << t->log2_ty) < ty) ++t->log2_ty;
+  t->ID = (t->TZ - 1) * t->sz + (t->kd - 1) * t->dz + 1;
   t->IH = (t->TY - 1) * t->sy + (t->kh - 1) * t->dy + 1;
   t->IW = (t->TX - 1) * t->sx + (t->kw - 1) * t->dx + 1;
-  const long long tsz = (long long)t->IH * t->IW;
+  const long long tsz = (long long)t->ID * t->IH * t->IW;
   if (tsz > (1 << 20)) return false;
+  t->PL = t->IH * t->IW;
   t->TSZ = int(tsz);
+  t->tiles_z = (t->OD + t->TZ - 1) / t->TZ;
   t->tiles_y = (t->OH + t->TY - 1) / t->TY;
   t->tiles_x = (t->OW + t->TX - 1) / t->TX;
   t->taps = g.taps;
-  return true;
+  return t->tiles() <= 0x7fffffffLL;
 }
 
-// Cooperative load of the input region of tile (tyi, txi) of image b, all channels: a thread owns one or two cells of
+// Where a thread stands: its tile (index within the image), its output position, and the offset of that position's
+// patch anchor inside the tile's input region.
+struct ConvPos {
+  int tzi, tyi, txi;  // tile
+  int base;           // anchor offset in the region
+  long long pos;      // output position within (image, out channel)
+  bool live;          // the position exists
+};
+
+__device__ __forceinline__ ConvPos conv_pos(const ConvTile &g, unsigned tile_index, unsigned tid) {
+  ConvPos p;
+  const unsigned row = tile_index / unsigned(g.tiles_x);
+  p.txi = int(tile_index - row * unsigned(g.tiles_x));
+  p.tzi = int(row / unsigned(g.tiles_y));
+  p.tyi = int(row - unsigned(p.tzi) * unsigned(g.tiles_y));
+  const int tx = int(tid) & (g.TX - 1), ty = (int(tid) >> g.log2_tx) & (g.TY - 1),
+            tz = int(tid) >> (g.log2_tx + g.log2_ty);
+  const int oz = p.tzi * g.TZ + tz, oy = p.tyi * g.TY + ty, ox = p.txi * g.TX + tx;
+  p.live = oz < g.OD && oy < g.OH && ox < g.OW;
+  p.base = tz * g.sz * g.PL + ty * g.sy * g.IW + tx * g.sx;
+  p.pos = ((long long)oz * g.OH + oy) * g.OW + ox;
+  return p;
+}
+
+// Image coordinates of cell r of the tile's input region: the flat offset inside a channel image, or -1 outside.
+__device__ __forceinline__ long long region_cell(const ConvTile &g, const ConvPos &p, int r) {
+  const int iz = r / g.PL, r2 = r - iz * g.PL;
+  const int iy = r2 / g.IW, ix = r2 - iy * g.IW;
+  const int gz = p.tzi * g.TZ * g.sz - g.pz + iz, gy = p.tyi * g.TY * g.sy - g.py + iy,
+            gx = p.txi * g.TX * g.sx - g.px + ix;
+  if (gz < 0 || gz >= g.D || gy < 0 || gy >= g.H || gx < 0 || gx >= g.W) return -1;
+  return ((long long)gz * g.H + gy) * g.W + gx;
+}
+
+// Cooperative load of the input region of tile `at` of image b, all channels: a thread owns one or two cells of
 // the region and copies them channel by channel (the coordinate arithmetic is done once per cell, not per element).
 // c0 / count: the window of channels to load (all of them by default); plane c0 + k goes to tile plane k.
 template <typename Real, bool CHECK = false>
 __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restrict__ x, const ConvTile &g, int C,
-                                               long long b, int tyi, int txi, int *special, int c0 = 0,
+                                               long long b, const ConvPos &at, int *special, int c0 = 0,
                                                int count = -1) {
-  const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
-  const long long chan = (long long)g.H * g.W;
+  const long long chan = (long long)g.D * g.H * g.W;
   const Real *img = x + (b * C + c0) * chan;
   if (count >= 0) C = count;
   for (int e = threadIdx.x; e < g.TSZ; e += int(blockDim.x)) {
-    const int iy = e / g.IW, ix = e - iy * g.IW;
-    const int gy = iy0 + iy, gx = ix0 + ix;
+    const long long cell = region_cell(g, at, e);
     Real *q = tile + e;
-    if (gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) {
-      const Real *p = img + (long long)gy * g.W + gx;
+    if (cell >= 0) {
+      const Real *p = img + cell;
       bool plain = true;
 #pragma unroll 4
       for (int c = 0; c < C; ++c) {
@@ -266,21 +313,45 @@ __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restric
   }
 }
 
+// The dX image of a tile's input region (fp64, C planes of TSZ cells) added to dx; cells outside the image are dropped
+// like the reference drops padded taps. Regions of neighbouring tiles overlap, hence atomics.
+template <typename Real>
+__device__ __forceinline__ void flush_dx_image(const double *acc, const ConvTile &g, const ConvPos &at, int C,
+                                               Real *dx_first /* image b, first channel of the window */) {
+  const long long chan = (long long)g.D * g.H * g.W;
+  for (int i = threadIdx.x; i < C * g.TSZ; i += int(blockDim.x)) {
+    const double v = acc[i];
+    if (v == 0.0) continue;
+    const int c = i / g.TSZ, r = i - c * g.TSZ;
+    const long long cell = region_cell(g, at, r);
+    if (cell >= 0) atomicAdd(dx_first + c * chan + cell, Real(v));
+  }
+}
+
+// Offset of every tap from the patch anchor inside the tile's input region; filled once per workgroup (a barrier
+// separates it from the first staging of trees), so that staging a vertex is a table lookup instead of divisions.
+__device__ __forceinline__ void fill_tap_offsets(int *tapoff, const ConvTile &g) {
+  for (int tap = threadIdx.x; tap < g.taps; tap += int(blockDim.x)) {
+    const int kz = tap / (g.kh * g.kw), rest = tap - kz * (g.kh * g.kw);
+    const int ky = rest / g.kw, kx = rest - ky * g.kw;
+    tapoff[tap] = kz * g.dz * g.PL + ky * g.dy * g.IW + kx * g.dx;
+  }
+}
+
 // Trees (and optionally leaf weights) of out channel j into LDS.
 // c0 / count: the window of channels whose trees are staged (all of them by default).
 template <typename Real, bool CHECK = false>
-__device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, const ConvTile &g, int C, int V, int LM,
-                                                 int j, const Real *__restrict__ thr, const int64_t *__restrict__ ord,
-                                                 const Real *__restrict__ w, int *special, int c0 = 0, int count = -1) {
+__device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, const ConvTile &g, const int *tapoff,
+                                                 int C, int V, int LM, int j, const Real *__restrict__ thr,
+                                                 const int64_t *__restrict__ ord, const Real *__restrict__ w,
+                                                 int *special, int c0 = 0, int count = -1) {
   const long long tree0 = (long long)j * C + c0;
   if (count >= 0) C = count;
   const long long first = tree0 * V;
   for (int i = threadIdx.x; i < C * V; i += int(blockDim.x)) {
-    const int tap = clamp_ordinal(ord[first + i], g.taps);
-    const int ky = tap / g.kw, kx = tap - ky * g.kw;
     Node<Real> n;
     n.thr = thr[first + i];
-    n.ord = ky * g.dy * g.IW + kx * g.dx;
+    n.ord = tapoff[clamp_ordinal(ord[first + i], g.taps)];
     nodes[i] = n;
     if (CHECK && !plain_threshold(n.thr)) *special = 1;
   }
@@ -291,7 +362,7 @@ __device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, co
 }
 
 struct ConvLds {
-  size_t tile, acc_x, nodes, wl, acc_w, acc_t, flag, total;
+  size_t tile, acc_x, nodes, wl, acc_w, acc_t, taps, flag, total;
 };
 
 template <typename Real>
@@ -310,6 +381,8 @@ static ConvLds conv_lds_layout(const ConvTile &t, int C, int V, int LM, bool dx_
   if (tree_acc) at += align_up(size_t(C) * LM * sizeof(double), 16);
   l.acc_t = at;
   if (tree_acc) at += align_up(size_t(C) * V * sizeof(double), 16);
+  l.taps = at;  // tap -> offset in the tile's input region
+  at += align_up(size_t(t.taps) * sizeof(int), 16);
   l.flag = at;  // one word: set once the tile or the staged trees hold a value that rules out walk_paths_plain
   at += 16;
   l.total = at;
@@ -367,27 +440,27 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_forward_kernel(ConvTi
   Real *tile = reinterpret_cast<Real *>(smem + lay.tile);
   Node<Real> *nodes = reinterpret_cast<Node<Real> *>(smem + lay.nodes);
   Real *wl = reinterpret_cast<Real *>(smem + lay.wl);
-  const int tyi = blockIdx.x / g.tiles_x, txi = blockIdx.x - tyi * g.tiles_x;
+  const ConvPos at = conv_pos(g, blockIdx.x, threadIdx.x);
   const long long b = blockIdx.z;
   int *special = reinterpret_cast<int *>(smem + lay.flag);
+  int *tapoff = reinterpret_cast<int *>(smem + lay.taps);
+  fill_tap_offsets(tapoff, g);
   if (threadIdx.x == 0) *special = 0;
-  const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
-  const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
-  const bool live = oy < g.OH && ox < g.OW;
-  const Real *mine = tile + ty * g.sy * g.IW + tx * g.sx;
+  const bool live = at.live;
+  const Real *mine = tile + at.base;
   const int LM = L * M;
   const int j_begin = blockIdx.y * j_per, j_end = min(Cout, j_begin + j_per);
   for (int c0 = 0; c0 < C_all; c0 += c_per) {
     const int C = min(c_per, C_all - c0);
     __syncthreads();  // the flag is cleared / the previous window's planes and trees are no longer read
-    load_conv_tile<Real, true>(tile, x, g, C_all, b, tyi, txi, special, c0, C);
+    load_conv_tile<Real, true>(tile, x, g, C_all, b, at, special, c0, C);
     for (int j = j_begin; j < j_end; ++j) {
       __syncthreads();  // the planes are complete / the previous out channel's trees are no longer read
-      stage_conv_trees<Real, true>(nodes, wl, g, C_all, V, LM, j, thr, ord, w, special, c0, C);
+      stage_conv_trees<Real, true>(nodes, wl, g, tapoff, C_all, V, LM, j, thr, ord, w, special, c0, C);
       __syncthreads();
       if (!live) continue;
       const bool plain = *special == 0;
-      Real *o = out + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+      Real *o = out + ((b * Cout + j) * g.positions() + at.pos) * M;
       for (int m0 = 0; m0 < M; m0 += MREG) {
         const int mc = min(MREG, M - m0);
         Real acc[MREG];
@@ -439,27 +512,27 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_dx_kernel(ConvTile g,
   double *acc = reinterpret_cast<double *>(smem + lay.acc_x);
   Node<Real> *nodes = reinterpret_cast<Node<Real> *>(smem + lay.nodes);
   Real *wl = reinterpret_cast<Real *>(smem + lay.wl);
-  const int tyi = blockIdx.x / g.tiles_x, txi = blockIdx.x - tyi * g.tiles_x;
+  const ConvPos at = conv_pos(g, blockIdx.x, threadIdx.x);
   const long long b = blockIdx.z;
   int *special = reinterpret_cast<int *>(smem + lay.flag);
+  int *tapoff = reinterpret_cast<int *>(smem + lay.taps);
+  fill_tap_offsets(tapoff, g);
   if (threadIdx.x == 0) *special = 0;
   __syncthreads();
-  load_conv_tile<Real, true>(tile, x, g, C, b, tyi, txi, special);
+  load_conv_tile<Real, true>(tile, x, g, C, b, at, special);
   for (int i = threadIdx.x; i < C * g.TSZ; i += kConvThreads) acc[i] = 0.0;
-  const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
-  const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
-  const bool live = oy < g.OH && ox < g.OW;
-  const int base = ty * g.sy * g.IW + tx * g.sx;
+  const bool live = at.live;
+  const int base = at.base;
   const Real *mine = tile + base;
   const int LM = L * M;
   const int j_begin = blockIdx.y * j_per, j_end = min(Cout, j_begin + j_per);
   for (int j = j_begin; j < j_end; ++j) {
     __syncthreads();
-    stage_conv_trees<Real, true>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
+    stage_conv_trees<Real, true>(nodes, wl, g, tapoff, C, V, LM, j, thr, ord, w, special);
     __syncthreads();
     if (!live) continue;
     const bool plain = *special == 0;
-    const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+    const Real *gp = gout + ((b * Cout + j) * g.positions() + at.pos) * M;
     for (int c = 0; c < C; c += kConvIlp) {
       WalkResult<Real> r[kConvIlp];
       const Node<Real> *nd[kConvIlp];
@@ -483,15 +556,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_dx_kernel(ConvTile g,
     }
   }
   __syncthreads();
-  const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
-  for (int i = threadIdx.x; i < C * g.TSZ; i += kConvThreads) {
-    const double v = acc[i];
-    if (v == 0.0) continue;
-    const int c = i / g.TSZ, r = i - c * g.TSZ;
-    const int iy = r / g.IW, ix = r - iy * g.IW;
-    const int gy = iy0 + iy, gx = ix0 + ix;
-    if (gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) atomicAdd(dx + ((b * C + c) * g.H + gy) * (long long)g.W + gx, Real(v));
-  }
+  flush_dx_image(acc, g, at, C, dx + b * C * (long long)g.D * g.H * g.W);
 }
 
 // dThr and dW: a workgroup owns out channel blockIdx.x and visits every blockIdx.y-th (image, tile); the gradients of
@@ -514,26 +579,25 @@ __global__ __launch_bounds__(kConvThreads) void conv_tiled_trees_kernel(ConvTile
   const int j = blockIdx.x;
   const int LM = L * M;
   int *special = reinterpret_cast<int *>(smem + lay.flag);
+  int *tapoff = reinterpret_cast<int *>(smem + lay.taps);
+  fill_tap_offsets(tapoff, g);
   if (threadIdx.x == 0) *special = 0;
   __syncthreads();
-  stage_conv_trees<Real, true>(nodes, wl, g, C, V, LM, j, thr, ord, w, special);
+  stage_conv_trees<Real, true>(nodes, wl, g, tapoff, C, V, LM, j, thr, ord, w, special);
   for (int i = threadIdx.x; i < C * LM; i += kConvThreads) acc_w[i] = 0.0;
   for (int i = threadIdx.x; i < C * V; i += kConvThreads) acc_t[i] = 0.0;
-  const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
-  const Real *mine = tile + ty * g.sy * g.IW + tx * g.sx;
-  const int tiles = g.tiles_y * g.tiles_x;
+  const long long tiles = g.tiles();
   const int skew = int(threadIdx.x & 63u) % C;
   for (long long it = blockIdx.y; it < items; it += gridDim.y) {
     const long long b = it / tiles;
-    const int t = int(it - b * tiles);
-    const int tyi = t / g.tiles_x, txi = t - tyi * g.tiles_x;
+    const ConvPos at = conv_pos(g, unsigned(it - b * tiles), threadIdx.x);
+    const Real *mine = tile + at.base;
     __syncthreads();  // the previous tile is no longer read (first pass: the staged trees are complete)
-    load_conv_tile<Real, true>(tile, x, g, C, b, tyi, txi, special);
+    load_conv_tile<Real, true>(tile, x, g, C, b, at, special);
     __syncthreads();
     const bool plain = *special == 0;
-    const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
-    if (oy >= g.OH || ox >= g.OW) continue;
-    const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+    if (!at.live) continue;
+    const Real *gp = gout + ((b * Cout + j) * g.positions() + at.pos) * M;
     for (int c = 0; c < C; c += kConvIlp) {
       WalkResult<Real> r[kConvIlp];
       const Node<Real> *nd[kConvIlp];
@@ -601,7 +665,7 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
   Real *wl = reinterpret_cast<Real *>(smem + lay.wl);
   double *acc_w = reinterpret_cast<double *>(smem + lay.acc_w);
   double *acc_t = reinterpret_cast<double *>(smem + lay.acc_t);
-  const int tyi = blockIdx.x / g.tiles_x, txi = blockIdx.x - tyi * g.tiles_x;
+  const ConvPos at = conv_pos(g, blockIdx.x, threadIdx.x);
   const long long b = blockIdx.z;
   // blockIdx.y = (block of out channels, window of channels): a workgroup holds the tile planes, the dX image and the
   // trees of c_per channels only, so that several workgroups fit a CU
@@ -609,6 +673,8 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
   const int c0 = int(blockIdx.y % unsigned(c_blocks)) * c_per, j_block = int(blockIdx.y / unsigned(c_blocks));
   const int C = min(c_per, C_all - c0);
   int *special = reinterpret_cast<int *>(smem + lay.flag);
+  int *tapoff = reinterpret_cast<int *>(smem + lay.taps);
+  fill_tap_offsets(tapoff, g);
   const int LM = L * M;
   // single-output float trees walk by the sign bit where the data allow it (walk_paths_plain_tracked)
   constexpr bool kLeanWalk = M1 && std::is_same<Real, float>::value;
@@ -616,14 +682,12 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
     if (threadIdx.x == 0) *special = 0;
     __syncthreads();
   }
-  load_conv_tile<Real, kLeanWalk>(tile, x, g, C_all, b, tyi, txi, special, c0, C);
+  load_conv_tile<Real, kLeanWalk>(tile, x, g, C_all, b, at, special, c0, C);
   for (int i = threadIdx.x; i < C * g.TSZ; i += NT) acc[i] = 0.0;
   for (int i = threadIdx.x; i < C * LM; i += NT) acc_w[i] = 0.0;
   for (int i = threadIdx.x; i < C * V; i += NT) acc_t[i] = 0.0;
-  const int ty = threadIdx.x >> g.log2_tx, tx = threadIdx.x & (g.TX - 1);
-  const int oy = tyi * g.TY + ty, ox = txi * g.TX + tx;
-  const bool live = oy < g.OH && ox < g.OW;
-  const int base = ty * g.sy * g.IW + tx * g.sx;
+  const bool live = at.live;
+  const int base = at.base;
   const Real *mine = tile + base;
   // Lane l takes the channels in the order skew(l), skew(l) + 1, ... (mod C): the lanes of a wavefront are spread over
   // min(C, 64) trees' tables and dX planes, so the atomics of one instruction rarely meet on one address.
@@ -654,10 +718,10 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
           }
         }
     }
-    stage_conv_trees<Real, kLeanWalk>(nodes, wl, g, C_all, V, LM, j, thr, ord, w, special, c0, C);
+    stage_conv_trees<Real, kLeanWalk>(nodes, wl, g, tapoff, C_all, V, LM, j, thr, ord, w, special, c0, C);
     __syncthreads();
     if (!live) continue;
-    const Real *gp = gout + ((b * Cout + j) * (long long)g.OH * g.OW + (long long)oy * g.OW + ox) * M;
+    const Real *gp = gout + ((b * Cout + j) * g.positions() + at.pos) * M;
     const Real g_one = M1 ? gp[0] : Real(0);
     if constexpr (kLeanWalk) {
       if (*special == 0) {
@@ -739,15 +803,7 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
       for (int i = threadIdx.x; i < C * V; i += NT)
         if (acc_t[i] != 0.0) atomicAdd(dthr + ((long long)jp * C_all + c0) * V + i, Real(acc_t[i]));
   }
-  const int iy0 = tyi * g.TY * g.sy - g.py, ix0 = txi * g.TX * g.sx - g.px;
-  for (int i = threadIdx.x; i < C * g.TSZ; i += NT) {
-    const double v = acc[i];
-    if (v == 0.0) continue;
-    const int c = i / g.TSZ, r = i - c * g.TSZ;
-    const int iy = r / g.IW, ix = r - iy * g.IW;
-    const int gy = iy0 + iy, gx = ix0 + ix;
-    if (gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) atomicAdd(dx + ((b * C_all + c0 + c) * g.H + gy) * (long long)g.W + gx, Real(v));
-  }
+  flush_dx_image(acc, g, at, C, dx + (b * C_all + c0) * (long long)g.D * g.H * g.W);
 }
 
 constexpr int kConvWideThreads = 512;  // workgroup of the one-walk backward kernel
@@ -831,8 +887,8 @@ int conv_forward(const ht_conv_shape &s, const Real *x, const Real *thr, const i
       c_per = (c_per + 1) / 2;
       lay = conv_lds_layout<Real>(t, c_per, V, LM, false, false, true);
     }
-    if (lay.total <= kConvTiledLdsMax && (long long)t.tiles_y * t.tiles_x <= 0x7fffffffLL) {
-      const long long tiles = (long long)t.tiles_y * t.tiles_x;
+    if (lay.total <= kConvTiledLdsMax) {
+      const long long tiles = t.tiles();
       const int j_per = conv_j_per(tiles * s.B, int(s.Cout));
       const dim3 tgrid((unsigned)tiles, (unsigned)((s.Cout + j_per - 1) / j_per), (unsigned)s.B);
       auto kernel = fern ? conv_tiled_forward_kernel<Real, true, 16> : conv_tiled_forward_kernel<Real, false, 16>;
@@ -902,8 +958,8 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
       c_per = (c_per + 1) / 2;
       lay = conv_lds_layout<Real>(t, c_per, V, LM, true, true, true);
     }
-    const long long tiles = (long long)t.tiles_y * t.tiles_x;
-    if (lay.total > kConvTiledLdsMax || tiles > 0x7fffffffLL) continue;
+    const long long tiles = t.tiles();
+    if (lay.total > kConvTiledLdsMax) continue;
     const int c_blocks = (int(s.C) + c_per - 1) / c_per;
     const int j_per = conv_j_per(tiles * s.B * c_blocks, int(s.Cout));
     const long long grid_y = (long long)((s.Cout + j_per - 1) / j_per) * c_blocks;
@@ -932,8 +988,8 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
     const int LM = L * int(s.M);
     const ConvLds lay_x = conv_lds_layout<Real>(t, int(s.C), V, LM, true, false, true);
     const ConvLds lay_t = conv_lds_layout<Real>(t, int(s.C), V, LM, false, true, true);
-    const long long tiles = (long long)t.tiles_y * t.tiles_x;
-    if (lay_x.total <= kConvTiledLdsMax && lay_t.total <= kConvTiledLdsMax && tiles <= 0x7fffffffLL) {
+    const long long tiles = t.tiles();
+    if (lay_x.total <= kConvTiledLdsMax && lay_t.total <= kConvTiledLdsMax) {
       if (dx) {
         const int j_per = conv_j_per(tiles * s.B, int(s.Cout));
         const dim3 grid((unsigned)tiles, (unsigned)((s.Cout + j_per - 1) / j_per), (unsigned)s.B);

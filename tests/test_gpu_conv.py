@@ -29,6 +29,10 @@ CASES = [
     (1, 70, 3, [20, 37], 6, [], [3, 3], [1, 1], [1, 1], [1, 1]),       # forward in channel windows (running sums pass through `out`)
     (1, 21, 2, [23, 35], 5, [5], [3, 3], [2, 1], [1, 1], [1, 1]),      # ... with several outputs per leaf and a stride
     (1, 6, 3, [24, 40], 10, [], [3, 3], [1, 1], [1, 1], [1, 1]),       # deep trees: the one-walk backward in windows of few channels
+    (2, 3, 4, [9, 21, 19], 4, [], [3, 3, 3], [1, 1, 1], [1, 1, 1], [1, 1, 1]),    # volumes: bricks of positions, ragged on every side
+    (1, 5, 2, [11, 10, 37], 3, [3], [3, 2, 3], [2, 1, 2], [1, 0, 2], [1, 2, 1]),  # ... stride, dilation and padding differ by axis
+    (1, 2, 3, [2, 30, 5], 5, [], [2, 3, 3], [1, 1, 1], [1, 1, 1], [1, 1, 1]),     # ... thin along z and x
+    (1, 20, 2, [6, 12, 18], 2, [], [3, 3, 3], [1, 1, 1], [1, 1, 1], [2, 2, 2]),   # ... dilated taps, channels in windows
 ]
 
 
