@@ -43,6 +43,7 @@ _I = ctypes.c_int
 SIGNATURES = {
     "ht_last_error": (ctypes.c_char_p, []),
     "ht_abi_version": (_I, []),
+    "ht_check_device": (_I, [ctypes.c_int32]),
     "ht_ordinal_range": (_I, [_P, ctypes.c_int64, _P, _P]),
     "ht_forest_forward_workspace": (_SZ, [ctypes.POINTER(ForestShape)]),
     "ht_forest_forward": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _SZ, _P]),

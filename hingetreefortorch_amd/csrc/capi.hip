@@ -1,5 +1,6 @@
 // extern "C" surface of libhingetree_hip.so (declared in include/hingetree_hip.h) and the host-only pieces.
 #include <cmath>
+#include <cstring>
 #include <limits>
 #include <mutex>
 
@@ -171,6 +172,15 @@ extern "C" {
 
 const char *ht_last_error(void) { return g_last_error.c_str(); }
 int ht_abi_version(void) { return 1; }
+
+int ht_check_device(int32_t device) {
+  hipDeviceProp_t prop;
+  HT_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(HT_ERR_RUNTIME, std::string("Error: this library holds kernels for gfx950 (MI355X) only; device ") +
+                                    std::to_string(device) + " is " + prop.gcnArchName + ".");
+  return HT_OK;
+}
 
 int ht_ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, void *stream) {
   if (!minmax || (n > 0 && !ord)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");

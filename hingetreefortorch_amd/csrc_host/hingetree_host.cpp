@@ -12,6 +12,7 @@
 #include <c10/core/DeviceGuard.h>
 #include <torch/extension.h>
 
+#include <atomic>
 #include <mutex>
 #include <sstream>
 #include <stdexcept>
@@ -58,7 +59,15 @@ int dtype_code(const torch::Tensor &t) { return t.scalar_type() == torch::kFloat
 
 void *ptr(const torch::Tensor &t) { return t.defined() ? t.data_ptr() : nullptr; }
 
+// The stream torch is using on the tensor's device; the first use of a device also asks the library whether it can run
+// there.
 void *current_stream(const torch::Tensor &t) {
+  static std::atomic<bool> checked[64];
+  const int index = t.device().index();
+  if (index >= 0 && index < 64 && !checked[index].load(std::memory_order_acquire)) {
+    check(ht_check_device(index));
+    checked[index].store(true, std::memory_order_release);
+  }
   return static_cast<void *>(at::hip::getCurrentHIPStream(t.device().index()).stream());
 }
 

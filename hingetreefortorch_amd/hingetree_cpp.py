@@ -40,7 +40,15 @@ def _ptr(t):
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
+_checked_devices = set()
+
+
 def _stream(device):
+    """The stream torch is using on `device`; the first use of a device also asks the library whether it can run there."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _checked_devices:
+        L.check(L.load().ht_check_device(index))
+        _checked_devices.add(index)
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 

@@ -60,6 +60,10 @@ typedef struct ht_tile_shape {
 const char *ht_last_error(void);
 /* ABI version of this header; bumped on any signature change. */
 int ht_abi_version(void);
+/* HT_OK if GPU `device` can run this library's code object (gfx950), else an error that names what it is. The tile
+ * sizes assume that part's 160 KB of LDS per workgroup, 256 compute units and 8 L2 domains; hosts call this once per
+ * device before the first launch. No counterpart in the reference, which compiles for whatever nvcc targets. */
+int ht_check_device(int32_t device);
 
 /* Device-side min and max of n int64 ordinals -> minmax[0], minmax[1] (device memory, 2 x int64).
  * Replaces the reference's per-call `inOrdinals.min()/.max()` range check (hingetree.cpp:91, hingetree_gpu.cu:445):

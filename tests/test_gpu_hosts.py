@@ -146,3 +146,9 @@ def test_module_trains_on_either_host(dev, either_host):
                                   model.weights.detach().cpu(), up.cpu())
     assert rel_err(x.grad.cpu(), rdx) <= 1e-5 and rel_err(model.thresholds.grad.cpu(), rdthr) <= 1e-5
     assert rel_err(model.weights.grad.cpu(), rdw) <= 1e-5
+
+
+def test_device_check(dev):
+    """The library says yes to the GPU it was built for; both hosts ask once per device before their first launch."""
+    from hingetreefortorch_amd import _lib
+    assert _lib.load().ht_check_device(dev.index or 0) == _lib.HT_OK
