@@ -393,6 +393,17 @@ __device__ __forceinline__ void walk_ferns_staged(int depth, const Node<Real> *m
   }
 }
 
+// What lane + 1 of the wavefront holds in v (lane 63: 0): one data-parallel move of the vector ALU per 32 bits.
+__device__ __forceinline__ float value_of_next_lane(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130 /* wave_shl:1 */, 0xf, 0xf, false));
+}
+__device__ __forceinline__ double value_of_next_lane(double v) {
+  const long long b = __double_as_longlong(v);
+  const int lo = __builtin_amdgcn_update_dpp(0, int(uint32_t(b)), 0x130, 0xf, 0xf, false);
+  const int hi = __builtin_amdgcn_update_dpp(0, int(uint32_t(uint64_t(b) >> 32)), 0x130, 0xf, 0xf, false);
+  return __longlong_as_double((long long)((uint64_t(uint32_t(hi)) << 32) | uint32_t(lo)));
+}
+
 constexpr int kRowIlp = 4;     // trees walked concurrently per lane
 constexpr int kRowUnroll = 5;  // output vectors per lane whose weight gathers are in flight together
 
@@ -405,7 +416,13 @@ constexpr int kRowUnroll = 5;  // output vectors per lane whose weight gathers a
 //
 // QUAD selects two-level vertices (float trees, F <= 1024); otherwise Node<Real> is walked level by level.
 // GW = elements per weight gather and per store (divides M). RECORD: also write the walk records.
-template <typename Real, bool FERN, bool QUAD, int BT, int GW, bool RECORD, bool COMPACT>
+// ODD (with GW = 2): an odd number of outputs per leaf written as pairs all the same. A sample's run of a step's trees
+// starts on an even element, so the pairs (e, e + 1), e even, are aligned stores; the leaf table is a padded copy whose
+// odd trees' rows are shifted by one element, which makes a pair's first element an even index of its row in every
+// tree: one aligned gather per pair, (M + 1) / 2 gather slots per tree instead of M (the cost of the output phase is
+// its number of gather instructions, and its stores must leave no holes for a later instruction to fill).
+// Needs an even tree count, so that every sample's row of the output starts on an even element.
+template <typename Real, bool FERN, bool QUAD, int BT, int GW, bool ODD, bool RECORD, bool COMPACT>
 __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims d, const Real *__restrict__ x,
                                                                       const void *__restrict__ vertices, int NQ,
                                                                       const Real *__restrict__ w,
@@ -462,13 +479,39 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
   int full_un = 0;
   {
     const int u_full = TPW * d.M / GW, total_full = BT * u_full;
-    if (n_live == BT) {
+    if (!ODD && n_live == BT) {
       if (total_full % (kWave * kRowUnroll) == 0 && (kWave * kRowUnroll) % u_full == 0) full_un = kRowUnroll;
     }
 #pragma unroll
     for (int q = 0; q < kRowUnroll; ++q) full_park[q] = full_wcol[q] = full_off[q] = 0;
     if (full_un == kRowUnroll)
       burst_constants(std::integral_constant<int, kRowUnroll>{}, u_full, div_u_full, full_park, full_wcol, full_off);
+  }
+
+  // ODD: what this lane does in every instruction of the output phase (see there)
+  constexpr int kOddUnroll = 4;
+  int odd_upi = 1, odd_unit = 0, odd_second = 0, odd_idx = 0, odd_role = 0;
+  bool odd_active = false;
+  uint32_t odd_park[kOddUnroll] = {}, odd_wcol[kOddUnroll] = {}, odd_off[kOddUnroll] = {};
+  if (ODD) {
+    const int slots = d.M + 1, hs = slots >> 1;
+    odd_upi = kWave / slots;                 // pairs of trees per wavefront instruction
+    odd_unit = lane / slots;
+    const int r = lane - odd_unit * slots;   // 0 .. M: the gather slot inside the pair of trees
+    odd_active = odd_unit < odd_upi;
+    odd_second = r >= hs ? 1 : 0;            // the odd tree of the pair
+    odd_idx = odd_second ? 2 * (r - hs) : 2 * r;  // first element read, as an index of its (shifted) row
+    odd_role = r == hs - 1 ? 1 : (r == hs ? 2 : 0);  // 1: the even tree's last element; 2: the odd tree's first
+    // complete steps of a complete tile, kOddUnroll instructions per iteration: an iteration is then a whole number of
+    // samples (kOddUnroll is a multiple of the TPW / 2 pairs of trees of a sample's run wherever BT >= 32), and
+    // what changes from one iteration to the next is the sample alone
+#pragma unroll
+    for (int q = 0; q < kOddUnroll; ++q) {
+      const int g = q * odd_upi + odd_unit, jj = g / (TPW / 2), tt = 2 * (g - jj * (TPW / 2)) + odd_second;
+      odd_park[q] = uint32_t(jj * LDP + tt);
+      odd_wcol[q] = uint32_t(tt) * uint32_t(d.L) * uint32_t(wpitch) + uint32_t(odd_idx);
+      odd_off[q] = uint32_t(jj) * TM + uint32_t(tt * d.M + odd_idx - odd_second);
+    }
   }
 
   for (int tb = t_begin + wave * TPW; tb < t_end; tb += kWaves * TPW) {
@@ -557,12 +600,91 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
 
     // ---- output: out[s0 + jj, tb .. tb + nt, 0 .. M) is one contiguous run per sample
     const int nt = min(TPW, t_end - tb);
+    Real *obase = out + ((long long)s0 * d.T + tb) * d.M;
+    const Real *wbase = w + (long long)tb * d.L * wpitch;  // wpitch: elements between leaf rows (M, or padded)
+    if constexpr (ODD) {
+      // nt is even here (the tree count is, and so is every step's first tree). Two trees are M + 1 gathers: the even
+      // tree's pairs (0,1) .. (M-3,M-2), its last element alone, the odd tree's first element alone, its pairs (1,2) ..
+      // (M-2,M-1) -- each one aligned 8-byte gather from the padded (and, in odd trees, shifted) rows. The two
+      // lone elements are neighbours in the output: the lane of the first fetches the second's product from the next
+      // lane and stores the pair, the lane of the second stores nothing. A wavefront instruction serves whole pairs
+      // of trees (64 / (M + 1) of them), so what a lane does is the same in every instruction and the two lone
+      // elements always sit in neighbouring lanes.
+      const int units = nt >> 1, total_units = n_live * units;
+      if ((kOddUnroll % (TPW / 2)) == 0 && nt == TPW && n_live == BT) {
+        uint32_t park[kOddUnroll], off[kOddUnroll];
+        int g[kOddUnroll];
+#pragma unroll
+        for (int q = 0; q < kOddUnroll; ++q) park[q] = odd_park[q], off[q] = odd_off[q], g[q] = q * odd_upi + odd_unit;
+        const int per_iteration = odd_upi * kOddUnroll;               // pairs of trees
+        const uint32_t samples = uint32_t(per_iteration / (TPW / 2));  // ... which are whole samples
+        for (int g0 = 0; g0 < total_units; g0 += per_iteration) {
+          Real a[kOddUnroll];
+          Vec wv[kOddUnroll];
+          bool live_q[kOddUnroll];
+#pragma unroll
+          for (int q = 0; q < kOddUnroll; ++q) {
+            live_q[q] = odd_active && g[q] < total_units;
+            const uint32_t at = live_q[q] ? park[q] : 0u;  // idle lanes read a parked result that exists
+            const uint32_t key = p_key[at];
+            a[q] = p_abs[at];
+            wv[q] = *reinterpret_cast<const Vec *>(wbase + key * uint32_t(wpitch) + odd_wcol[q]);
+          }
+#pragma unroll
+          for (int q = 0; q < kOddUnroll; ++q) {
+            Vec o;
+            o[0] = a[q] * wv[q][0];
+            o[1] = a[q] * wv[q][1];
+            const Real from_next = value_of_next_lane(o[1]);
+            if (odd_role == 1) o[1] = from_next;
+            if (live_q[q] && odd_role != 2) __builtin_nontemporal_store(o, reinterpret_cast<Vec *>(obase + off[q]));
+            park[q] += samples * LDP;
+            off[q] += samples * TM;
+            g[q] += per_iteration;
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+        continue;
+      }
+      const FastDiv by_units = nt == TPW ? FastDiv(TPW / 2) : FastDiv(units);  // (the first: a constant)
+      for (int g0 = 0; g0 < total_units; g0 += odd_upi * kRowUnroll) {
+        Real a[kRowUnroll];
+        Vec wv[kRowUnroll], o[kRowUnroll];
+        uint32_t off[kRowUnroll];
+        bool live_q[kRowUnroll];
+#pragma unroll
+        for (int q = 0; q < kRowUnroll; ++q) {
+          const int g = g0 + q * odd_upi + odd_unit;
+          live_q[q] = odd_active && g < total_units;
+          const int gc = min(g, total_units - 1);
+          const int jj = by_units.div(gc), tt = 2 * (gc - jj * units) + odd_second;
+          const uint32_t key = p_key[jj * LDP + tt];
+          a[q] = p_abs[jj * LDP + tt];
+          wv[q] = *reinterpret_cast<const Vec *>(wbase + (uint32_t(tt) * uint32_t(d.L) + key) * uint32_t(wpitch) +
+                                                 odd_idx);
+          off[q] = uint32_t(jj) * TM + uint32_t(tt * d.M + odd_idx - odd_second);
+        }
+#pragma unroll
+        for (int q = 0; q < kRowUnroll; ++q) {
+          o[q][0] = a[q] * wv[q][0];
+          o[q][1] = a[q] * wv[q][1];
+        }
+#pragma unroll
+        for (int q = 0; q < kRowUnroll; ++q) {
+          const Real from_next = value_of_next_lane(o[q][1]);
+          if (odd_role == 1) o[q][1] = from_next;
+          // (ordinary stores for the pairs in sectors that the step's run covers only in part -- an odd run of 8 M
+          // elements is not a whole number of 64-byte sectors -- were measured and cost 15 %)
+          if (live_q[q] && odd_role != 2) __builtin_nontemporal_store(o[q], reinterpret_cast<Vec *>(obase + off[q]));
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      continue;
+    }
     const int U = nt * d.M / GW;  // vectors per sample
     FastDiv div_u = div_u_full;   // divisor TPW * M / GW, prepared by the host
     if (nt != TPW) div_u = FastDiv(U);
     const int total = n_live * U;
-    Real *obase = out + ((long long)s0 * d.T + tb) * d.M;
-    const Real *wbase = w + (long long)tb * d.L * wpitch;  // wpitch: elements between leaf rows (M, or padded)
     // Whole bursts, and a burst is a whole number of samples: which tree and output a lane serves in slot q of a
     // burst is the same in every burst, so the divisions are done once (complete tiles of the benchmark shapes: 32
     // samples x 8 trees x 10 outputs = 4 bursts of 5 vectors per lane, 8 samples each) and a burst only advances the
@@ -670,7 +792,7 @@ static inline bool quads_ok(const ForestDims &d, bool fern) {
          (long long)d.T * quads_per_tree(d.depth) < (1ll << 31);
 }
 
-template <typename Real, bool FERN, bool QUAD, int BT, int GW, bool RECORD, bool COMPACT>
+template <typename Real, bool FERN, bool QUAD, int BT, int GW, bool ODD, bool RECORD, bool COMPACT>
 int launch_rows(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, Real *out,
                 void *records, hipStream_t stream) {
   constexpr int TPW = kWave / BT * kRowIlp;
@@ -680,7 +802,7 @@ int launch_rows(const ForestDims &d, const Real *x, const void *vertices, const 
   int trees_per_block, gy;
   split_trees(tiles, d.T, TP, &trees_per_block, &gy);
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
-  auto kernel = forward_rows_kernel<Real, FERN, QUAD, BT, GW, RECORD, COMPACT>;
+  auto kernel = forward_rows_kernel<Real, FERN, QUAD, BT, GW, ODD, RECORD, COMPACT>;
   Records<Real, COMPACT> rec{};
   if (RECORD) rec = carve_records<Real, COMPACT>(d, records, nullptr);
   HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -692,19 +814,22 @@ int launch_rows(const ForestDims &d, const Real *x, const void *vertices, const 
   return HT_OK;
 }
 
-template <typename Real, bool FERN, bool QUAD, int BT, int GW>
+template <typename Real, bool FERN, bool QUAD, int BT, int GW, bool ODD = false>
 int launch_rows_rec(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, Real *out,
                     void *records, hipStream_t stream) {
-  if (!records) return launch_rows<Real, FERN, QUAD, BT, GW, false, true>(d, x, vertices, w, wpitch, out, records, stream);
+  if (!records)
+    return launch_rows<Real, FERN, QUAD, BT, GW, ODD, false, true>(d, x, vertices, w, wpitch, out, records, stream);
   if (compact_ok(d))
-    return launch_rows<Real, FERN, QUAD, BT, GW, true, true>(d, x, vertices, w, wpitch, out, records, stream);
-  return launch_rows<Real, FERN, QUAD, BT, GW, true, false>(d, x, vertices, w, wpitch, out, records, stream);
+    return launch_rows<Real, FERN, QUAD, BT, GW, ODD, true, true>(d, x, vertices, w, wpitch, out, records, stream);
+  return launch_rows<Real, FERN, QUAD, BT, GW, ODD, true, false>(d, x, vertices, w, wpitch, out, records, stream);
 }
 
 template <typename Real, bool FERN, bool QUAD, int BT>
-int launch_rows_gw(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, Real *out,
-                   void *records, hipStream_t stream) {
+int launch_rows_gw(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, bool shifted,
+                   Real *out, void *records, hipStream_t stream) {
   const uintptr_t pw = reinterpret_cast<uintptr_t>(w), po = reinterpret_cast<uintptr_t>(out);
+  if (shifted)  // odd rows in pairs: the table was laid out for it and the alignments were checked, see odd_pairs_ok
+    return launch_rows_rec<Real, FERN, QUAD, BT, 2, true>(d, x, vertices, w, wpitch, out, records, stream);
   if (d.M % 4 == 0 && wpitch % 4 == 0 && pw % (4 * sizeof(Real)) == 0 && po % (4 * sizeof(Real)) == 0)
     return launch_rows_rec<Real, FERN, QUAD, BT, 4>(d, x, vertices, w, wpitch, out, records, stream);
   if (d.M % 2 == 0 && wpitch % 2 == 0 && pw % (2 * sizeof(Real)) == 0 && po % (2 * sizeof(Real)) == 0)
@@ -713,13 +838,13 @@ int launch_rows_gw(const ForestDims &d, const Real *x, const void *vertices, con
 }
 
 template <typename Real, bool FERN, bool QUAD>
-int dispatch_rows(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, Real *out,
-                  void *records, hipStream_t stream) {
+int dispatch_rows(const ForestDims &d, const Real *x, const void *vertices, const Real *w, int wpitch, bool shifted,
+                  Real *out, void *records, hipStream_t stream) {
   switch (pick_rows_tile<Real>(d.F)) {
-    case 64: return launch_rows_gw<Real, FERN, QUAD, 64>(d, x, vertices, w, wpitch, out, records, stream);
-    case 32: return launch_rows_gw<Real, FERN, QUAD, 32>(d, x, vertices, w, wpitch, out, records, stream);
-    case 16: return launch_rows_gw<Real, FERN, QUAD, 16>(d, x, vertices, w, wpitch, out, records, stream);
-    default: return launch_rows_gw<Real, FERN, QUAD, 8>(d, x, vertices, w, wpitch, out, records, stream);
+    case 64: return launch_rows_gw<Real, FERN, QUAD, 64>(d, x, vertices, w, wpitch, shifted, out, records, stream);
+    case 32: return launch_rows_gw<Real, FERN, QUAD, 32>(d, x, vertices, w, wpitch, shifted, out, records, stream);
+    case 16: return launch_rows_gw<Real, FERN, QUAD, 16>(d, x, vertices, w, wpitch, shifted, out, records, stream);
+    default: return launch_rows_gw<Real, FERN, QUAD, 8>(d, x, vertices, w, wpitch, shifted, out, records, stream);
   }
 }
 
@@ -861,14 +986,24 @@ size_t forest_forward_workspace(const ForestDims &d) {
   return vertex_bytes<Real>(d) + (p != d.M ? align_up(size_t(d.T) * d.L * p * sizeof(Real), 256) : 0);
 }
 
+// An odd number (> 1) of outputs per leaf goes out in pairs where every sample's row of the output starts on an even
+// element (even tree count), the output is aligned for pairs, and the leaf table is copied to an even pitch with room
+// for the shift of the odd trees' rows.
+template <typename Real>
+static bool odd_pairs_ok(const ForestDims &d, int wpitch, const Real *out) {
+  return d.M > 1 && (d.M & 1) && d.M + 1 <= kWave / 2 && (d.T & 1) == 0 && wpitch != d.M && wpitch % 2 == 0 && wpitch >= d.M + 1 &&
+         reinterpret_cast<uintptr_t>(out) % (2 * sizeof(Real)) == 0;
+}
+
+// shift_odd (with L = rows per tree): the rows of odd trees start at element 1 of their pitch, see forward_rows_kernel.
 template <typename Real>
 __global__ __launch_bounds__(256) void pad_rows_kernel(const Real *__restrict__ w, Real *__restrict__ dst, long long rows,
-                                                       int M, int P) {
+                                                       int M, int P, bool shift_odd, int L) {
   const long long n = rows * P;
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
     const long long r = i / P;
-    const int m = int(i - r * P);
-    dst[i] = m < M ? w[r * M + m] : Real(0);
+    const int m = int(i - r * P) - ((shift_odd && ((r / L) & 1)) ? 1 : 0);
+    dst[i] = (m >= 0 && m < M) ? w[r * M + m] : Real(0);
   }
 }
 
@@ -901,6 +1036,9 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: an image result needs inner data positions (inData of 3 or more dimensions).");
   if (rows_ok<Real>(d)) {
     int wpitch = weight_pitch<Real>(d);
+    const bool shifted =
+        odd_pairs_ok<Real>(d, wpitch, out) &&
+        (reinterpret_cast<uintptr_t>(ws) + vertex_bytes<Real>(d)) % (2 * sizeof(Real)) == 0;  // the padded table
     if (wpitch != d.M) {
       Real *padded = reinterpret_cast<Real *>(static_cast<unsigned char *>(ws) + vertex_bytes<Real>(d));
       const long long rows = (long long)d.T * d.L;
@@ -915,7 +1053,7 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
         long long blocks = (rows * wpitch + 255) / 256;
         if (blocks > 16 * kNumCUs) blocks = 16 * kNumCUs;
         hipLaunchKernelGGL(pad_rows_kernel<Real>, dim3((unsigned)blocks), dim3(256), 0, stream, w, padded, rows, d.M,
-                           wpitch);
+                           wpitch, shifted, d.L);
       }
       HT_LAUNCH_CHECK("pad leaf rows");
       w = padded;
@@ -927,13 +1065,13 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
         hipLaunchKernelGGL(pack_quads_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, thr, ord,
                            static_cast<QuadNode *>(ws), d.T, d.V, NQ, d.F, slots);
         HT_LAUNCH_CHECK("pack two-level vertices");
-        return dispatch_rows<Real, false, true>(d, x, ws, w, wpitch, out, records, stream);
+        return dispatch_rows<Real, false, true>(d, x, ws, w, wpitch, shifted, out, records, stream);
       }
     }
     int rc = pack_nodes<Real>(d, thr, ord, ws, stream, slots);
     if (rc != HT_OK) return rc;
-    return fern ? dispatch_rows<Real, true, false>(d, x, ws, w, wpitch, out, records, stream)
-                : dispatch_rows<Real, false, false>(d, x, ws, w, wpitch, out, records, stream);
+    return fern ? dispatch_rows<Real, true, false>(d, x, ws, w, wpitch, shifted, out, records, stream)
+                : dispatch_rows<Real, false, false>(d, x, ws, w, wpitch, shifted, out, records, stream);
   }
   int rc = pack_nodes<Real>(d, thr, ord, ws, stream, slots);
   if (rc != HT_OK) return rc;

@@ -85,9 +85,10 @@ __global__ __launch_bounds__(kReachThreads) void reach_histogram_kernel(const ui
   }
 }
 
-// The histogram needs 16-bit keys and a tree's counters in LDS, and pays off once there are enough pairs.
+// The histogram needs 16-bit keys and a tree's counters in LDS, and pays off once there are enough pairs and a tree
+// sees more samples than it has counters to clear and flush.
 inline bool reach_by_histogram(const ForestDims &d) {
-  return d.L <= 65536 && size_t(d.L) * 4 <= kLdsBytes && d.S * (long long)d.T >= (1 << 16);
+  return d.L <= 65536 && size_t(d.L) * 4 <= kLdsBytes && d.S * (long long)d.T >= (1 << 16) && d.S >= 2LL * d.L;
 }
 
 template <typename Real, bool FERN, int BT, bool XLDS>

@@ -161,6 +161,26 @@ def test_backward_row_widths(dev, M, B, fern):
             assert rel_err(got.cpu().double(), want.double()) <= 1e-5
 
 
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("T", [2, 10, 13, 40, 262])
+@pytest.mark.parametrize("M", [3, 5, 7, 9, 11, 15, 17, 33])
+def test_forward_odd_row_widths(dev, M, T, dtype, fern):
+    """An odd number of outputs per leaf is written in pairs where the tree count is even (the leaf table is copied
+    with the odd trees' rows shifted by one element, so that every pair is one aligned gather and one aligned store)
+    and element by element where it is odd; either way bit for bit the reference's products, with and without walk
+    records, on a ragged last tile."""
+    B, F, D = 203, 24, 4          # enough samples per leaf for the padded copy of the leaf table
+    x, thr, ordn, w, _ = make_forest(B, F, [], T, D, [M], fern, dtype, seed=M * 1000 + T)
+    ref = ho.forward(x, thr, ordn, w, fern)
+    gx, gthr, gord, gw = _gpu(dev, x, thr, ordn, w)
+    pre = "fern_" if fern else "tree_"
+    out = getattr(ops, pre + "forward")(gx, gthr, gord, gw)
+    assert torch.equal(out.cpu(), ref)
+    out2, _ = getattr(ops, pre + "forward_records")(gx, gthr, gord, gw)
+    assert torch.equal(out2.cpu(), ref)
+
+
 def _same_or_nan(a, b):
     return bool(((a == b) | (a.isnan() & b.isnan())).all())
 
@@ -342,8 +362,9 @@ EMPTY = {"no samples": (0, 5, [], 3, 2, []), "no inner positions": (4, 5, [0], 3
 
 
 # B, F, K dims, T, depth: launches with 2^16 (sample, tree) pairs and more count reachability as a histogram of 16-bit
-# leaf keys when a tree's counters fit the LDS (depth <= 15); below that, and at depth 16, by one atomic per pair.
-REACH = [(30000, 12, [], 5, 6), (30001, 12, [], 5, 6), (700, 9, [5, 3], 11, 4), (9000, 20, [], 9, 15),
+# leaf keys when a tree's counters fit the LDS (depth <= 15) and the tree sees at least two samples per counter; below
+# that, and at depth 16, by one atomic per pair.
+REACH = [(30000, 12, [], 5, 6), (30001, 12, [], 5, 6), (700, 9, [5, 3], 11, 4), (70000, 20, [], 3, 15), (9000, 20, [], 9, 15),
          (5000, 20, [], 14, 16), (262144, 4, [], 1, 2), (70000, 6, [], 1, 1)]
 
 
@@ -352,7 +373,7 @@ REACH = [(30000, 12, [], 5, 6), (30001, 12, [], 5, 6), (700, 9, [5, 3], 11, 4), 
 def test_reachability_counts(dev, case, fern):
     B, F, Kd, T, D = case
     x, thr, ordn, w, _ = make_forest(B, F, Kd, T, D, [1], fern, torch.float32, seed=11)
-    if case == REACH[5]:
+    if B == 262144:
         thr[:] = 1e9                                    # every sample of the batch in the same leaf of each tree
     ref_reach = ho.maps(x, thr, ordn, w, fern)[3].to(torch.int64)
     gx, gthr, gord, gw = _gpu(dev, x, thr, ordn, w)
@@ -360,7 +381,7 @@ def test_reachability_counts(dev, case, fern):
     for _ in range(2):                                  # the workspace of the first call is reused by the second
         reach = getattr(ops, pre + "reachability")(gx, gthr, gord, gw)
         assert reach.dtype == torch.int64 and torch.equal(reach.cpu(), ref_reach)
-    if case == REACH[5]:
+    if B == 262144:
         assert int(reach.max()) == B
 
 
