@@ -14,6 +14,7 @@ HT_F32, HT_F64 = 0, 1
 HT_TREE, HT_FERN = 0, 1
 HT_BACKWARD_ATOMIC, HT_BACKWARD_DETERMINISTIC = 0, 1
 HT_MAX_CONV_DIMS = 3
+HT_ABI_VERSION = 2  # of include/hingetree_hip.h as this file mirrors it; load() refuses a library built from another
 
 
 class ForestShape(ctypes.Structure):
@@ -101,6 +102,9 @@ def load():
             fn = getattr(lib, name)  # AttributeError here means the library and the header disagree
             fn.restype = res
             fn.argtypes = args
+        if lib.ht_abi_version() != HT_ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH} has ABI version {lib.ht_abi_version()}, this package expects "
+                               f"{HT_ABI_VERSION}: run `python -m hingetreefortorch_amd.build`.")
         _lib = lib
     return _lib
 

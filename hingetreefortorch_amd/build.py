@@ -83,7 +83,7 @@ def build_host(verbose=True):
     tmp = HOST_PATH + ".tmp"
     cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-w",
            "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_hingetree_host",
-           "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=1",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch.compiled_with_cxx11_abi()),
            "-I" + os.path.join(torch_dir, "include"),
            "-I" + os.path.join(torch_dir, "include", "torch", "csrc", "api", "include"),
            "-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(rocm, "include"),

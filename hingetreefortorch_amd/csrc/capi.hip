@@ -3,6 +3,8 @@
 #include <cstring>
 #include <limits>
 #include <mutex>
+#include <set>
+#include <utility>
 
 #include "common.hpp"
 
@@ -164,6 +166,24 @@ static int static_scratch(void **ptr) {
   return HT_OK;
 }
 
+// ---- dynamic LDS limit of a kernel, granted once per kernel and device -------------------------------------------
+hipError_t grant_lds(const void *kernel) {
+  static std::mutex mutex;
+  static std::set<std::pair<int, const void *>> granted;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  std::lock_guard<std::mutex> lock(mutex);
+  const std::pair<int, const void *> key(dev, kernel);
+  if (granted.count(key)) return hipSuccess;
+  hipFuncAttributes attr;
+  if ((e = hipFuncGetAttributes(&attr, kernel)) != hipSuccess) return e;
+  const int room = kLdsBytes - int(attr.sharedSizeBytes);  // what the kernel's static arrays leave
+  if ((e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, room)) != hipSuccess) return e;
+  granted.insert(key);
+  return hipSuccess;
+}
+
 }  // namespace ht
 
 using namespace ht;
@@ -171,7 +191,7 @@ using namespace ht;
 extern "C" {
 
 const char *ht_last_error(void) { return g_last_error.c_str(); }
-int ht_abi_version(void) { return 1; }
+int ht_abi_version(void) { return HT_ABI_VERSION; }
 
 int ht_check_device(int32_t device) {
   hipDeviceProp_t prop;

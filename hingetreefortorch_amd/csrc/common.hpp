@@ -175,6 +175,11 @@ int projection_backward(long long B, long long K, long long N, const float *x, c
 int gemm_tile_map(int tiles_i, int tiles_j, int *tile_i, int *tile_j);
 int ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, hipStream_t stream);
 
+// Lets `kernel` use all of a workgroup's LDS as dynamic shared memory. The runtime call behind it is made once per
+// kernel and device, not per launch: later launches -- also those recorded into a HIP graph -- make no attribute
+// calls at all.
+hipError_t grant_lds(const void *kernel);
+
 // Fills `bytes` bytes with zero through a kernel (safe to record into a HIP graph, unlike a memset node).
 int zero_fill(void *p, size_t bytes, hipStream_t stream);
 

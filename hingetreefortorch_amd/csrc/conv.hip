@@ -894,8 +894,7 @@ int conv_forward(const ht_conv_shape &s, const Real *x, const Real *thr, const i
       auto kernel = fern ? conv_tiled_forward_kernel<Real, true, 16> : conv_tiled_forward_kernel<Real, false, 16>;
       if (s.M == 1) kernel = fern ? conv_tiled_forward_kernel<Real, true, 1> : conv_tiled_forward_kernel<Real, false, 1>;
       else if (s.M <= 4) kernel = fern ? conv_tiled_forward_kernel<Real, true, 4> : conv_tiled_forward_kernel<Real, false, 4>;
-      HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lay.total)));
+      HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
       hipLaunchKernelGGL(kernel, tgrid, dim3(kConvThreads), lay.total, stream, t, lay, int(s.C), c_per, int(s.Cout),
                          int(s.depth), V, L, int(s.M), j_per, x, thr, ord, w, out);
       HT_LAUNCH_CHECK("conv forward (tiled)");
@@ -920,8 +919,7 @@ int launch_conv_backward(const ConvGeom &g, const ht_conv_shape &s, int V, int L
                          Real *dw, hipStream_t stream) {
   const dim3 grid((g.rows + kConvThreads - 1) / kConvThreads, (unsigned)s.Cout, (unsigned)s.B);
   auto kernel = conv_backward_kernel<Real, FERN, LDS_ACC>;
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   int(lds)));
+  HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   hipLaunchKernelGGL(kernel, grid, dim3(kConvThreads), lds, stream, g, int(s.C), int(s.Cout), int(s.depth), V, L,
                      int(s.M), x, thr, ord, w, gout, dx, dthr, dw);
   HT_LAUNCH_CHECK("conv backward");
@@ -977,8 +975,7 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
         kernel = fern ? conv_tiled_backward_kernel<Real, true, kConvThreads, true>
                       : conv_tiled_backward_kernel<Real, false, kConvThreads, true>;
     }
-    HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(lay.total)));
+    HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
     hipLaunchKernelGGL(kernel, grid, dim3(threads), lay.total, stream, t, lay, int(s.C), c_per, int(s.Cout),
                        int(s.depth), V, L, int(s.M), j_per, x, thr, ord, w, gout, dx, dthr, dw);
     HT_LAUNCH_CHECK("conv backward (one walk, tiled)");
@@ -994,8 +991,7 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
         const int j_per = conv_j_per(tiles * s.B, int(s.Cout));
         const dim3 grid((unsigned)tiles, (unsigned)((s.Cout + j_per - 1) / j_per), (unsigned)s.B);
         auto kernel = fern ? conv_tiled_dx_kernel<Real, true> : conv_tiled_dx_kernel<Real, false>;
-        HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(lay_x.total)));
+        HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
         hipLaunchKernelGGL(kernel, grid, dim3(kConvThreads), lay_x.total, stream, t, lay_x, int(s.C), int(s.Cout),
                            int(s.depth), V, L, int(s.M), j_per, x, thr, ord, w, gout, dx);
         HT_LAUNCH_CHECK("conv backward (dX, tiled)");
@@ -1008,8 +1004,7 @@ int conv_backward(const ht_conv_shape &s, const Real *x, const Real *thr, const 
         if (parts < 1) parts = 1;
         const dim3 grid((unsigned)s.Cout, (unsigned)parts);
         auto kernel = fern ? conv_tiled_trees_kernel<Real, true> : conv_tiled_trees_kernel<Real, false>;
-        HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(lay_t.total)));
+        HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
         hipLaunchKernelGGL(kernel, grid, dim3(kConvThreads), lay_t.total, stream, t, lay_t, int(s.C), int(s.Cout),
                            int(s.depth), V, L, int(s.M), items, x, thr, ord, w, gout, dthr, dw);
         HT_LAUNCH_CHECK("conv backward (trees, tiled)");

@@ -84,8 +84,7 @@ int launch_records(const ForestDims &d, const Real *x, const Node<Real> *nodes, 
   split_trees(tiles, d.T, TP, &trees_per_block, &gy);
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
   auto kernel = records_kernel<Real, FERN, BT, XLDS, COMPACT>;
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   int(lds)));
+  HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, nodes, rec,
                      trees_per_block);
   HT_LAUNCH_CHECK("forest walk records");
@@ -1549,8 +1548,7 @@ int launch_backward_fused(const ForestDims &d, const Real *x, const Node<Real> *
   split_trees(tiles, d.T, TC, &trees_per_block, &gy);
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
   auto kernel = backward_fused_kernel<Real, FERN, BT, XLDS>;
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   int(lds)));
+  HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, nodes, w, gout,
                      dx, dthr, dw, trees_per_block, FastDiv(d.M));
   HT_LAUNCH_CHECK("forest backward (fused, atomics)");
@@ -1818,8 +1816,7 @@ int launch_tree_kernel_u(const ForestDims &d, const TreePlan &p, int P, const Re
                          Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
                          bool need_c, hipStream_t stream) {
   auto kernel = tree_kernel<Real, COMPACT, FIXED, U>;
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   int(p.lds)));
+  HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
   hipLaunchKernelGGL(kernel, dim3((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts), dim3(kForestThreads), p.lds,
                      stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB, p.part_size, need_c, p.parts > 1, P, p.groups,
@@ -1884,8 +1881,7 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
 #define HT_LEAN_LAUNCH(MM, WLDS_)                                                                                     \
   {                                                                                                                   \
     auto kernel = tree_lean_kernel<MM, FIXED, WLDS_>;                                                                 \
-    HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                                          \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));                          \
+    HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));                          \
     hipLaunchKernelGGL(kernel, grid, dim3(kForestThreads), lds, stream, d, w, gout, rec, dw, dw_fixed, hdr, log2_tb,  \
                        p.part_size, need_c, p.parts > 1, p.groups, dthr_fold, uint32_t(thr_off), uint32_t(w_off),     \
                        second_run);                                                                                   \
@@ -1916,8 +1912,7 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
 #define HT_WIDE(PP)                                                                                                   \
   case PP: {                                                                                                          \
     auto kernel = gout_image ? tree_wide_kernel<PP, FIXED, true> : tree_wide_kernel<PP, FIXED, false>;                \
-    HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                                          \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(p.lds)));                        \
+    HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));                        \
     hipLaunchKernelGGL(kernel, grid, dim3(kForestThreads), p.lds, stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB,   \
                        p.part_size, need_c, p.parts > 1, p.groups, img);                                              \
     break;                                                                                                            \
@@ -1957,8 +1952,7 @@ int launch_dx(const ForestDims &d, Records<Real, COMPACT> rec, Real *dx, const D
     if (windows > 1) kernel = dx_kernel<Real, BT, COMPACT, FIXED, true>;
   }
   if (BT != 8 && windows > 1) return fail(HT_ERR_RUNTIME, "Error: feature windows on a tile other than the smallest.");
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   int(lds)));
+  HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)windows), dim3(kForestThreads), lds, stream, d, rec, dx, hdr,
                      f_per);
   HT_LAUNCH_CHECK("forest backward (dX)");
@@ -2109,8 +2103,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
       const size_t need = size_t(d.L) * d.M * sizeof(Real);
       if (need <= size_t(kLdsBytes) / 3) {
         auto kernel = det_tree_kernel<Real, true, COMPACT>;
-        HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(need)));
+        HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
         hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, (Real *)nullptr,
                            dw, &hdr->fallback_w);
       } else {
@@ -2132,8 +2125,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
     const size_t thr_lds = size_t((d.V + vslices - 1) / vslices) * sizeof(double);
     if ((long long)d.T * vslices > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many trees for one launch.");
     auto thr_kernel = vslices > 1 ? dthr_kernel<Real, COMPACT, FIXED, true> : dthr_kernel<Real, COMPACT, FIXED, false>;
-    HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(thr_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(thr_lds)));
+    HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(thr_kernel)));
     hipLaunchKernelGGL(thr_kernel, dim3((unsigned)(d.T * vslices), (unsigned)dthr_gy), dim3(256), thr_lds, stream, d,
                        rec, dthr, dthr_fixed, hdr, dthr_part, dthr_gy > 1, vslices);
     HT_LAUNCH_CHECK("forest backward (dThr)");
@@ -2147,8 +2139,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
       const size_t need = size_t(d.V) * sizeof(Real);
       if (need <= size_t(kLdsBytes) / 3) {
         auto kernel = det_tree_kernel<Real, true, COMPACT>;
-        HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(need)));
+        HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
         hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, dthr,
                            (Real *)nullptr, &hdr->fallback_c);
       } else {
@@ -2196,8 +2187,7 @@ int backward_sequential(const ForestDims &d, const Real *x, const Node<Real> *no
     const size_t need = (dw ? size_t(d.L) * d.M : 0) * sizeof(Real) + (dthr ? size_t(d.V) : 0) * sizeof(Real);
     if (need <= size_t(kLdsBytes) / 3) {
       auto kernel = det_tree_kernel<Real, true, COMPACT>;
-      HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(need)));
+      HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
       hipLaunchKernelGGL(kernel, dim3((unsigned)d.T), dim3(kWave), need, stream, d, w, gout, rec, dthr, dw,
                          (const int *)nullptr);
     } else {

@@ -517,6 +517,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
   for (int tb = t_begin + wave * TPW; tb < t_end; tb += kWaves * TPW) {
     // ---- walk: this lane's sample through trees tb + slot + i * SLOTS
     {
+      __builtin_amdgcn_s_setprio(0);
       WalkResult<Real> r[kRowIlp];
       int t[kRowIlp];
 #pragma unroll
@@ -599,6 +600,11 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
     // ---- output: out[s0 + jj, tb .. tb + nt, 0 .. M) is one contiguous run per sample
+    // A wavefront in this phase issues few instructions and waits on memory in between; with the higher priority its
+    // gathers and stores are issued as soon as their operands are there instead of queueing behind the walks of the
+    // SIMD's other wavefronts (forward at 65536 x 1024 features, 1000 trees of depth 10, 10 outputs: 0.958 -> 0.931 ms;
+    // the opposite order of priorities changes nothing).
+    __builtin_amdgcn_s_setprio(3);
     const int nt = min(TPW, t_end - tb);
     Real *obase = out + ((long long)s0 * d.T + tb) * d.M;
     const Real *wbase = w + (long long)tb * d.L * wpitch;  // wpitch: elements between leaf rows (M, or padded)
@@ -805,8 +811,7 @@ int launch_rows(const ForestDims &d, const Real *x, const void *vertices, const 
   auto kernel = forward_rows_kernel<Real, FERN, QUAD, BT, GW, ODD, RECORD, COMPACT>;
   Records<Real, COMPACT> rec{};
   if (RECORD) rec = carve_records<Real, COMPACT>(d, records, nullptr);
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   int(lds)));
+  HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, vertices,
                      int(quads_per_tree(d.depth)), w, out, rec, trees_per_block, FastDiv(d.M),
                      FastDiv(TPW * d.M / GW), wpitch);
@@ -865,8 +870,7 @@ int launch_forward_vw(const ForestDims &d, const Real *x, const Node<Real> *node
   auto kernel = forward_kernel<Real, FERN, BT, XLDS, ILP, KeyT, VW, NT, RECORD, COMPACT>;
   Records<Real, COMPACT> rec{};
   if (RECORD) rec = carve_records<Real, COMPACT>(d, records, nullptr);
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   int(lds)));
+  HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(NT), lds, stream, d, x, nodes, w, out, rec,
                      trees_per_block, FastDiv(d.M), img);
   HT_LAUNCH_CHECK("forest forward");

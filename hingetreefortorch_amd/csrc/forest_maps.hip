@@ -104,8 +104,7 @@ int launch_maps(const ForestDims &d, const Real *x, const Real *thr, const int64
   const int gy = (d.T + trees_per_block - 1) / trees_per_block;
   if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
   auto kernel = maps_kernel<Real, FERN, BT, XLDS>;
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   int(lds)));
+  HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, thr, ord,
                      leafmap, margins, ordinals, reinterpret_cast<unsigned long long *>(reach), keys,
                      trees_per_block);
@@ -224,8 +223,7 @@ int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, 
   per_part = (per_part + 7) / 8 * 8;
   parts = (d.S + per_part - 1) / per_part;
   const size_t lds = size_t(d.L) * 4;
-  HT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(reach_histogram_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
+  HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(reach_histogram_kernel)));
   hipLaunchKernelGGL(reach_histogram_kernel, dim3((unsigned)d.T, (unsigned)parts), dim3(kReachThreads), lds, stream,
                      keys, (long long)d.S, d.L, per_part, reinterpret_cast<unsigned long long *>(reach));
   HT_LAUNCH_CHECK("reachability histogram");

@@ -274,10 +274,17 @@ py::list forest_backward_records(int kind, int mode, const torch::Tensor &record
                                  bool bInDataGrad, const torch::Tensor &inThresholds, bool bInThresholdsGrad,
                                  const torch::Tensor &inOrdinals, bool bInOrdinalsGrad, const torch::Tensor &inWeights,
                                  bool bInWeightsGrad, const torch::Tensor &outDataGrad) {
+  // the library reads `records` as raw bytes through a device pointer: anything but the byte buffer a forward pass
+  // filled, on the data's device, is refused here instead of reaching a kernel
+  if (!records.defined() || records.scalar_type() != torch::kUInt8 || !records.is_contiguous())
+    invalid("Error: records must be the contiguous uint8 tensor a *_forward_records call returned.");
+  if (records.device() != inData.device()) invalid("Error: records and inData are on different devices.");
   common_checks({&inData, &inThresholds, &inWeights, &outDataGrad}, inOrdinals, true);
   if (bInOrdinalsGrad) runtime("Error: Gradient on inOrdinals is requested, but inOrdinals never has a gradient.");
   std::vector<int64_t> out_sizes;
   const ht_forest_shape s = forest_shape(kind, inData, inThresholds, inOrdinals, inWeights, &outDataGrad, &out_sizes);
+  if (size_t(records.numel()) != ht_forest_records_bytes(&s))
+    invalid("Error: records do not belong to a forest of this shape.");
   const c10::DeviceGuard guard(inData.device());
   torch::Tensor dx = bInDataGrad ? torch::empty_like(inData) : torch::Tensor();
   torch::Tensor dthr = bInThresholdsGrad ? torch::empty_like(inThresholds) : torch::Tensor();
@@ -459,7 +466,7 @@ py::list conv_backward(int kind, int nd, const torch::Tensor &inData, bool bInDa
 // not defined here (the Python layer's stubs raise for them).
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "native host of hingetree_cpp (forest / fern / convolution path) over libhingetree_hip.so";
-  m.attr("abi_version") = ht_abi_version();
+  m.attr("abi_version") = HT_ABI_VERSION;  // of the header this module was compiled against, not of the loaded library
   m.def("forget_ordinal_checks", &forget_ordinal_checks);
 
   m.def("forest_forward", &forest_forward);

@@ -585,10 +585,18 @@ def _forward_records(kind, inData, inThresholds, inOrdinals, inWeights):
 def _backward_records(kind, mode, records, inData, bInDataGrad, inThresholds, bInThresholdsGrad, inOrdinals,
                       bInOrdinalsGrad, inWeights, bInWeightsGrad, outDataGrad):
     """`_backward` from the records of `_forward_records`; inData / inThresholds / inOrdinals only give shapes."""
+    # the library reads `records` as raw bytes through a device pointer: anything but the byte buffer a forward pass
+    # filled, on the data's device, is refused here instead of reaching a kernel
+    if not isinstance(records, torch.Tensor) or records.dtype != torch.uint8 or not records.is_contiguous():
+        _invalid("Error: records must be the contiguous uint8 tensor a *_forward_records call returned.")
+    if records.device != inData.device:
+        _invalid("Error: records and inData are on different devices.")
     _common_checks([inData, inThresholds, inWeights, outDataGrad], inOrdinals, True)
     if bInOrdinalsGrad:
         _runtime("Error: Gradient on inOrdinals is requested, but inOrdinals never has a gradient.")
     shape, _ = _forest_shape(kind, inData, inThresholds, inOrdinals, inWeights, outDataGrad)
+    if records.numel() != L.load().ht_forest_records_bytes(ctypes.byref(shape)):
+        _invalid("Error: records do not belong to a forest of this shape.")
     with torch.cuda.device(inData.device):
         dx = torch.empty_like(inData) if bInDataGrad else None
         dthr = torch.empty_like(inThresholds) if bInThresholdsGrad else None
@@ -961,7 +969,7 @@ host = "python"
 def _load_native():
     try:
         from . import _hingetree_host as native
-    except ImportError:
+    except (ImportError, OSError):  # not built, or built against libraries that are not there any more
         return None
     if native.abi_version != L.load().ht_abi_version():
         raise RuntimeError("hingetreefortorch_amd/_hingetree_host.so was built against another libhingetree_hip.so; "

@@ -181,6 +181,26 @@ def test_forward_odd_row_widths(dev, M, T, dtype, fern):
     assert torch.equal(out2.cpu(), ref)
 
 
+@pytest.mark.parametrize("fern", [False, True], ids=["tree", "fern"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("F", [1024, 1500, 4000])
+@pytest.mark.parametrize("M", [3, 9, 15])
+def test_forward_odd_row_widths_on_every_tile(dev, M, F, dtype, fern):
+    """The same on the smaller sample tiles that wide feature spaces force (64 / 32 / 16 / 8 samples by F and dtype):
+    there a wavefront's step holds 8, 16 or 32 trees and the generic pair loop runs instead of the unrolled one; with
+    F = 1024 float trees walk two-level vertices. Even tree count, padded (and shifted) leaf table, ragged last tile."""
+    B, T, D = 203, 40, 4
+    x, thr, ordn, w, _ = make_forest(B, F, [], T, D, [M], fern, dtype, seed=M * 100 + F)
+    ref = ho.forward(x, thr, ordn, w, fern)
+    gx, gthr, gord, gw = _gpu(dev, x, thr, ordn, w)
+    pre = "fern_" if fern else "tree_"
+    print(f"case odd rows on tiles: F={F} M={M} {dtype} fern={fern}", flush=True)
+    out = getattr(ops, pre + "forward")(gx, gthr, gord, gw)
+    assert torch.equal(out.cpu(), ref)
+    out2, _ = getattr(ops, pre + "forward_records")(gx, gthr, gord, gw)
+    assert torch.equal(out2.cpu(), ref)
+
+
 def _same_or_nan(a, b):
     return bool(((a == b) | (a.isnan() & b.isnan())).all())
 

@@ -27,7 +27,17 @@ def test_library_exports_header_symbols():
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert _lib.load().ht_abi_version() == 1
+    # the library, the header and the Python mirror of the header carry the same version number
+    assert int(re.search(r"#define HT_ABI_VERSION (\d+)", header).group(1)) == _lib.HT_ABI_VERSION
+    assert _lib.load().ht_abi_version() == _lib.HT_ABI_VERSION
+
+
+def test_stale_library_is_refused(monkeypatch):
+    """A library built from another version of the header is refused when it is loaded, with the way out named."""
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "HT_ABI_VERSION", _lib.HT_ABI_VERSION + 1)
+    with pytest.raises(RuntimeError, match="ABI version"):
+        _lib.load()
 
 
 def test_no_fallback_when_library_missing(monkeypatch):
@@ -76,6 +86,22 @@ def test_validation_order_on_cpu_tensors(either_host):
         ops.tree_fused_linear_backward(x, True, thr, True, ordn, True, w, True, lin, True, bias, True, torch.randn(8, 4))
     with pytest.raises(RuntimeError, match="no CPU back-end"):
         ops.tree_fused_linear_forward(x, thr, ordn, w, lin, bias)
+
+
+def test_records_are_validated_before_any_launch(either_host):
+    """*_backward_records hands `records` to the kernels as raw bytes: a tensor that is not the contiguous uint8 buffer
+    of a forward pass, or lives elsewhere than the data, raises ValueError in the host layer (no GPU involved)."""
+    x, thr, ordn, w, gout = make_forest(8, 5, [], 3, 2, [], False, torch.float32)
+    args = (x, True, thr, True, ordn, False, w, True, gout)
+    with pytest.raises(ValueError, match="contiguous uint8"):
+        ops.tree_backward_records(torch.zeros(64, dtype=torch.float32), False, *args)
+    with pytest.raises(ValueError, match="contiguous uint8"):
+        ops.fern_backward_records(torch.zeros(64, 2, dtype=torch.uint8)[:, 0], True, *args)
+    with pytest.raises(ValueError, match="different devices"):
+        ops.tree_backward_records(torch.zeros(64, dtype=torch.uint8, device="meta"), False, *args)
+    # a well-formed buffer goes on to the usual checks (here: the refusal to compute on the CPU)
+    with pytest.raises(RuntimeError, match="no CPU back-end"):
+        ops.tree_backward_records(torch.zeros(64, dtype=torch.uint8), False, *args)
 
 
 def test_conv_validation_on_cpu_tensors(either_host):
@@ -248,3 +274,18 @@ def test_gemm_tile_map_is_a_bijection():
     small = np.empty(8, dtype=np.int32)
     assert lib.ht_gemm_tile_map(128, 100, small.ctypes.data_as(ctypes.c_void_p), small.ctypes.data_as(ctypes.c_void_p),
                                 8) == _lib.HT_ERR_INVALID_ARGUMENT
+
+
+def test_library_sources_never_allocate_device_memory():
+    """The C ABI promises that nothing in the library allocates or frees device memory (callers bring workspaces, or
+    use the static one): no allocating or memset runtime call appears anywhere under csrc/."""
+    import glob
+    import os
+    import re
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "hingetreefortorch_amd", "csrc")
+    files = glob.glob(os.path.join(root, "*.hip")) + glob.glob(os.path.join(root, "*.hpp"))
+    assert files
+    banned = re.compile(r"\bhip(Malloc\w*|Free\w*|Memset\w*|HostMalloc|HostAlloc|ExtMallocWithFlags)\s*\(")
+    for f in files:
+        text = open(f).read()
+        assert not banned.search(text), f

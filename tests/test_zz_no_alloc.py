@@ -40,10 +40,17 @@ def _both(lib, B, F, T, D, M, dtype, kind, seed):
     _lib.check(lib.ht_forest_forward(ctypes.byref(s), _ptr(x), _ptr(thr), _ptr(ordn), _ptr(w), _ptr(want), _ptr(ws),
                                      need, stream))
     torch.cuda.synchronize()
+    # a first call loads the kernels' code objects and looks up the static array; the call that is measured comes after
+    _lib.check(lib.ht_forest_forward_static(ctypes.byref(s), _ptr(x), _ptr(thr), _ptr(ordn), _ptr(w), _ptr(got), stream))
+    torch.cuda.synchronize()
+    got.fill_(float("nan"))
+    torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]          # the device's own count: sees allocations torch does not make
     _lib.check(lib.ht_forest_forward_static(ctypes.byref(s), _ptr(x), _ptr(thr), _ptr(ordn), _ptr(w), _ptr(got), stream))
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     assert not torch.isnan(want).any()
     assert torch.equal(got, want), f"static forward differs: B={B} F={F} T={T} D={D} M={M} {dtype} kind={kind}"
 
@@ -70,3 +77,47 @@ def test_static_forward_limits():
     # an empty shape is the set-up call: no launch, no pointers needed
     e = _shape(0, 16, 4, 3, 2, torch.float32, _lib.HT_TREE)
     assert lib.ht_forest_forward_static(ctypes.byref(e), None, None, None, None, None, None) == _lib.HT_OK
+
+
+def test_static_forward_under_graph_capture():
+    """The entry point is meant for code under HIP graph capture: after the set-up call it makes no runtime call but
+    kernel launches on the caller's stream. Captured once, replayed three times with eager work in between, each
+    replay bit for bit the eager result; then new inputs in the captured buffers."""
+    lib = _lib.load()
+    B, F, T, D, M = 4096, 64, 64, 6, 10
+    x, thr, ordn, w = _forest(B, F, T, D, M, torch.float32, _lib.HT_TREE, seed=21)
+    s = _shape(B, F, T, D, M, torch.float32, _lib.HT_TREE)
+    e = _shape(0, F, T, D, M, torch.float32, _lib.HT_TREE)
+    assert lib.ht_forest_forward_static(ctypes.byref(e), None, None, None, None, None, None) == _lib.HT_OK  # set-up
+    out = torch.full((B, T, M), float("nan"), dtype=torch.float32, device="cuda")
+
+    def call():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        _lib.check(lib.ht_forest_forward_static(ctypes.byref(s), _ptr(x), _ptr(thr), _ptr(ordn), _ptr(w), _ptr(out),
+                                                stream))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()                                           # eager, also loads the kernels before the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    want = out.clone()
+    assert not torch.isnan(want).any()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for replay in range(3):
+        x.mul_(1.0)
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), replay
+    x.copy_(torch.randn(x.shape, generator=torch.Generator().manual_seed(5)).cuda())
+    graph.replay()
+    torch.cuda.synchronize()
+    replayed = out.clone()
+    call()
+    torch.cuda.synchronize()
+    assert torch.equal(replayed, out)
