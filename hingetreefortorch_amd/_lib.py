@@ -60,7 +60,7 @@ SIGNATURES = {
     "ht_forest_forward_records": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _SZ, _P, _SZ, _P]),
     "ht_forest_backward_records_workspace": (_SZ, [ctypes.POINTER(ForestShape), _I, _I, _I, _I]),
     "ht_forest_backward_records": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _SZ, _P, _P, _P, _I, _P, _SZ, _P]),
-    "ht_forest_maps_workspace": (_SZ, [ctypes.POINTER(ForestShape)]),
+    "ht_forest_maps_workspace": (_SZ, [ctypes.POINTER(ForestShape), ctypes.c_int32]),
     "ht_forest_maps": (_I, [ctypes.POINTER(ForestShape), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "ht_conv_output_size": (_I, [ctypes.POINTER(ConvShape), ctypes.POINTER(ctypes.c_int64)]),
     "ht_conv_forward": (_I, [ctypes.POINTER(ConvShape), _P, _P, _P, _P, _P, _P]),

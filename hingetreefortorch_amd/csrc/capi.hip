@@ -406,10 +406,11 @@ int ht_forest_backward_image(const ht_forest_shape *s, const ht_tile_shape *g, c
                                 workspace_bytes, static_cast<hipStream_t>(stream), &img);
 }
 
-size_t ht_forest_maps_workspace(const ht_forest_shape *s) {
+size_t ht_forest_maps_workspace(const ht_forest_shape *s, int32_t want_reach) {
   ForestDims d;
   if (make_dims(s, &d) != HT_OK) return 0;
-  return s->dtype == HT_F32 ? forest_maps_workspace<float>(d) : forest_maps_workspace<double>(d);
+  return s->dtype == HT_F32 ? forest_maps_workspace<float>(d, want_reach != 0)
+                            : forest_maps_workspace<double>(d, want_reach != 0);
 }
 
 int ht_forest_maps(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, int64_t *leafmap,

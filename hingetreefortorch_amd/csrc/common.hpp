@@ -130,8 +130,16 @@ template <typename Real>
 int forest_backward_records(const ForestDims &d, bool fern, const Real *w, const Real *gout, const void *records,
                             Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes, hipStream_t stream);
 
+// The maps on the forward's row kernel walk (forest_forward.hip): bytes of packed vertices it wants (0: shape not
+// served), and the launch; keys16 (optional) receives the leaf keys as 16-bit values tree major.
 template <typename Real>
-size_t forest_maps_workspace(const ForestDims &d);
+size_t forest_maps_rows_workspace(const ForestDims &d);
+template <typename Real>
+int forest_maps_rows(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord,
+                     int64_t *leafmap, uint16_t *keys16, Real *margins, int64_t *ordinals, void *ws, hipStream_t stream);
+
+template <typename Real>
+size_t forest_maps_workspace(const ForestDims &d, bool want_reach);
 template <typename Real>
 int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap,
                 Real *margins, int64_t *ordinals, int64_t *reach, void *ws, size_t ws_bytes, hipStream_t stream);

@@ -407,6 +407,82 @@ __device__ __forceinline__ double value_of_next_lane(double v) {
 constexpr int kRowIlp = 4;     // trees walked concurrently per lane
 constexpr int kRowUnroll = 5;  // output vectors per lane whose weight gathers are in flight together
 
+// One step of a wavefront of the row kernels: this lane's sample (column xs_j of the tile) through the kRowIlp trees
+// tb + slot + i * SLOTS of the step's TPW = SLOTS * kRowIlp trees. stage_area is the wavefront's own piece of LDS (BT *
+// (TPW + 1) values), free while the walks run: the top quads of the step's trees (QUAD) or the vertices of its ferns
+// are copied there once per step. TRACK: also the selected vertex, its ordinal and the signed margin.
+template <typename Real, bool FERN, bool QUAD, int BT, bool TRACK>
+__device__ __forceinline__ void rows_walk_step(const ForestDims &d, const void *__restrict__ vertices, int NQ, int tb,
+                                               int t_end, int slot, int lane, const Real *xs_j, Real *stage_area,
+                                               WalkResult<Real> (&r)[kRowIlp]) {
+  constexpr int SLOTS = kWave / BT;
+  constexpr int TPW = SLOTS * kRowIlp;
+  constexpr int LDP = TPW + 1;
+  int t[kRowIlp];
+#pragma unroll
+  for (int i = 0; i < kRowIlp; ++i) t[i] = min(tb + slot + i * SLOTS, t_end - 1);  // surplus slots re-walk, unused
+  if constexpr (QUAD) {
+    const QuadNode *all = static_cast<const QuadNode *>(vertices);
+    const QuadNode *qn[kRowIlp];
+#pragma unroll
+    for (int i = 0; i < kRowIlp; ++i) qn[i] = all + (long long)t[i] * NQ;
+    // The top of every tree is the same for all samples: the wavefront copies the first quads of its TPW trees
+    // into LDS once per step (into the space of the parked results, which nobody reads before this step's walks
+    // are over), where they fit.
+    constexpr bool kTopFits = size_t(TPW) * kTopQuads * sizeof(QuadNode) <= size_t(BT) * LDP * sizeof(Real);
+    if (kTopFits && NQ >= kTopQuads) {
+      QuadNode *stage = reinterpret_cast<QuadNode *>(stage_area);
+      for (int i = lane; i < TPW * kTopQuads; i += kWave) {
+        const int tt = i / kTopQuads, q = i - tt * kTopQuads;
+        stage[i] = all[(long long)min(tb + tt, t_end - 1) * NQ + q];
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const QuadNode *top[kRowIlp];
+#pragma unroll
+      for (int i = 0; i < kRowIlp; ++i) top[i] = stage + (slot + i * SLOTS) * kTopQuads;
+      walk_quads<kRowIlp, BT, true, TRACK>(d.depth, qn, top, xs_j, r);
+      // every lane has read its quads before any lane overwrites them with results
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    } else {
+      walk_quads<kRowIlp, BT, false, TRACK>(d.depth, qn, qn, xs_j, r);
+    }
+  } else {
+    const Node<Real> *all = static_cast<const Node<Real> *>(vertices);
+    bool staged = false;
+    if constexpr (FERN) {
+      // A fern's vertex is the same for every sample, so a vector load of it would fetch one address per tree
+      // slot and still cost a full trip through the vector memory pipeline per level. Instead the wavefront
+      // copies the vertices of its TPW ferns into LDS once per step -- into the space of the parked results,
+      // which nobody reads before this step's walks are over -- and the walk reads them as LDS broadcasts.
+      Node<Real> *stage = reinterpret_cast<Node<Real> *>(stage_area);
+      if (size_t(TPW) * d.depth * sizeof(Node<Real>) <= size_t(BT) * LDP * sizeof(Real)) {
+        staged = true;
+        // level major, [level][fern]: the ferns of a lane's kRowIlp walks then lie a compile-time distance apart
+        for (int i = lane; i < TPW * d.depth; i += kWave) {
+          const int lv = i / TPW, tt = i - lv * TPW;
+          stage[i] = all[(long long)min(tb + tt, t_end - 1) * d.V + lv];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        walk_ferns_staged<Real, kRowIlp, BT, SLOTS, TPW, TRACK>(d.depth, stage + slot, xs_j, r);
+        // every lane has read its vertices before any lane overwrites them with results
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
+    if (!staged) {
+      const Node<Real> *nd[kRowIlp];
+#pragma unroll
+      for (int i = 0; i < kRowIlp; ++i) nd[i] = all + (long long)t[i] * d.V;
+      walk_many<Real, FERN, kRowIlp>(d.depth, nd, [&](int, int f) { return xs_j[f * BT]; }, r);
+    }
+  }
+}
+
 // One workgroup = one tile of BT samples (all features in LDS, feature major) x a range of trees, like
 // forward_kernel, but every wavefront works on its own: lanes = BT samples x 64/BT tree slots, each lane walks
 // kRowIlp trees, parks (|margin|, leaf) in a wavefront-private piece of LDS, and the same wavefront then writes the
@@ -519,69 +595,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
     {
       __builtin_amdgcn_s_setprio(0);
       WalkResult<Real> r[kRowIlp];
-      int t[kRowIlp];
-#pragma unroll
-      for (int i = 0; i < kRowIlp; ++i) t[i] = min(tb + slot + i * SLOTS, t_end - 1);  // surplus slots re-walk, unused
-      if constexpr (QUAD) {
-        const QuadNode *all = static_cast<const QuadNode *>(vertices);
-        const QuadNode *qn[kRowIlp];
-#pragma unroll
-        for (int i = 0; i < kRowIlp; ++i) qn[i] = all + (long long)t[i] * NQ;
-        // The top of every tree is the same for all samples: the wavefront copies the first quads of its TPW trees
-        // into LDS once per step (into the space of the parked results, which nobody reads before this step's walks
-        // are over), where they fit.
-        constexpr bool kTopFits = size_t(TPW) * kTopQuads * sizeof(QuadNode) <= size_t(BT) * LDP * sizeof(Real);
-        if (kTopFits && NQ >= kTopQuads) {
-          QuadNode *stage = reinterpret_cast<QuadNode *>(p_abs);
-          for (int i = lane; i < TPW * kTopQuads; i += kWave) {
-            const int tt = i / kTopQuads, q = i - tt * kTopQuads;
-            stage[i] = all[(long long)min(tb + tt, t_end - 1) * NQ + q];
-          }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          const QuadNode *top[kRowIlp];
-#pragma unroll
-          for (int i = 0; i < kRowIlp; ++i) top[i] = stage + (slot + i * SLOTS) * kTopQuads;
-          walk_quads<kRowIlp, BT, true, RECORD>(d.depth, qn, top, xs_j, r);
-          // every lane has read its quads before any lane overwrites them with results
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-        } else {
-          walk_quads<kRowIlp, BT, false, RECORD>(d.depth, qn, qn, xs_j, r);
-        }
-      } else {
-        const Node<Real> *all = static_cast<const Node<Real> *>(vertices);
-        bool staged = false;
-        if constexpr (FERN) {
-          // A fern's vertex is the same for every sample, so a vector load of it would fetch one address per tree
-          // slot and still cost a full trip through the vector memory pipeline per level. Instead the wavefront
-          // copies the vertices of its TPW ferns into LDS once per step -- into the space of the parked results,
-          // which nobody reads before this step's walks are over -- and the walk reads them as LDS broadcasts.
-          Node<Real> *stage = reinterpret_cast<Node<Real> *>(p_abs);
-          if (size_t(TPW) * d.depth * sizeof(Node<Real>) <= size_t(BT) * LDP * sizeof(Real)) {
-            staged = true;
-            // level major, [level][fern]: the ferns of a lane's kRowIlp walks then lie a compile-time distance apart
-            for (int i = lane; i < TPW * d.depth; i += kWave) {
-              const int lv = i / TPW, tt = i - lv * TPW;
-              stage[i] = all[(long long)min(tb + tt, t_end - 1) * d.V + lv];
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            walk_ferns_staged<Real, kRowIlp, BT, SLOTS, TPW, RECORD>(d.depth, stage + slot, xs_j, r);
-            // every lane has read its vertices before any lane overwrites them with results
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-          }
-        }
-        if (!staged) {
-          const Node<Real> *nd[kRowIlp];
-#pragma unroll
-          for (int i = 0; i < kRowIlp; ++i) nd[i] = all + (long long)t[i] * d.V;
-          walk_many<Real, FERN, kRowIlp>(d.depth, nd, [&](int, int f) { return xs_j[f * BT]; }, r);
-        }
-      }
+      rows_walk_step<Real, FERN, QUAD, BT, RECORD>(d, vertices, NQ, tb, t_end, slot, lane, xs_j, p_abs, r);
 #pragma unroll
       for (int i = 0; i < kRowIlp; ++i) {
         const Real a = ht_abs(r[i].margin);
@@ -765,6 +779,85 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
     __builtin_amdgcn_wave_barrier();
   }
   if (RECORD) bound_publish(margin_bound_value<Real>(margin_bound.bits), rec.bound, (blockIdx.y * gridDim.x + blockIdx.x) % unsigned(kBoundSlots));
+}
+
+// The walk of forward_rows_kernel without its output phase, for the maps: a wavefront parks one or two values per
+// (sample, tree) pair of its step and writes them with its lanes running along the tree axis of [S][T], so that a
+// sample's values of the step's TPW trees leave as one run (the int64 leaf keys of 8 trees are a whole 64-byte sector).
+// MARGIN = false: leaf keys, as int64 [S][T] (leafmap) and / or as 16-bit keys tree major [T][S] (keys16, what the
+// reachability histogram reads; stored by the walking lane itself, whose neighbours hold the neighbouring samples).
+// MARGIN = true: signed margins [S][T] and the selected ordinals as int64 [S][T].
+template <typename Real, bool FERN, bool QUAD, int BT, bool MARGIN>
+__global__ __launch_bounds__(kForestThreads) void maps_rows_kernel(ForestDims d, const Real *__restrict__ x,
+                                                                   const void *__restrict__ vertices, int NQ,
+                                                                   int64_t *__restrict__ leafmap,
+                                                                   uint16_t *__restrict__ keys16,
+                                                                   Real *__restrict__ margins,
+                                                                   int64_t *__restrict__ ordinals,
+                                                                   int trees_per_block) {
+  constexpr int NT = kForestThreads;
+  constexpr int kWaves = NT / kWave;
+  constexpr int SLOTS = kWave / BT;
+  constexpr int TPW = SLOTS * kRowIlp;
+  constexpr int LDP = TPW + 1;
+  extern __shared__ __align__(16) unsigned char smem[];
+  Real *xs = reinterpret_cast<Real *>(smem);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  Real *p_val = xs + size_t(d.F) * BT + size_t(wave) * (BT * LDP);
+  uint16_t *p_u16 = reinterpret_cast<uint16_t *>(xs + size_t(d.F) * BT + size_t(kWaves) * (BT * LDP)) +
+                    size_t(wave) * (BT * LDP);
+  const long long s0 = (long long)blockIdx.x * BT;
+  load_tile<Real, BT, NT>(xs, x, d, s0);
+  __syncthreads();
+  const int j = lane % BT, slot = lane / BT;
+  const long long s = s0 + j;
+  const bool live = s < d.S;
+  const int n_live = int(min<long long>(BT, d.S - s0));
+  const Real *xs_j = xs + j;
+  const int t_begin = blockIdx.y * trees_per_block;
+  const int t_end = min(d.T, t_begin + trees_per_block);
+  for (int tb = t_begin + wave * TPW; tb < t_end; tb += kWaves * TPW) {
+    {
+      WalkResult<Real> r[kRowIlp];
+      rows_walk_step<Real, FERN, QUAD, BT, MARGIN>(d, vertices, NQ, tb, t_end, slot, lane, xs_j, p_val, r);
+#pragma unroll
+      for (int i = 0; i < kRowIlp; ++i) {
+        const int at = j * LDP + slot + i * SLOTS;
+        if (MARGIN) {
+          p_val[at] = r[i].margin;
+          p_u16[at] = uint16_t(r[i].ord);
+        } else {
+          p_u16[at] = uint16_t(r[i].key);
+          const int t = tb + slot + i * SLOTS;
+          if (keys16 && live && t < t_end) keys16[(long long)t * d.S + s] = uint16_t(r[i].key);
+        }
+      }
+    }
+    // the parked values are read by other lanes of this wavefront only
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int nt = min(TPW, t_end - tb);
+    const int total = n_live * nt;
+    const FastDiv by_nt(nt);
+    const long long base = s0 * d.T + tb;
+    if (MARGIN || leafmap) {
+      for (int u = lane; u < total; u += kWave) {
+        const int jj = nt == TPW ? u / TPW : by_nt.div(u);
+        const int tt = u - jj * nt;
+        const long long at = base + (long long)jj * d.T + tt;
+        if (MARGIN) {
+          if (margins) __builtin_nontemporal_store(p_val[jj * LDP + tt], margins + at);
+          if (ordinals) __builtin_nontemporal_store((long long)p_u16[jj * LDP + tt], reinterpret_cast<long long *>(ordinals) + at);
+        } else {
+          __builtin_nontemporal_store((long long)p_u16[jj * LDP + tt], reinterpret_cast<long long *>(leafmap) + at);
+        }
+      }
+    }
+    // the next step's parking writes follow this step's reads in program order
+    __builtin_amdgcn_wave_barrier();
+  }
 }
 
 template <typename Real>
@@ -1084,13 +1177,81 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
               : dispatch_forward<Real, false>(d, x, nodes, w, out, records, stream, img);
 }
 
+// ---- maps on the row kernel's walk ----------------------------------------------------------------------------------
+template <typename Real, bool FERN, bool QUAD, int BT>
+static int launch_maps_rows(const ForestDims &d, const Real *x, const void *vertices, int64_t *leafmap, uint16_t *keys16,
+                            Real *margins, int64_t *ordinals, hipStream_t stream) {
+  constexpr int TPW = kWave / BT * kRowIlp;
+  constexpr int TP = kForestThreads / kWave * TPW;
+  const size_t lds = rows_lds_bytes<Real>(d.F, BT);
+  const long long tiles = (d.S + BT - 1) / BT;
+  int trees_per_block, gy;
+  split_trees(tiles, d.T, TP, &trees_per_block, &gy);
+  if (tiles > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: too many sample tiles for one launch.");
+  const int NQ = int(quads_per_tree(d.depth));
+  if (leafmap || keys16) {
+    auto kernel = maps_rows_kernel<Real, FERN, QUAD, BT, false>;
+    HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
+    hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, vertices, NQ,
+                       leafmap, keys16, (Real *)nullptr, (int64_t *)nullptr, trees_per_block);
+    HT_LAUNCH_CHECK("forest maps (leaf keys)");
+  }
+  if (margins || ordinals) {
+    auto kernel = maps_rows_kernel<Real, FERN, QUAD, BT, true>;
+    HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
+    hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(kForestThreads), lds, stream, d, x, vertices, NQ,
+                       (int64_t *)nullptr, (uint16_t *)nullptr, margins, ordinals, trees_per_block);
+    HT_LAUNCH_CHECK("forest maps (margins)");
+  }
+  return HT_OK;
+}
+
+template <typename Real, bool FERN, bool QUAD>
+static int dispatch_maps_rows(const ForestDims &d, const Real *x, const void *vertices, int64_t *leafmap,
+                              uint16_t *keys16, Real *margins, int64_t *ordinals, hipStream_t stream) {
+  switch (pick_rows_tile<Real>(d.F)) {
+    case 64: return launch_maps_rows<Real, FERN, QUAD, 64>(d, x, vertices, leafmap, keys16, margins, ordinals, stream);
+    case 32: return launch_maps_rows<Real, FERN, QUAD, 32>(d, x, vertices, leafmap, keys16, margins, ordinals, stream);
+    case 16: return launch_maps_rows<Real, FERN, QUAD, 16>(d, x, vertices, leafmap, keys16, margins, ordinals, stream);
+    default: return launch_maps_rows<Real, FERN, QUAD, 8>(d, x, vertices, leafmap, keys16, margins, ordinals, stream);
+  }
+}
+
+template <typename Real>
+size_t forest_maps_rows_workspace(const ForestDims &d) {
+  return rows_ok<Real>(d) ? vertex_bytes<Real>(d) : 0;
+}
+
+template <typename Real>
+int forest_maps_rows(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord,
+                     int64_t *leafmap, uint16_t *keys16, Real *margins, int64_t *ordinals, void *ws,
+                     hipStream_t stream) {
+  if constexpr (std::is_same<Real, float>::value) {
+    if (quads_ok<Real>(d, fern)) {
+      const int NQ = int(quads_per_tree(d.depth));
+      const long long n = (long long)d.T * NQ;
+      hipLaunchKernelGGL(pack_quads_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, thr, ord,
+                         static_cast<QuadNode *>(ws), d.T, d.V, NQ, d.F, (unsigned long long *)nullptr);
+      HT_LAUNCH_CHECK("pack two-level vertices");
+      return dispatch_maps_rows<Real, false, true>(d, x, ws, leafmap, keys16, margins, ordinals, stream);
+    }
+  }
+  int rc = pack_nodes<Real>(d, thr, ord, ws, stream, nullptr);
+  if (rc != HT_OK) return rc;
+  return fern ? dispatch_maps_rows<Real, true, false>(d, x, ws, leafmap, keys16, margins, ordinals, stream)
+              : dispatch_maps_rows<Real, false, false>(d, x, ws, leafmap, keys16, margins, ordinals, stream);
+}
+
 #define HT_INSTANTIATE(Real)                                                                                          \
   template size_t packed_nodes_bytes<Real>(const ForestDims &);                                                       \
   template int pack_nodes<Real>(const ForestDims &, const Real *, const int64_t *, void *, hipStream_t,                \
                                 unsigned long long *);                                                                \
   template size_t forest_forward_workspace<Real>(const ForestDims &);                                                 \
   template int forest_forward<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,            \
-                                    const Real *, Real *, void *, void *, size_t, hipStream_t, const ImageStore *);
+                                    const Real *, Real *, void *, void *, size_t, hipStream_t, const ImageStore *);   \
+  template size_t forest_maps_rows_workspace<Real>(const ForestDims &);                                               \
+  template int forest_maps_rows<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,          \
+                                      int64_t *, uint16_t *, Real *, int64_t *, void *, hipStream_t);
 HT_INSTANTIATE(float)
 HT_INSTANTIATE(double)
 #undef HT_INSTANTIATE

@@ -193,26 +193,18 @@ int ordinal_range(const int64_t *ord, int64_t n, int64_t *minmax, hipStream_t st
   return HT_OK;
 }
 
-// Bytes that let reachability run as a histogram; the call works without them, slower.
+// Workspace: the 16-bit leaf keys that let reachability run as a histogram, then the packed vertices that let every
+// map run on the forward's row kernel walk. The call works without either (or with less), slower.
+static size_t reach_keys_bytes(const ForestDims &d) {
+  return reach_by_histogram(d) ? align_up(size_t(d.S) * d.T * sizeof(uint16_t), 256) : 0;
+}
 template <typename Real>
-size_t forest_maps_workspace(const ForestDims &d) {
-  return reach_by_histogram(d) ? size_t(d.S) * d.T * sizeof(uint16_t) : 0;
+size_t forest_maps_workspace(const ForestDims &d, bool want_reach) {
+  if (d.S == 0 || d.T == 0) return 0;
+  return (want_reach ? reach_keys_bytes(d) : 0) + forest_maps_rows_workspace<Real>(d);
 }
 
-template <typename Real>
-int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap,
-                Real *margins, int64_t *ordinals, int64_t *reach, void *workspace, size_t workspace_bytes,
-                hipStream_t stream) {
-  int rc;
-  if (reach && (rc = zero_fill(reach, size_t(d.T) * d.L * sizeof(int64_t), stream)) != HT_OK) return rc;
-  if (d.S == 0 || d.T == 0) return HT_OK;
-  uint16_t *keys = nullptr;
-  if (reach && workspace && reach_by_histogram(d) && workspace_bytes >= size_t(d.S) * d.T * sizeof(uint16_t) &&
-      (reinterpret_cast<uintptr_t>(workspace) & 15) == 0)
-    keys = static_cast<uint16_t *>(workspace);
-  rc = fern ? dispatch_maps<Real, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream)
-            : dispatch_maps<Real, false>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream);
-  if (rc != HT_OK || !keys) return rc;
+static int launch_reach_histogram(const ForestDims &d, const uint16_t *keys, int64_t *reach, hipStream_t stream) {
   // enough workgroups to fill the part, each with a stretch of keys that is worth its counter flush
   long long parts = (2048 + d.T - 1) / d.T;
   const long long most = (d.S + 4LL * d.L - 1) / (4LL * d.L);
@@ -230,8 +222,35 @@ int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, 
   return HT_OK;
 }
 
-template size_t forest_maps_workspace<float>(const ForestDims &);
-template size_t forest_maps_workspace<double>(const ForestDims &);
+template <typename Real>
+int forest_maps(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, int64_t *leafmap,
+                Real *margins, int64_t *ordinals, int64_t *reach, void *workspace, size_t workspace_bytes,
+                hipStream_t stream) {
+  int rc;
+  if (reach && (rc = zero_fill(reach, size_t(d.T) * d.L * sizeof(int64_t), stream)) != HT_OK) return rc;
+  if (d.S == 0 || d.T == 0) return HT_OK;
+  const bool aligned = workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
+  const size_t key_bytes = reach_keys_bytes(d), row_bytes = forest_maps_rows_workspace<Real>(d);
+  // the row kernel's walk: wherever its packed vertices have room in the workspace -- and, for reachability, the keys
+  // of the histogram as well (its other form, one global atomic per pair, stays with the plain kernel below)
+  const bool keys_fit = key_bytes != 0 && aligned && workspace_bytes >= key_bytes;
+  const size_t rows_at = reach ? key_bytes : 0;
+  if (row_bytes != 0 && aligned && workspace_bytes >= rows_at + row_bytes && (!reach || keys_fit)) {
+    uint16_t *keys = reach ? static_cast<uint16_t *>(workspace) : nullptr;
+    void *vertices = static_cast<unsigned char *>(workspace) + rows_at;
+    if ((rc = forest_maps_rows<Real>(d, fern, x, thr, ord, leafmap, keys, margins, ordinals, vertices, stream)) != HT_OK)
+      return rc;
+    return reach ? launch_reach_histogram(d, keys, reach, stream) : HT_OK;
+  }
+  uint16_t *keys = (reach && keys_fit) ? static_cast<uint16_t *>(workspace) : nullptr;
+  rc = fern ? dispatch_maps<Real, true>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream)
+            : dispatch_maps<Real, false>(d, x, thr, ord, leafmap, margins, ordinals, reach, keys, stream);
+  if (rc != HT_OK || !keys) return rc;
+  return launch_reach_histogram(d, keys, reach, stream);
+}
+
+template size_t forest_maps_workspace<float>(const ForestDims &, bool);
+template size_t forest_maps_workspace<double>(const ForestDims &, bool);
 template int forest_maps<float>(const ForestDims &, bool, const float *, const float *, const int64_t *, int64_t *,
                                 float *, int64_t *, int64_t *, void *, size_t, hipStream_t);
 template int forest_maps<double>(const ForestDims &, bool, const double *, const double *, const int64_t *, int64_t *,

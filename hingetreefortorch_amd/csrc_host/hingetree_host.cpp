@@ -314,8 +314,8 @@ py::object forest_maps(int kind, const torch::Tensor &inData, const torch::Tenso
     ordinals = torch::empty(map_sizes, longs);
   }
   if (want == kReach) reach = torch::empty({inWeights.size(0), inWeights.size(1)}, longs);
-  // only reachability has a use for the workspace (leaf keys for its histogram)
-  const size_t bytes = want == kReach ? ht_forest_maps_workspace(&s) : 0;
+  // packed vertices for the walk and, for reachability, the leaf keys of its histogram
+  const size_t bytes = ht_forest_maps_workspace(&s, want == kReach);
   const torch::Tensor ws = workspace(bytes, inData);
   check(ht_forest_maps(&s, ptr(inData), ptr(inThresholds), static_cast<const int64_t *>(ptr(inOrdinals)),
                        static_cast<int64_t *>(ptr(leaf)), ptr(margins), static_cast<int64_t *>(ptr(ordinals)),

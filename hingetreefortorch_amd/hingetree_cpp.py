@@ -622,8 +622,8 @@ def _maps(kind, inData, inThresholds, inOrdinals, inWeights, want):
         ordinals = torch.empty(map_sizes, dtype=torch.int64, device=dev) if want == "margin" else None
         reach = torch.empty(list(inWeights.shape[:2]), dtype=torch.int64, device=dev) if want == "reach" else None
         lib = L.load()
-        # only reachability has a use for the workspace (leaf keys for its histogram)
-        nbytes = lib.ht_forest_maps_workspace(ctypes.byref(shape)) if want == "reach" else 0
+        # packed vertices for the walk and, for reachability, the leaf keys of its histogram
+        nbytes = lib.ht_forest_maps_workspace(ctypes.byref(shape), int(want == "reach"))
         ws = _workspace(nbytes, dev)
         L.check(lib.ht_forest_maps(ctypes.byref(shape), _ptr(inData), _ptr(inThresholds), _ptr(inOrdinals), _ptr(leaf),
                                    _ptr(margins), _ptr(ordinals), _ptr(reach), _ptr(ws), nbytes, _stream(dev)))

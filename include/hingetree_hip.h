@@ -147,9 +147,11 @@ int ht_forest_backward_records(const ht_forest_shape *s, const void *w, const vo
 
 /* Per-(b,t,k) leaf key / signed margin + selected ordinal / per-(t,leaf) visit counts; any output may be NULL.
  * Replaces hingetree_gpu_leafmap, _marginmap, _reachability (hingetree.cpp:54-60; hingetree_gpu.cu:732-933), which
- * return the leaf map and the counts as int64 on the GPU. The workspace serves `reach` alone (16-bit leaf keys for a
- * histogram per tree); without it the counts come from one global atomic per pair, several times slower. */
-size_t ht_forest_maps_workspace(const ht_forest_shape *s);
+ * return the leaf map and the counts as int64 on the GPU. The workspace (its size depends on whether `reach` will be
+ * asked for) holds the packed vertices that let the maps run on the forward pass's walk and, for `reach`, 16-bit leaf
+ * keys for a histogram per tree; the call works without it or with less -- maps several times slower, counts from one
+ * global atomic per pair. */
+size_t ht_forest_maps_workspace(const ht_forest_shape *s, int32_t want_reach);
 int ht_forest_maps(const ht_forest_shape *s, const void *x, const void *thr, const int64_t *ord, int64_t *leafmap,
                    void *margins, int64_t *ordinals, int64_t *reach, void *workspace, size_t workspace_bytes,
                    void *stream);
