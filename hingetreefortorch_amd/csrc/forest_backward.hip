@@ -400,7 +400,11 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
                                                               Records<Real, COMPACT> rec, Real *dw,
                                                               unsigned long long *dw_fixed, const DetHeader *hdr,
                                                               int TB, long long part_size, bool need_c,
-                                                              bool dw_atomic, int P, int num_groups, int slices) {
+                                                              bool dw_atomic, int P, int num_groups, int slices,
+                                                              int m0, int Mw) {
+  // [m0, m0 + Mw): the window of a leaf row's elements this launch serves. A row wider than the 64 lanes x 16 bytes a
+  // wavefront can give one pair is worked off in several launches, each with accumulators for its window only; c,
+  // a sum over the whole row, is then built up launch by launch.
   constexpr int VE = 16 / sizeof(Real);  // elements per 16-byte chunk
   typedef typename std::conditional<FIXED, unsigned long long, double>::type Acc;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -428,7 +432,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
   const int t0 = group * TB;
   const int nt = min(TB, d.T - t0);
   const long long LM = (long long)d.L * d.M;
-  const long long acc_cells = (long long)nt * leaves * d.M;  // (nt == 1 whenever slices > 1)
+  const long long acc_cells = (long long)nt * leaves * Mw;  // (nt == 1 whenever slices > 1)
   if (dw) {
     for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads) acc[i] = Acc(0);
     __syncthreads();
@@ -454,18 +458,18 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
   // the 16-byte chunk that starts at its first element (shifted back where it would pass the end of the row): lanes
   // with overlapping chunks hit the same line, which costs nothing extra.
   const int grp = lane / P, li = lane & (P - 1);
-  const int own_begin = li * d.M / P, own_end = (li + 1) * d.M / P;
-  const int e0 = d.M >= VE ? min(own_begin, d.M - VE) : 0;  // first element of this lane's chunk
-  const int own = own_begin - e0;                            // chunk elements [own, own + cnt) belong to this lane
+  const int own_begin = li * Mw / P, own_end = (li + 1) * Mw / P;  // inside the window
+  const int e0 = Mw >= VE ? min(own_begin, Mw - VE) : 0;  // first element of this lane's chunk
+  const int own = own_begin - e0;                          // chunk elements [own, own + cnt) belong to this lane
   const int cnt = own_end - own_begin;
-  const int rounds = (d.M + P - 1) / P;                      // wave uniform: max cnt over the lanes
+  const int rounds = (Mw + P - 1) / P;                     // wave uniform: max cnt over the lanes
 
   auto load_chunk = [&](const Real *p, Real (&v)[VE]) {
-    if (d.M >= VE) {
+    if (Mw >= VE) {
       __builtin_memcpy(v, p, sizeof(Real) * VE);  // 16 bytes, element aligned
     } else {
 #pragma unroll
-      for (int k = 0; k < VE; ++k) v[k] = k < d.M ? p[k] : Real(0);
+      for (int k = 0; k < VE; ++k) v[k] = k < Mw ? p[k] : Real(0);
     }
   };
 
@@ -511,9 +515,9 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
       q.src[u] = tq * SPT + j;
       q.tq_of[u] = tq;
       if (d.K == 1)
-        load_chunk(gbase + (uint32_t(j) * d.T + tq) * d.M + e0, q.gv[u]);
+        load_chunk(gbase + (uint32_t(j) * d.T + tq) * d.M + m0 + e0, q.gv[u]);
       else
-        load_chunk(gout + out_offset(d, sblk + j, t0 + tq, e0), q.gv[u]);
+        load_chunk(gout + out_offset(d, sblk + j, t0 + tq, m0 + e0), q.gv[u]);
     }
   };
 
@@ -530,11 +534,12 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
     for (int u = 0; u < U; ++u) {
       const uint32_t key = __shfl(cur.key_r, cur.src[u], kWave);
       mg[u] = __shfl(cur.mg_r, cur.src[u], kWave);
-      rel[u] = (uint32_t(cur.tq_of[u]) * d.L + key) * d.M + e0;
-      if (need_c) load_chunk(wbase + rel[u], wv[u]);
-      // the pair's accumulator row: this slice's leaves only, counted from the slice's first leaf
+      const uint32_t row = uint32_t(cur.tq_of[u]) * d.L + key;
+      if (need_c) load_chunk(wbase + (row * uint32_t(d.M) + uint32_t(m0) + e0), wv[u]);
+      // the pair's accumulator row: this slice's leaves only, counted from the slice's first leaf; the window's
+      // elements only
       in_slice[u] = cur.on[u] && key - leaf_begin < uint32_t(leaves);
-      rel[u] -= leaf_begin * uint32_t(d.M);
+      rel[u] = (row - leaf_begin) * uint32_t(Mw) + e0;
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -567,6 +572,7 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
       }
     }
     if (need_c && sub0 + U == P && cur.have) {
+      if (m0 != 0) c_mine += rec.c[cur.at];  // the earlier windows' share (the launches follow each other)
       rec.c[cur.at] = c_mine;
       if (FIXED) bound_take(c_bound, c_mine);
     }
@@ -574,23 +580,30 @@ __global__ __launch_bounds__(kForestThreads) void tree_kernel(ForestDims d, cons
   if (FIXED && need_c) publish_c_bound(c_bound, hdr);
   if (dw) {
     __syncthreads();
-    const long long first = (long long)t0 * LM + (long long)leaf_begin * d.M;
+    const long long first = (long long)t0 * LM + (long long)leaf_begin * d.M + m0;
     Real *dst = dw + first;
+    // cell i of the table is element i % Mw of accumulator row i / Mw: where it lies in a row of d.M elements
+    const FastDiv by_mw(Mw);
+    auto at = [&](long long i) -> long long {
+      if (Mw == d.M) return i;
+      const long long row = acc_cells < (1ll << 31) ? (long long)by_mw.div(int(i)) : i / Mw;
+      return row * d.M + (i - row * Mw);
+    };
     if (FIXED) {
       const unsigned long long *q = reinterpret_cast<const unsigned long long *>(acc);
       if (dw_atomic) {
         for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads)
-          if (q[i] != 0ull) atomicAdd(dw_fixed + first + i, q[i]);
+          if (q[i] != 0ull) atomicAdd(dw_fixed + first + at(i), q[i]);
       } else {
-        for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads) dst[i] = from_fixed<Real>(q[i], inv_scale);
+        for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads) dst[at(i)] = from_fixed<Real>(q[i], inv_scale);
       }
     } else {
       const double *q = reinterpret_cast<const double *>(acc);
       if (dw_atomic) {
         for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads)
-          if (q[i] != 0.0) atomicAdd(dst + i, Real(q[i]));
+          if (q[i] != 0.0) atomicAdd(dst + at(i), Real(q[i]));
       } else {
-        for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads) dst[i] = Real(q[i]);
+        for (long long i = threadIdx.x; i < acc_cells; i += kForestThreads) dst[at(i)] = Real(q[i]);
       }
     }
   }
@@ -1709,6 +1722,13 @@ __global__ __launch_bounds__(kWave) void det_tree_kernel(ForestDims d, const Rea
 // host side
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int kLeanMaxOutputs = 16;  // tree_lean_kernel: at most four lanes of four values per pair
+// Elements of a leaf row that a wavefront's 64 lanes cover with one 16-byte chunk each: wider rows take the tree kernel
+// several launches, one per window of this many elements (at most kMaxRowWindows of them).
+template <typename Real>
+constexpr int row_window() {
+  return kWave * (16 / int(sizeof(Real)));
+}
+constexpr int kMaxRowWindows = 4;
 struct TreePlan {
   int TB;               // trees per workgroup
   int groups, parts;    // grid (groups counts tree groups x leaf slices)
@@ -1724,8 +1744,9 @@ static inline size_t staged_weights_per_tree(const ForestDims &d, bool lean) {
   return lean && d.M == 1 ? size_t(d.L) * sizeof(float) : 0;
 }
 
-static bool plan_trees(const ForestDims &d, bool need_dw, bool lean, TreePlan *p) {
-  const size_t per_tree = size_t(d.L) * d.M * sizeof(double);
+// row_limit: the elements of a leaf row that one launch of the tree kernel accumulates (row_window below).
+static bool plan_trees(const ForestDims &d, bool need_dw, bool lean, TreePlan *p, int row_limit) {
+  const size_t per_tree = size_t(d.L) * (d.M < row_limit ? d.M : row_limit) * sizeof(double);
   const size_t w_tree = staged_weights_per_tree(d, lean);
   int tb = 4;
   p->slices = 1;
@@ -1814,13 +1835,13 @@ static void plan_dthr(const ForestDims &d, long long *part_size, int *gy) {
 template <typename Real, bool COMPACT, bool FIXED, int U>
 int launch_tree_kernel_u(const ForestDims &d, const TreePlan &p, int P, const Real *w, const Real *gout,
                          Records<Real, COMPACT> rec, Real *dw, unsigned long long *dw_fixed, const DetHeader *hdr,
-                         bool need_c, hipStream_t stream) {
+                         bool need_c, hipStream_t stream, int m0, int Mw) {
   auto kernel = tree_kernel<Real, COMPACT, FIXED, U>;
   HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   const int per_xcd = (p.groups + kNumXCDs - 1) / kNumXCDs;
   hipLaunchKernelGGL(kernel, dim3((unsigned)(per_xcd * kNumXCDs), (unsigned)p.parts), dim3(kForestThreads), p.lds,
                      stream, d, w, gout, rec, dw, dw_fixed, hdr, p.TB, p.part_size, need_c, p.parts > 1, P, p.groups,
-                     p.slices);
+                     p.slices, m0, Mw);
   HT_LAUNCH_CHECK("forest backward (trees)");
   return HT_OK;
 }
@@ -1930,12 +1951,22 @@ int launch_tree_kernel(const ForestDims &d, const TreePlan &p, const Real *w, co
     }
   }
   constexpr int VE = 16 / sizeof(Real);
-  const int Q = d.M >= VE ? (d.M + VE - 1) / VE : 1;  // 16-byte chunks in one pair's values
-  int P = 1;                                          // lanes per pair
-  while (P < Q) P <<= 1;
-  if (P >= 4) return launch_tree_kernel_u<Real, COMPACT, FIXED, 4>(d, p, P, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
-  if (P == 2) return launch_tree_kernel_u<Real, COMPACT, FIXED, 2>(d, p, P, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
-  return launch_tree_kernel_u<Real, COMPACT, FIXED, 1>(d, p, P, w, gout, rec, dw, dw_fixed, hdr, need_c, stream);
+  // one launch per window of the leaf rows (a single one unless a row is wider than a wavefront's 64 chunks)
+  for (int m0 = 0; m0 < d.M; m0 += row_window<Real>()) {
+    const int Mw = d.M - m0 < row_window<Real>() ? d.M - m0 : row_window<Real>();
+    const int Q = Mw >= VE ? (Mw + VE - 1) / VE : 1;  // 16-byte chunks in one pair's values
+    int P = 1;                                        // lanes per pair
+    while (P < Q) P <<= 1;
+    int rc;
+    if (P >= 4)
+      rc = launch_tree_kernel_u<Real, COMPACT, FIXED, 4>(d, p, P, w, gout, rec, dw, dw_fixed, hdr, need_c, stream, m0, Mw);
+    else if (P == 2)
+      rc = launch_tree_kernel_u<Real, COMPACT, FIXED, 2>(d, p, P, w, gout, rec, dw, dw_fixed, hdr, need_c, stream, m0, Mw);
+    else
+      rc = launch_tree_kernel_u<Real, COMPACT, FIXED, 1>(d, p, P, w, gout, rec, dw, dw_fixed, hdr, need_c, stream, m0, Mw);
+    if (rc != HT_OK) return rc;
+  }
+  return HT_OK;
 }
 
 template <typename Real, int BT, bool COMPACT, bool FIXED>
@@ -1970,9 +2001,9 @@ static int pick_dx_tile(int F, size_t cell) {
 template <typename Real>
 bool staged_ok(const ForestDims &d, bool need_dx, bool need_dw, bool fixed) {
   if (d.M < 1) return false;
-  // the lanes serving one (sample, tree) pair (16 bytes each) must fit a wavefront, and the tree kernel addresses
-  // the gradient rows of one 64-sample step with 32-bit offsets
-  if ((d.M + 16 / int(sizeof(Real)) - 1) / (16 / int(sizeof(Real))) > kWave) return false;
+  // a leaf row is served in at most kMaxRowWindows windows of a wavefront's 64 chunks of 16 bytes, and the tree kernel
+  // addresses the gradient rows of one 64-sample step with 32-bit offsets
+  if (d.M > kMaxRowWindows * row_window<Real>()) return false;
   if ((long long)d.T * d.M * kWave >= (1ll << 31)) return false;
   // (a leaf table beyond LDS is accumulated in slices of its leaves, each at least one leaf row)
   if (need_dw && size_t(d.L) * d.M * sizeof(double) > size_t(kLdsBytes) * kMaxLeafSlices) return false;
@@ -1993,13 +2024,13 @@ static bool prefer_fused(const ForestDims &d) { return double(d.S) * double(d.T)
 struct FixedLayout {
   size_t header, dw, dthr, total;
 };
-static FixedLayout fixed_layout(const ForestDims &d, bool need_dthr, bool need_dw, bool lean) {
+static FixedLayout fixed_layout(const ForestDims &d, bool need_dthr, bool need_dw, bool lean, int row_limit) {
   FixedLayout l{};
   TreePlan plan;
   l.header = 0;
   size_t at = kDetHeaderBytes;
   l.dw = at;
-  if (need_dw && plan_trees(d, true, lean, &plan) && plan.parts > 1) at += align_up(size_t(d.T) * d.L * d.M * 8, 256);
+  if (need_dw && plan_trees(d, true, lean, &plan, row_limit) && plan.parts > 1) at += align_up(size_t(d.T) * d.L * d.M * 8, 256);
   l.dthr = at;
   long long part_size;
   int gy;
@@ -2034,7 +2065,8 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
   const long long pairs = (long long)d.T * d.S;
   TreePlan plan;
   constexpr bool kLean = std::is_same<Real, float>::value && COMPACT;
-  if (!plan_trees(d, dw != nullptr, kLean && d.K == 1, &plan)) return fail(HT_ERR_RUNTIME, "Error: leaf table too large.");
+  if (!plan_trees(d, dw != nullptr, kLean && d.K == 1, &plan, row_window<Real>()))
+    return fail(HT_ERR_RUNTIME, "Error: leaf table too large.");
   long long dthr_part;
   int dthr_gy;
   plan_dthr(d, &dthr_part, &dthr_gy);
@@ -2043,7 +2075,7 @@ int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes,
   unsigned long long *dw_fixed = nullptr, *dthr_fixed = nullptr;
   bool sampled = false;  // the scale of dW rests on a sample of the upstream gradient (see DetHeader)
   if (FIXED) {
-    const FixedLayout lay = fixed_layout(d, dthr != nullptr, dw != nullptr, kLean && d.K == 1);
+    const FixedLayout lay = fixed_layout(d, dthr != nullptr, dw != nullptr, kLean && d.K == 1, row_window<Real>());
     unsigned char *base = static_cast<unsigned char *>(fixed_ws);
     hdr = reinterpret_cast<DetHeader *>(base + lay.header);
     dw_fixed = reinterpret_cast<unsigned long long *>(base + lay.dw);
@@ -2217,7 +2249,8 @@ size_t route_bytes(const ForestDims &d, Route r, bool need_dthr, bool need_dw, b
   if (r == Route::kFused) return 0;
   size_t bytes = (have_records ? 0 : records_saved_bytes<Real>(d)) + records_scratch_bytes<Real>(d);
   if (r == Route::kFixed)
-    bytes += fixed_layout(d, need_dthr, need_dw, std::is_same<Real, float>::value && compact_ok(d) && d.K == 1).total;
+    bytes += fixed_layout(d, need_dthr, need_dw, std::is_same<Real, float>::value && compact_ok(d) && d.K == 1,
+                          row_window<Real>()).total;
   return bytes;
 }
 
@@ -2270,7 +2303,8 @@ int clear_gradients(const ForestDims &d, Route route, Real *dx, Real *dthr, Real
     long long dthr_part;
     int dthr_gy;
     plan_dthr(d, &dthr_part, &dthr_gy);
-    if (plan_trees(d, dw != nullptr, std::is_same<Real, float>::value && compact_ok(d) && d.K == 1, &plan) &&
+    if (plan_trees(d, dw != nullptr, std::is_same<Real, float>::value && compact_ok(d) && d.K == 1, &plan,
+                   row_window<Real>()) &&
         plan.parts == 1) {
       clear_dw = false;
       clear_dthr = dthr_gy > 1;
@@ -2300,7 +2334,7 @@ bool forest_backward_image_ok(const ForestDims &d, int mode, bool need_dx, bool 
   if (mode != HT_BACKWARD_ATOMIC || !compact_ok(d)) return false;
   if (pick_route<Real>(d, mode, need_dx, need_dw, false) != Route::kStaged) return false;
   TreePlan plan;
-  if (!plan_trees(d, need_dw, false, &plan) || !wide_rows_ok(d, plan)) return false;
+  if (!plan_trees(d, need_dw, false, &plan, row_window<Real>()) || !wide_rows_ok(d, plan)) return false;
   return img.win[2] % 4 == 0 && img.pad[2] % 4 == 0 && img.size[2] % 4 == 0 && img.plane % 4 == 0;
 }
 
