@@ -284,16 +284,35 @@ __device__ __forceinline__ long long region_cell(const ConvTile &g, const ConvPo
   return ((long long)gz * g.H + gy) * g.W + gx;
 }
 
+// Magnitude bits of a float (its bit pattern without the sign orders like |v|, every NaN above infinity); 0 for doubles,
+// whose callers do not use the bound.
+__device__ __forceinline__ uint32_t magnitude_bits(float v) { return __float_as_uint(v) & 0x7fffffffu; }
+__device__ __forceinline__ uint32_t magnitude_bits(double) { return 0u; }
+
+// Largest value over the wavefront, to every lane (row operations of the vector ALU, then across the rows).
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0xB1, 0xF, 0xF, true)));   // quad_perm [1,0,3,2]
+  v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x4E, 0xF, 0xF, true)));   // quad_perm [2,3,0,1]
+  v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x141, 0xF, 0xF, true)));  // row_half_mirror
+  v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x140, 0xF, 0xF, true)));  // row_mirror
+  // every lane of a row of 16 now holds its row's maximum: the four rows meet in scalar registers
+  const uint32_t r0 = uint32_t(__builtin_amdgcn_readlane(int(v), 0)), r1 = uint32_t(__builtin_amdgcn_readlane(int(v), 16));
+  const uint32_t r2 = uint32_t(__builtin_amdgcn_readlane(int(v), 32)), r3 = uint32_t(__builtin_amdgcn_readlane(int(v), 48));
+  return max(max(r0, r1), max(r2, r3));
+}
+
 // Cooperative load of the input region of tile `at` of image b, all channels: a thread owns one or two cells of
 // the region and copies them channel by channel (the coordinate arithmetic is done once per cell, not per element).
 // c0 / count: the window of channels to load (all of them by default); plane c0 + k goes to tile plane k.
+// bound (optional): an LDS word that receives the largest magnitude_bits of the tile's values.
 template <typename Real, bool CHECK = false>
 __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restrict__ x, const ConvTile &g, int C,
                                                long long b, const ConvPos &at, int *special, int c0 = 0,
-                                               int count = -1) {
+                                               int count = -1, uint32_t *bound = nullptr) {
   const long long chan = (long long)g.D * g.H * g.W;
   const Real *img = x + (b * C + c0) * chan;
   if (count >= 0) C = count;
+  uint32_t big = 0u;
   for (int e = threadIdx.x; e < g.TSZ; e += int(blockDim.x)) {
     const long long cell = region_cell(g, at, e);
     Real *q = tile + e;
@@ -304,6 +323,7 @@ __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restric
       for (int c = 0; c < C; ++c) {
         const Real v = p[c * chan];
         if (CHECK) plain = plain && plain_feature(v);
+        big = max(big, magnitude_bits(v));
         q[c * g.TSZ] = v;
       }
       if (CHECK && !plain) *special = 1;  // see walk_paths_plain; never reset, every writer stores the same value
@@ -311,16 +331,22 @@ __device__ __forceinline__ void load_conv_tile(Real *tile, const Real *__restric
       for (int c = 0; c < C; ++c) q[c * g.TSZ] = Real(0);
     }
   }
+  if (bound) {  // (one atomic per wavefront: same-address atomics are served one lane at a time)
+    big = wave_max_u32(big);
+    if ((threadIdx.x & 63) == 0 && big) atomicMax(bound, big);
+  }
 }
 
 // The dX image of a tile's input region (fp64, C planes of TSZ cells) added to dx; cells outside the image are dropped
 // like the reference drops padded taps. Regions of neighbouring tiles overlap, hence atomics.
+// fixed: the cells are 64-bit integers, multiples of `unit` (see conv_tiled_backward_kernel).
 template <typename Real>
 __device__ __forceinline__ void flush_dx_image(const double *acc, const ConvTile &g, const ConvPos &at, int C,
-                                               Real *dx_first /* image b, first channel of the window */) {
+                                               Real *dx_first /* image b, first channel of the window */,
+                                               bool fixed = false, double unit = 1.0) {
   const long long chan = (long long)g.D * g.H * g.W;
   for (int i = threadIdx.x; i < C * g.TSZ; i += int(blockDim.x)) {
-    const double v = acc[i];
+    const double v = fixed ? double(reinterpret_cast<const long long *>(acc)[i]) * unit : acc[i];
     if (v == 0.0) continue;
     const int c = i / g.TSZ, r = i - c * g.TSZ;
     const long long cell = region_cell(g, at, r);
@@ -340,24 +366,41 @@ __device__ __forceinline__ void fill_tap_offsets(int *tapoff, const ConvTile &g)
 
 // Trees (and optionally leaf weights) of out channel j into LDS.
 // c0 / count: the window of channels whose trees are staged (all of them by default).
+// thr_bound / w_bound (optional): LDS words that receive the largest magnitude_bits of the staged thresholds / weights.
 template <typename Real, bool CHECK = false>
 __device__ __forceinline__ void stage_conv_trees(Node<Real> *nodes, Real *wl, const ConvTile &g, const int *tapoff,
                                                  int C, int V, int LM, int j, const Real *__restrict__ thr,
                                                  const int64_t *__restrict__ ord, const Real *__restrict__ w,
-                                                 int *special, int c0 = 0, int count = -1) {
+                                                 int *special, int c0 = 0, int count = -1,
+                                                 uint32_t *thr_bound = nullptr, uint32_t *w_bound = nullptr) {
   const long long tree0 = (long long)j * C + c0;
   if (count >= 0) C = count;
   const long long first = tree0 * V;
+  uint32_t big = 0u;
   for (int i = threadIdx.x; i < C * V; i += int(blockDim.x)) {
     Node<Real> n;
     n.thr = thr[first + i];
     n.ord = tapoff[clamp_ordinal(ord[first + i], g.taps)];
     nodes[i] = n;
+    big = max(big, magnitude_bits(n.thr));
     if (CHECK && !plain_threshold(n.thr)) *special = 1;
+  }
+  if (thr_bound) {  // (one atomic per wavefront: same-address atomics are served one lane at a time)
+    big = wave_max_u32(big);
+    if ((threadIdx.x & 63) == 0 && big) atomicMax(thr_bound, big);
   }
   if (wl) {
     const long long wfirst = tree0 * LM;
-    for (int i = threadIdx.x; i < C * LM; i += int(blockDim.x)) wl[i] = w[wfirst + i];
+    big = 0u;
+    for (int i = threadIdx.x; i < C * LM; i += int(blockDim.x)) {
+      const Real v = w[wfirst + i];
+      big = max(big, magnitude_bits(v));
+      wl[i] = v;
+    }
+    if (w_bound) {
+      big = wave_max_u32(big);
+      if ((threadIdx.x & 63) == 0 && big) atomicMax(w_bound, big);
+    }
   }
 }
 
@@ -383,8 +426,10 @@ static ConvLds conv_lds_layout(const ConvTile &t, int C, int V, int LM, bool dx_
   if (tree_acc) at += align_up(size_t(C) * V * sizeof(double), 16);
   l.taps = at;  // tap -> offset in the tile's input region
   at += align_up(size_t(t.taps) * sizeof(int), 16);
-  l.flag = at;  // one word: set once the tile or the staged trees hold a value that rules out walk_paths_plain
-  at += 16;
+  // word 0: set once the tile or the staged trees hold a value that rules out walk_paths_plain; words 1 .. 7: the
+  // magnitude bounds behind the fixed-point cells of conv_tiled_backward_kernel
+  l.flag = at;
+  at += 64;
   l.total = at;
   return l;
 }
@@ -678,11 +723,25 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
   const int LM = L * M;
   // single-output float trees walk by the sign bit where the data allow it (walk_paths_plain_tracked)
   constexpr bool kLeanWalk = M1 && std::is_same<Real, float>::value;
-  if (kLeanWalk) {
+  // Float data: the LDS cells are 64-bit integers. ds_add_u64 costs 13 cycles per wave instruction where ds_add_f64
+  // costs 23, and the three atomics of a walk are most of what this kernel does with its LDS (backward of 32 images
+  // [16,128,128] -> 64 channels, depth 6: 2.47 -> 2.0 ms). A term is scaled by a power of two that puts the largest
+  // possible one just below 2^29, rounded to an integer once, and added; the workgroup finds the bounds behind the
+  // scales in the data it stages anyway: max|x| of its tile, and per out channel max|g| of its positions, max|thr| and
+  // max|w| of the staged trees (magnitude bits into LDS words 1 .. 7 of the flag area). dW terms are |thr - x| * g,
+  // dThr and dX terms sign * sum_m w * g. The per-out-channel tables are flushed per out channel with that channel's
+  // unit; the dX image lives through all of them, so it is shifted right when a later out channel needs a coarser
+  // unit. A bound that is not finite (or scales beyond float's exponent range) puts the out channel -- for the dX image:
+  // the rest of the workgroup's life -- on fp64 cells instead. Sums of at most a few thousand terms below 2^29 are
+  // far from the ends of 64 bits.
+  constexpr bool kFix = std::is_same<Real, float>::value;
+  uint32_t *bnd = reinterpret_cast<uint32_t *>(smem + lay.flag);  // [1] tile; [2..4], [5..7]: g, thr, w of out channel parity 0, 1
+  if (kLeanWalk || kFix) {
     if (threadIdx.x == 0) *special = 0;
+    if (threadIdx.x >= 1 && threadIdx.x < 8) bnd[threadIdx.x] = 0u;
     __syncthreads();
   }
-  load_conv_tile<Real, kLeanWalk>(tile, x, g, C_all, b, at, special, c0, C);
+  load_conv_tile<Real, kLeanWalk>(tile, x, g, C_all, b, at, special, c0, C, kFix ? bnd + 1 : nullptr);
   for (int i = threadIdx.x; i < C * g.TSZ; i += NT) acc[i] = 0.0;
   for (int i = threadIdx.x; i < C * LM; i += NT) acc_w[i] = 0.0;
   for (int i = threadIdx.x; i < C * V; i += NT) acc_t[i] = 0.0;
@@ -695,15 +754,43 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
   const int skew = ((lane & 31) + (lane >> 5) * (C >> 1)) % C;
   const int j_begin = j_block * j_per, j_count = min(Cout, j_begin + j_per) - j_begin;
   const int rot = int((blockIdx.x * 7u + blockIdx.z * 13u) % unsigned(j_count));
-  for (int jj = 0; jj < j_count; ++jj) {
+  // Fixed-point state (all of it wave uniform: every thread derives it from the same LDS words).
+  // tab_fixed / unit_w / unit_c: cells and units of the tables of the out channel in hand; img_*: of the dX image.
+  bool tab_fixed = false, img_fixed = kFix;
+  int img_exp = -100000;  // exponent of the dX image's bound so far: its unit is 2^(img_exp - 29)
+  float scale_w = 1.f, scale_t = 1.f, scale_x = 1.f;
+  double unit_w = 1.0, unit_t = 1.0;
+  // a term into a cell that holds either a double or, times `scale`, a 64-bit integer
+  auto add = [&](double *cell, Real v, bool fixed, float scale) {
+    if constexpr (kFix) {
+      if (fixed) {
+        atomicAdd(reinterpret_cast<unsigned long long *>(cell), (unsigned long long)(long long)__float2int_rn(v * scale));
+        return;
+      }
+    }
+    atomicAdd(cell, double(v));
+  };
+  // 2^e as a float, e inside the range of normal floats
+  auto pow2f = [](int e) -> float { return __uint_as_float(uint32_t(e + 127) << 23); };
+  auto g_of = [&](int jj) -> const Real * {
     const int j = j_begin + (jj + rot >= j_count ? jj + rot - j_count : jj + rot);
+    return gout + ((b * Cout + j) * g.positions() + (live ? at.pos : 0)) * M;
+  };
+  auto j_of = [&](int jj) { return j_begin + (jj + rot >= j_count ? jj + rot - j_count : jj + rot); };
+  // (single output) a position's gradient for the next out channel is requested while the current one is walked: its
+  // bound is wanted before the barrier, where a fresh load's latency would be on every workgroup's critical path
+  Real g_ahead = (M1 && live) ? *g_of(0) : Real(0);
+  for (int jj = 0; jj < j_count; ++jj) {
+    const int j = j_of(jj);
+    uint32_t *now = bnd + 2 + 3 * (jj & 1), *next = bnd + 2 + 3 * ((jj & 1) ^ 1);
     __syncthreads();  // the tile and the zeroed tables are complete / the previous out channel's walks are done
+    if (kFix && threadIdx.x < 3) next[threadIdx.x] = 0u;  // (read last before the barrier above)
     if (jj > 0) {
       // flush the previous out channel's tables (its trees are still known by index only: jp)
-      const int jp = j_begin + (jj - 1 + rot >= j_count ? jj - 1 + rot - j_count : jj - 1 + rot);
+      const int jp = j_of(jj - 1);
       if (dw)
         for (int i = threadIdx.x; i < C * LM; i += NT) {
-          const double v = acc_w[i];
+          const double v = tab_fixed ? double(reinterpret_cast<long long *>(acc_w)[i]) * unit_w : acc_w[i];
           if (v != 0.0) {
             atomicAdd(dw + ((long long)jp * C_all + c0) * LM + i, Real(v));
             acc_w[i] = 0.0;
@@ -711,20 +798,79 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
         }
       if (dthr)
         for (int i = threadIdx.x; i < C * V; i += NT) {
-          const double v = acc_t[i];
+          const double v = tab_fixed ? double(reinterpret_cast<long long *>(acc_t)[i]) * unit_t : acc_t[i];
           if (v != 0.0) {
             atomicAdd(dthr + ((long long)jp * C_all + c0) * V + i, Real(v));
             acc_t[i] = 0.0;
           }
         }
     }
-    stage_conv_trees<Real, kLeanWalk>(nodes, wl, g, tapoff, C_all, V, LM, j, thr, ord, w, special, c0, C);
+    stage_conv_trees<Real, kLeanWalk>(nodes, wl, g, tapoff, C_all, V, LM, j, thr, ord, w, special, c0, C,
+                                      kFix ? now + 1 : nullptr, kFix ? now + 2 : nullptr);
+    const Real *gp = gout + ((b * Cout + j) * g.positions() + (live ? at.pos : 0)) * M;
+    const Real g_one = M1 ? g_ahead : Real(0);
+    if constexpr (kFix) {
+      // this position's largest |g|, over the wavefront, into the out channel's word
+      uint32_t gb = 0u;
+      if (live) {
+        if (M1) {
+          gb = magnitude_bits(g_one);
+        } else {
+          for (int m = 0; m < M; ++m) gb = max(gb, magnitude_bits(gp[m]));
+        }
+      }
+      gb = wave_max_u32(gb);
+      if ((threadIdx.x & 63) == 0 && gb) atomicMax(now, gb);
+    }
+    if (M1 && live && jj + 1 < j_count) g_ahead = *g_of(jj + 1);
     __syncthreads();
-    if (!live) continue;
-    const Real *gp = gout + ((b * Cout + j) * g.positions() + at.pos) * M;
-    const Real g_one = M1 ? gp[0] : Real(0);
+    if constexpr (kFix) {
+      // bounds -> units. A float's exponent field e means |v| < 2^(e - 126).
+      const uint32_t xb = bnd[1], gb = now[0], tb = now[1], wb = now[2];
+      const bool finite = max(max(xb, gb), max(tb, wb)) < 0x7f800000u;
+      const float g_max = __uint_as_float(gb);
+      const float bound_w = (__uint_as_float(tb) + __uint_as_float(xb)) * g_max;
+      const float bound_c = float(M) * __uint_as_float(wb) * g_max;
+      const int exp_w = int(__float_as_uint(bound_w) >> 23) - 126, exp_c = int(__float_as_uint(bound_c) >> 23) - 126;
+      // (a bound of zero: every term is zero, any unit will do)
+      const bool ok_w = bound_w == 0.f || (exp_w > -90 && exp_w < 90), ok_c = bound_c == 0.f || (exp_c > -90 && exp_c < 90);
+      tab_fixed = finite && ok_w && ok_c;
+      if (tab_fixed) {
+        const int ew = bound_w == 0.f ? 0 : exp_w, ec = bound_c == 0.f ? 0 : exp_c;
+        scale_w = pow2f(29 - ew), unit_w = double(pow2f(ew - 29));
+        scale_t = pow2f(29 - ec), unit_t = double(pow2f(ec - 29));
+      }
+      if (img_fixed) {
+        const int ec = bound_c == 0.f ? -100000 : exp_c;
+        if (!tab_fixed) {
+          // the image goes over to fp64 cells for good
+          if (img_exp > -100000) {
+            const double unit = double(pow2f(img_exp - 29));
+            for (int i = threadIdx.x; i < C * g.TSZ; i += NT) acc[i] = double(reinterpret_cast<long long *>(acc)[i]) * unit;
+          }
+          img_fixed = false;
+          __syncthreads();
+        } else if (ec > img_exp) {
+          // a coarser unit from here on: what the image holds is shifted down to it
+          if (img_exp > -100000) {
+            const int shift = min(ec - img_exp, 63);
+            for (int i = threadIdx.x; i < C * g.TSZ; i += NT)
+              reinterpret_cast<long long *>(acc)[i] = reinterpret_cast<long long *>(acc)[i] >> shift;
+            __syncthreads();
+          }
+          img_exp = ec;
+        }
+        if (img_fixed && img_exp > -100000) scale_x = pow2f(29 - img_exp);
+      }
+    }
+    auto walks = [&]() {
+    if (!live) return;
     if constexpr (kLeanWalk) {
       if (*special == 0) {
+        // (the usual case, every cell an integer, as code of its own: no test per atomic)
+        auto lean_walks = [&](auto all_fixed_tag) {
+        constexpr bool ALL = decltype(all_fixed_tag)::value;
+        const bool tab_f = ALL || tab_fixed, img_f = ALL || img_fixed;
         for (int c = 0; c < C; c += kConvIlp) {
           TrackedPath st[kConvIlp];
           const Node<float> *nd[kConvIlp];
@@ -745,16 +891,21 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
             if (c + i >= C) break;
             const float t = st[i].t;  // thr - x at the selected vertex: margin = -t
             const int cell = ch[i] * L + int(st[i].key(depth));
-            if (dw) atomicAdd(acc_w + cell, double(ht_abs(t) * g_one));
+            if (dw) add(acc_w + cell, ht_abs(t) * g_one, tab_f, scale_w);
             // sign(margin) * (w * g): the product with the sign bit of t flipped in, zero where the margin is zero
             const float wg = wl[cell] * g_one;
             const float cs = t == 0.f ? 0.f
                                       : __uint_as_float(__float_as_uint(wg) ^ (~__float_as_uint(t) & 0x80000000u));
-            if (dthr) atomicAdd(acc_t + ch[i] * V + int(st[i].template vertex<FERN>(depth)), -double(cs));
-            atomicAdd(acc + (px[i] - tile) + int(st[i].ordinal()), double(cs));
+            if (dthr) add(acc_t + ch[i] * V + int(st[i].template vertex<FERN>(depth)), -cs, tab_f, scale_t);
+            add(acc + (px[i] - tile) + int(st[i].ordinal()), cs, img_f, scale_x);
           }
         }
-        continue;
+        };
+        if (tab_fixed && img_fixed)
+          lean_walks(std::true_type{});
+        else
+          lean_walks(std::false_type{});
+        return;
       }
     }
     for (int c = 0; c < C; c += kConvIlp) {
@@ -779,31 +930,39 @@ __global__ __launch_bounds__(NT) void conv_tiled_backward_kernel(ConvTile g, Con
         Real cs = Real(0);
         if (M1) {
           cs += wl[cell] * g_one;
-          if (dw) atomicAdd(acc_w + cell, double(a * g_one));
+          if (dw) add(acc_w + cell, a * g_one, tab_fixed, scale_w);
         } else {
           for (int m = 0; m < M; ++m) {
             const Real gv = gp[m];
             cs += wl[cell + m] * gv;
-            if (dw) atomicAdd(acc_w + cell + m, double(a * gv));
+            if (dw) add(acc_w + cell + m, a * gv, tab_fixed, scale_w);
           }
         }
         cs = ht_sign(r[i].margin) * cs;
-        if (dthr) atomicAdd(acc_t + ch[i] * V + int(r[i].vertex), -double(cs));
-        atomicAdd(acc + ch[i] * g.TSZ + base + int(r[i].ord), double(cs));  // r.ord is the tap's tile offset
+        if (dthr) add(acc_t + ch[i] * V + int(r[i].vertex), -cs, tab_fixed, scale_t);
+        add(acc + ch[i] * g.TSZ + base + int(r[i].ord), cs, img_fixed, scale_x);  // r.ord is the tap's tile offset
       }
     }
+    };
+    walks();
   }
   __syncthreads();
   {
-    const int jp = j_begin + (j_count - 1 + rot >= j_count ? rot - 1 : j_count - 1 + rot);
+    const int jp = j_of(j_count - 1);
     if (dw)
-      for (int i = threadIdx.x; i < C * LM; i += NT)
-        if (acc_w[i] != 0.0) atomicAdd(dw + ((long long)jp * C_all + c0) * LM + i, Real(acc_w[i]));
+      for (int i = threadIdx.x; i < C * LM; i += NT) {
+        const double v = tab_fixed ? double(reinterpret_cast<long long *>(acc_w)[i]) * unit_w : acc_w[i];
+        if (v != 0.0) atomicAdd(dw + ((long long)jp * C_all + c0) * LM + i, Real(v));
+      }
     if (dthr)
-      for (int i = threadIdx.x; i < C * V; i += NT)
-        if (acc_t[i] != 0.0) atomicAdd(dthr + ((long long)jp * C_all + c0) * V + i, Real(acc_t[i]));
+      for (int i = threadIdx.x; i < C * V; i += NT) {
+        const double v = tab_fixed ? double(reinterpret_cast<long long *>(acc_t)[i]) * unit_t : acc_t[i];
+        if (v != 0.0) atomicAdd(dthr + ((long long)jp * C_all + c0) * V + i, Real(v));
+      }
   }
-  flush_dx_image(acc, g, at, C, dx + (b * C_all + c0) * (long long)g.D * g.H * g.W);
+  const bool img_ints = img_fixed && img_exp > -100000;
+  flush_dx_image(acc, g, at, C, dx + (b * C_all + c0) * (long long)g.D * g.H * g.W, img_ints,
+                 img_ints ? double(pow2f(img_exp - 29)) : 1.0);
 }
 
 constexpr int kConvWideThreads = 512;  // workgroup of the one-walk backward kernel

@@ -133,3 +133,55 @@ def test_conv_special_values(dev, special, fern):
     assert rel_err(dx.cpu(), rdx) <= 1e-5
     _, dthr, _, dw = getattr(ops, pre + "backward")(d[0], False, d[1], True, d[2], False, d[3], True, gout.to(dev), *args)
     assert rel_err(dthr.cpu(), rdthr) <= 1e-5 and rel_err(dw.cpu(), rdw) <= 1e-5
+
+
+def _classes_match(got, ref):
+    """NaN, +inf and -inf in the same places."""
+    return (torch.equal(got.isnan(), ref.isnan()) and torch.equal(got.isposinf(), ref.isposinf())
+            and torch.equal(got.isneginf(), ref.isneginf()))
+
+
+@pytest.mark.parametrize("Md", [[], [3]], ids=["one output", "three outputs"])
+@pytest.mark.parametrize("spread", ["growing", "shrinking", "huge and tiny", "zero channels", "inf"])
+def test_conv_backward_gradient_ranges(dev, spread, Md):
+    """The one-walk backward accumulates float gradients in LDS as integers whose unit every workgroup derives, per out
+    channel, from the largest magnitudes it sees; the dX image changes its unit when a later out channel brings larger
+    terms, and out channels whose bound is not finite, or far from 1, are accumulated in fp64 instead. Upstream
+    gradients whose size differs by out channel take every one of these branches. dThr and dW are compared per out
+    channel (each has a unit of its own), dX against its largest entry as everywhere else."""
+    B, C, Cout, size, D, ker = 2, 16, 8, [20, 24], 6, [3, 3]
+    args = (ker, [1, 1], [1, 1], [1, 1])
+    x, thr, ordn, w = make_conv(B, C, Cout, size, D, Md, ker, False, torch.float32, seed=21)
+    ref = ho.conv_forward(x, thr, ordn, w, *args, False)
+    gout = torch.randn(ref.shape, generator=torch.Generator().manual_seed(22))
+    factor = {
+        "growing": [2.0 ** (5 * j) for j in range(Cout)],
+        "shrinking": [2.0 ** (-5 * j) for j in range(Cout)],
+        "huge and tiny": [1e30, 1e-30, 1.0, 1e33, 1e-36, 1e12, 1e-12, 1.0],
+        "zero channels": [0.0, 1.0, 0.0, 0.0, 3.0, 0.0, 1e-3, 0.0],
+        "inf": [1.0] * Cout,
+    }[spread]
+    gout = gout * torch.tensor(factor).view(1, Cout, *([1] * (gout.dim() - 2)))
+    if spread == "inf":
+        gout[1, 3, 7, 11] = float("inf")
+        gout[0, 5, 2, 2] = float("-inf")
+    rdx, rdthr, rdw = ho.conv_backward(x, thr, ordn, w, gout, *args, fern=False)
+    d = [t.to(dev) for t in (x, thr, ordn, w)]
+    dx, dthr, _, dw = ops.tree_conv2d_backward(d[0], True, d[1], True, d[2], False, d[3], True, gout.to(dev), *args)
+    dx, dthr, dw = dx.cpu(), dthr.cpu(), dw.cpu()
+
+    def close(got, want):
+        if not _classes_match(got, want):
+            return False
+        fin = want.isfinite()
+        scale = want[fin].abs().max().item() if fin.any() else 0.0
+        return scale == 0.0 and not got[fin].any() or (got[fin] - want[fin]).abs().max().item() <= 1e-5 * scale
+
+    if spread in ("huge and tiny", "inf"):
+        # (images differ by 60 orders of magnitude only through their out channels: dX per image is one sum over all)
+        assert close(dx, rdx)
+    else:
+        assert rel_err(dx, rdx) <= 1e-5
+    for j in range(Cout):
+        assert close(dthr[j], rdthr[j]), f"dThr of out channel {j}"
+        assert close(dw[j], rdw[j]), f"dW of out channel {j}"
