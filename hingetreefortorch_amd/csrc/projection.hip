@@ -140,10 +140,35 @@ struct GemmArgs {
   bool vec_a, vec_b;
   double *stats;
   const float *bias_i, *bias_j;
+  // A_BN: operand A is not read as it lies in memory but as the batch-norm backward of it, element (i, r) =
+  // bn_rstd[i] * (A(i, r) - mean_1[i] - bn_zhat(i, r) * mean_2[i]) with mean_1[i] = bn_sums[i] / bn_count and
+  // mean_2[i] = bn_sums[n_i + i] / bn_count (bn_zhat laid out like A)
+  const float *bn_zhat, *bn_rstd;
+  const double *bn_sums;
+  double bn_count;
 };
 
-template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS, bool SUM_BATCHES>
-__global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
+// The batch-norm backward of a fetched operand piece: rstd * (a - mean_1 - zh * mean_2) as two fused multiply-adds,
+// a * rstd + (zh * (-rstd * mean_2) + (-rstd * mean_1)) -- a staging step of every reduction step, so its instruction
+// count matters; bn_backward_apply_kernel rounds after each of its four operations instead, and the two forms differ
+// in the last bits.
+// rows: the tile's constants in LDS, [rstd | -rstd * mean_1 | -rstd * mean_2][kTile] (zeros for rows outside the
+// operand, which makes their elements zero; in LDS because the kernel has no registers to spare for twelve more values
+// per thread); row_ok: the piece's reduction index lies inside the operand (outside, the operand contributes zeros).
+__device__ __forceinline__ void bn_backward_piece(Vec4 &a, const Vec4 &zh, const float *rows, bool row_ok) {
+  const int i = (int(threadIdx.x) % 32) * 4;
+  const Vec4 c0 = *reinterpret_cast<const Vec4 *>(rows + i), c1 = *reinterpret_cast<const Vec4 *>(rows + kTile + i),
+             c2 = *reinterpret_cast<const Vec4 *>(rows + 2 * kTile + i);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float v = __builtin_fmaf(a[e], c0[e], __builtin_fmaf(zh[e], c2[e], c1[e]));
+    a[e] = row_ok ? v : 0.f;
+  }
+}
+
+template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS, bool SUM_BATCHES, bool A_BN = false>
+__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(3, 4))) void gemm_kernel(GemmArgs g) {
+  static_assert(!A_BN || (!A_RED_CONTIG && !SUM_BATCHES), "the fused batch-norm backward reads a row-contiguous operand");
   __shared__ float As[2][kRed * kPitch];
   __shared__ float Bs[2][kRed * kPitch];
   const int n_i = g.n_i, n_j = g.n_j, n_r = g.n_r;
@@ -177,19 +202,37 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
   const int steps = max(0, min(chunk, all_steps - step0));
   if (g.splits > 1 && steps == 0) return;
   const bool rows_a_full = g.vec_a && i0 + kTile <= n_i, rows_b_full = g.vec_b && j0 + kTile <= n_j;
+  __shared__ __align__(16) float bn[A_BN ? 3 * kTile : 4];
+  if constexpr (A_BN) {
+    if (threadIdx.x < kTile) {
+      const int i = i0 + int(threadIdx.x);
+      const bool in = i < n_i;
+      const float rstd = in ? g.bn_rstd[i] : 0.f;
+      bn[threadIdx.x] = rstd;
+      bn[kTile + threadIdx.x] = in ? -rstd * float(g.bn_sums[i] / g.bn_count) : 0.f;
+      bn[2 * kTile + threadIdx.x] = in ? -rstd * float(g.bn_sums[n_i + i] / g.bn_count) : 0.f;
+    }
+    __syncthreads();
+  }
   // Pipeline: while step s is multiplied out of LDS buffer s & 1, the operands of step s + 1 (fetched during step
   // s - 1) are written to the other buffer in the middle of the multiply, and the global loads of step s + 2 are in
   // flight. A wavefront therefore issues its LDS writes and address arithmetic in the shadow of its own MFMAs, and one
   // barrier per step remains.
-  auto multiply = [&](const float *as, const float *bs, int kk_begin, int kk_end) {
+  // 32-wide blocks of this wavefront's corner that hold any result at all (wave uniform). In a tile on the ragged edge
+  // of the result the others are skipped: a dLin of 784 columns ends in a tile column with 16 of them, where one
+  // wavefront in two has nothing to multiply and the other one block column instead of two.
+  const int na = __builtin_amdgcn_readfirstlane(max(0, min(2, (n_i - i0 - wi + 31) / 32)));
+  const int nb = __builtin_amdgcn_readfirstlane(max(0, min(2, (n_j - j0 - wj + 31) / 32)));
+  auto multiply = [&](const float *as, const float *bs, int kk_begin, int kk_end, auto edge_tag) {
+    constexpr bool EDGE = decltype(edge_tag)::value;
 #pragma unroll
     for (int kk = kk_begin; kk < kk_end; kk += 2) {
       const float a0 = as[(kk + lk) * kPitch + wi + lr], a1 = as[(kk + lk) * kPitch + wi + 32 + lr];
       const float b0 = bs[(kk + lk) * kPitch + wj + lr], b1 = bs[(kk + lk) * kPitch + wj + 32 + lr];
-      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+      if (!EDGE || (na > 0 && nb > 0)) acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+      if (!EDGE || (na > 0 && nb > 1)) acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+      if (!EDGE || (na > 1 && nb > 0)) acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+      if (!EDGE || (na > 1 && nb > 1)) acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
     }
   };
   // The loop exists twice: for workgroups whose operand tiles all lie inside the matrices (FULL: exactly four
@@ -197,34 +240,68 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
   // and for the edge tiles (bounds checks, a data-dependent number of loads, hence full waits).
   auto run = [&](auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
-    auto fetch = [&](Fetch &fa, Fetch &fb, int s) {
+    // (A_BN: an operand piece of A travels with the matching piece of zhat, in the second half of the same structure)
+    struct FetchA {
+      Fetch a, zh;
+    };
+    auto fetch = [&](FetchA &fa, Fetch &fb, int s) {
       const int gs = s + step0;
       const int z = SUM_BATCHES ? gs / per_batch : 0;
       const int r0 = (gs - z * per_batch) * kRed;
-      fetch_tile<A_RED_CONTIG>(fa, A + (long long)z * g.stride_a, g.lda, i0, n_i, r0, n_r, g.vec_a, FULL);
+      fetch_tile<A_RED_CONTIG>(fa.a, A + (long long)z * g.stride_a, g.lda, i0, n_i, r0, n_r, g.vec_a, FULL);
+      if constexpr (A_BN) fetch_tile<false>(fa.zh, g.bn_zhat, g.lda, i0, n_i, r0, n_r, g.vec_a, FULL);
       fetch_tile<B_RED_CONTIG>(fb, B + (long long)z * g.stride_b, g.ldb, j0, n_j, r0, n_r, g.vec_b, FULL);
     };
-    Fetch fa0, fb0, fa1, fb1;
+    // operands of step s from registers into an LDS buffer
+    auto stash = [&](int buffer, FetchA &fa, const Fetch &fb, int s) {
+      if constexpr (A_BN) {
+        const int r0 = (s + step0) * kRed;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          bn_backward_piece(fa.a.v[h], fa.zh.v[h], bn, FULL || r0 + int(threadIdx.x) / 32 + 8 * h < n_r);
+      }
+      stash_tile<A_RED_CONTIG>(As[buffer], fa.a);
+      stash_tile<B_RED_CONTIG>(Bs[buffer], fb);
+    };
+    if constexpr (A_BN) {
+      // One step of lookahead only: the operands of step s + 1 are requested when step s begins and written to LDS
+      // when its products are done. With zhat travelling beside A, two steps in flight need more registers than three
+      // wavefronts per SIMD leave, and the third wavefront hides more latency than the second step ahead did.
+      FetchA fa;
+      Fetch fb;
+      if (steps > 0) {
+        fetch(fa, fb, 0);
+        stash(0, fa, fb, 0);
+      }
+      __syncthreads();
+      for (int s = 0; s < steps; ++s) {
+        const int cur = s & 1;
+        const bool more = s + 1 < steps;
+        if (more) fetch(fa, fb, s + 1);
+        multiply(As[cur], Bs[cur], 0, kRed, std::integral_constant<bool, !FULL>{});
+        if (more) stash(cur ^ 1, fa, fb, s + 1);
+        __syncthreads();
+      }
+      return;
+    }
+    FetchA fa0, fa1;
+    Fetch fb0, fb1;
     if (steps > 0) {
       fetch(fa0, fb0, 0);
-      stash_tile<A_RED_CONTIG>(As[0], fa0);
-      stash_tile<B_RED_CONTIG>(Bs[0], fb0);
+      stash(0, fa0, fb0, 0);
       if (steps > 1) fetch(fa0, fb0, 1);
     }
     __syncthreads();
     // one step: `held` carries the operands of step s + 1, `next` receives those of step s + 2. PREFETCH is a
     // compile-time property of the call site: the steady-state loop always fetches (so the wait in front of the LDS
     // writes may leave exactly those newest loads in flight), the last two steps never do.
-    auto step = [&](int s, Fetch &held_a, Fetch &held_b, Fetch &next_a, Fetch &next_b, auto prefetch_tag) {
+    auto step = [&](int s, FetchA &held_a, Fetch &held_b, FetchA &next_a, Fetch &next_b, auto prefetch_tag) {
       constexpr bool PREFETCH = decltype(prefetch_tag)::value;
       const int cur = s & 1;
       if (PREFETCH) fetch(next_a, next_b, s + 2);
-      multiply(As[cur], Bs[cur], 0, kRed / 2);
-      if (PREFETCH || s + 1 < steps) {
-        stash_tile<A_RED_CONTIG>(As[cur ^ 1], held_a);
-        stash_tile<B_RED_CONTIG>(Bs[cur ^ 1], held_b);
-      }
-      multiply(As[cur], Bs[cur], kRed / 2, kRed);
+      multiply(As[cur], Bs[cur], 0, kRed / 2, std::integral_constant<bool, !FULL>{});
+      if (PREFETCH || s + 1 < steps) stash(cur ^ 1, held_a, held_b, s + 1);
+      multiply(As[cur], Bs[cur], kRed / 2, kRed, std::integral_constant<bool, !FULL>{});
       __syncthreads();
     };
     int s = 0;
@@ -409,17 +486,25 @@ bool aligned16(const void *p, long long ld, long long stride) {
   return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0 && stride % 4 == 0;
 }
 
-template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS, bool SUM_BATCHES>
+// The batch-norm backward that a product applies to its operand A while loading it (see GemmArgs).
+struct BnOperand {
+  const float *zhat, *rstd;
+  const double *sums;
+  double count;
+};
+
+template <bool A_RED_CONTIG, bool B_RED_CONTIG, bool STATS, bool SUM_BATCHES, bool A_BN = false>
 int launch_gemm_batched(const float *A, long long lda, long long stride_a, const float *B, long long ldb,
                         long long stride_b, float *C, long long ldc, long long stride_c, long long n_i, long long n_j,
                         long long n_r, long long batches, double *stats, const float *bias_i, const float *bias_j,
-                        hipStream_t stream, bool allow_split = false, float *partials = nullptr, int ordered_splits = 0) {
+                        hipStream_t stream, bool allow_split = false, float *partials = nullptr, int ordered_splits = 0,
+                        const BnOperand *bn = nullptr) {
   if (n_i <= 0 || n_j <= 0 || batches <= 0) return HT_OK;
   if (!SUM_BATCHES && batches > kMaxGridZ) {
     // one result per batch rides on blockIdx.z: longer batch lists go out in several launches
     for (long long b0 = 0; b0 < batches; b0 += kMaxGridZ) {
       const long long nb = batches - b0 < kMaxGridZ ? batches - b0 : kMaxGridZ;
-      int rc = launch_gemm_batched<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES>(
+      int rc = launch_gemm_batched<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES, false>(
           A + b0 * stride_a, lda, stride_a, B + b0 * stride_b, ldb, stride_b, C + b0 * stride_c, ldc, stride_c, n_i, n_j,
           n_r, nb, stats, bias_i, bias_j, stream, allow_split);
       if (rc != HT_OK) return rc;
@@ -441,6 +526,12 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
   if (slots > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: matrix product too large for this build.");
   g.vec_a = aligned16(A, lda, stride_a), g.vec_b = aligned16(B, ldb, stride_b);
   g.stats = stats, g.bias_i = bias_i, g.bias_j = bias_j;
+  g.bn_zhat = g.bn_rstd = nullptr, g.bn_sums = nullptr, g.bn_count = 1.0;
+  if (A_BN) {
+    if (!bn || batches != 1) return fail(HT_ERR_RUNTIME, "Error: fused batch-norm operand needs its statistics.");
+    g.bn_zhat = bn->zhat, g.bn_rstd = bn->rstd, g.bn_sums = bn->sums, g.bn_count = bn->count;
+    g.vec_a = g.vec_a && aligned16(bn->zhat, lda, 0);
+  }
   // A product with few result tiles and a long reduction (dLin of a narrow linear head: 10 x 1000 from 65536 rows)
   // would leave most of the device idle: the reduction is then split over blockIdx.y and the shares are added into
   // the zeroed result with float atomics (a few thousand elements times the number of shares).
@@ -452,7 +543,7 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
     g.splits = ordered_splits;
     g.split_stride = n_i * n_j;
     g.C = partials;
-    hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES>),
+    hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES, A_BN>),
                        dim3((unsigned)slots, (unsigned)g.splits, 1u), dim3(kGemmThreads), 0, stream, g);
     HT_LAUNCH_CHECK("matrix product (matrix cores, split reduction)");
     const long long chunk = (all_steps + g.splits - 1) / g.splits;
@@ -473,7 +564,7 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
       if (rc != HT_OK) return rc;
     }
   }
-  hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES>),
+  hipLaunchKernelGGL((gemm_kernel<A_RED_CONTIG, B_RED_CONTIG, STATS, SUM_BATCHES, A_BN>),
                      dim3((unsigned)slots, (unsigned)g.splits, (unsigned)(SUM_BATCHES ? 1 : batches)), dim3(kGemmThreads),
                      0, stream, g);
   HT_LAUNCH_CHECK("matrix product (matrix cores)");
@@ -501,13 +592,27 @@ int gemm_tile_map(int tiles_i, int tiles_j, int *tile_i, int *tile_j) {
 
 size_t projection_workspace(long long N) { return align_up(size_t(2) * size_t(N) * sizeof(double), 256); }
 
-// Shares of the reduction of a product with rows x cols results over `red` terms (1: no split). Few result tiles and
-// a long reduction only.
+// Shares of the reduction of a product with rows x cols results over `red` terms (1: no split): long reductions whose
+// result tiles do not fill the device evenly by themselves.
 int reduction_shares(long long rows, long long cols, long long red) {
   const long long tiles = ((rows + kTile - 1) / kTile) * ((cols + kTile - 1) / kTile), steps = (red + kRed - 1) / kRed;
-  if (tiles <= 0 || tiles >= kNumCUs / 2 || steps < 64) return 1;
-  long long want = (2 * kNumCUs + tiles - 1) / tiles;
-  if (want > steps / 16) want = steps / 16;
+  if (tiles <= 0 || steps < 64) return 1;
+  long long want;
+  if (tiles < kNumCUs / 2) {
+    // a handful of tiles: enough shares to put two workgroups on every CU
+    want = (2 * kNumCUs + tiles - 1) / tiles;
+    if (want > steps / 16) want = steps / 16;
+  } else {
+    // A few tiles per CU: tiles are equal pieces of work, so 700 of them leave some CUs with three and some with two
+    // while the product takes as long as three. About twenty pieces per CU level that out (the README model's dLin,
+    // 100 x 7 tiles over 16 384 rows: backward pass 4.22 ms with one share, 3.90 with six, 3.79 with eight, 3.86 with
+    // sixteen, the sum of the shares included), each still a reduction of 64 steps or more and all of them together
+    // within a GiB of partial results.
+    want = (20 * kNumCUs + tiles - 1) / tiles;
+    if (want > steps / 64) want = steps / 64;
+    const long long bytes = rows * cols * (long long)sizeof(float);
+    if (bytes > 0 && want > (1LL << 30) / bytes) want = (1LL << 30) / bytes;
+  }
   return want > 1 ? int(want) : 1;
 }
 // dLin [N x K] reduces over the batch, dX [B x K] over the N columns; the two products run one after the other and
@@ -540,7 +645,8 @@ int projection_forward(long long B, long long K, long long N, const float *x, co
   return HT_OK;
 }
 
-// g [B x N] holds dL/dzhat on entry and dL/dz on return. dlin [N x K] and / or dx [B x K] out (either may be null).
+// g [B x N] holds dL/dzhat on entry; where dx is wanted it holds dL/dz on return, otherwise it is left as it came.
+// dlin [N x K] and / or dx [B x K] out (either may be null).
 int projection_backward(long long B, long long K, long long N, const float *x, const float *lin, const float *zhat,
                         const float *rstd, float *g, float *dlin, float *dx, void *ws, hipStream_t stream) {
   int rc;
@@ -554,12 +660,20 @@ int projection_backward(long long B, long long K, long long N, const float *x, c
   const dim3 grid((unsigned)((N + 1023) / 1024), (unsigned)rows_grid(B));
   hipLaunchKernelGGL(bn_backward_sums_kernel, grid, dim3(256), 0, stream, g, zhat, B, int(N), sums);
   HT_LAUNCH_CHECK("batch-norm backward (sums)");
+  float *partials = reinterpret_cast<float *>(static_cast<unsigned char *>(ws) + projection_workspace(N));
+  if (dlin && !dx) {
+    // dLin alone, the training case of a first layer: dL/dz is not written out and read back, the product's loader
+    // turns dL/dzhat into it on the way into LDS (same arithmetic, same dLin bit for bit); g stays as it came
+    const BnOperand bn = {zhat, rstd, sums, double(B)};
+    return launch_gemm_batched<false, false, false, false, true>(g, N, 0, x, K, 0, dlin, K, 0, N, K, B, 1, nullptr, nullptr,
+                                                                  nullptr, stream, false, partials,
+                                                                  reduction_shares(N, K, B), &bn);
+  }
   hipLaunchKernelGGL(bn_backward_apply_kernel, grid, dim3(256), 0, stream, g, zhat, B, int(N), rstd, sums);
   HT_LAUNCH_CHECK("batch-norm backward");
   // dlin[n, k] = sum_b g[b, n] * x[b, k]: both operands row contiguous, reduction over the batch. A small layer under a
   // large batch has a handful of result tiles and a long reduction: it is then split over workgroups whose shares are
   // summed in a fixed order (reproducible, unlike a split that meets in atomics).
-  float *partials = reinterpret_cast<float *>(static_cast<unsigned char *>(ws) + projection_workspace(N));
   if (dlin && (rc = launch_gemm_batched<false, false, false, false>(g, N, 0, x, K, 0, dlin, K, 0, N, K, B, 1, nullptr,
                                                                      nullptr, nullptr, stream, false, partials,
                                                                      reduction_shares(N, K, B))) != HT_OK)

@@ -384,8 +384,9 @@ def linear_bn_forward(inData, inLinearWeights, eps=1e-5):
 
 
 def linear_bn_backward(inData, bInDataGrad, inLinearWeights, bInLinearWeightsGrad, zhat, rstd, outDataGrad):
-    """Gradients of linear_bn_forward for an upstream gradient on zhat. `outDataGrad` is overwritten (it becomes the
-    gradient with respect to the un-normalised product). Returns [dData | None, dLinearWeights | None]."""
+    """Gradients of linear_bn_forward for an upstream gradient on zhat. With bInDataGrad, `outDataGrad` is overwritten
+    (it becomes the gradient with respect to the un-normalised product); without, it is left as it came.
+    Returns [dData | None, dLinearWeights | None]."""
     for t in (inData, inLinearWeights, zhat, rstd, outDataGrad):
         if t.dtype != torch.float32:
             _invalid("Error: the projection supports torch.float32 only.")

@@ -175,8 +175,9 @@ int ht_conv_backward(const ht_conv_shape *s, const void *x, const void *thr, con
  *   forward : zhat [B, N] = (z - mean) * rstd with z = x [B, K] * lin [N, K]^T computed on the matrix cores; the batch
  *             sums of z are accumulated by the same kernel. mean, rstd, var [N] are outputs (var: biased variance, for
  *             the caller's running statistics; may be NULL).
- *   backward: g [B, N] holds dL/dzhat on entry and is overwritten with dL/dz; dlin [N, K] and dx [B, K] receive the
- *             parameter / input gradients (either may be NULL).
+ *   backward: g [B, N] holds dL/dzhat on entry; dlin [N, K] and dx [B, K] receive the parameter / input gradients
+ *             (either may be NULL). With dx, g is overwritten with dL/dz; without it g is left as it came (the
+ *             normalisation's backward is then applied while the dlin product loads g, with the same result).
  * workspace: ht_projection_workspace(N) bytes for the forward pass, ht_projection_backward_workspace(B, K, N) for the
  * backward pass (a small layer under a large batch splits the batch reduction of dlin over workgroups and sums their
  * shares in a fixed order, so the result does not depend on scheduling). */

@@ -143,8 +143,8 @@ def test_projection_full_size(dev):
         dz = rstd[cs].double() * (gd - gd.mean(0) - rz * (gd * rz).mean(0))
         want = dz.t() @ x64
         assert rel_err(dlin[cs].double(), want) <= 2e-5, cs
-        # the in-place batch-norm backward left dL/dz in the gradient buffer
-        assert rel_err(dz_in[:, cs].double(), dz) <= 1e-5, cs
+    # dLin alone: the batch-norm backward ran inside the product's operand loader, the gradient buffer is as it came
+    assert torch.equal(dz_in, up)
 
 
 def test_conv_full_size(dev):

@@ -51,8 +51,13 @@ def test_projection_forward_backward(dev, shape):
     scale = max(float(rrstd.abs().max()), 1.0)   # near-constant columns amplify rounding by rstd
     assert rel_err(dlin.cpu().double(), rdlin) <= 2e-5 * scale
     assert rel_err(dx.cpu().double(), rdx) <= 2e-5 * scale
-    only = ops.linear_bn_backward(x.to(dev), False, lin.to(dev), True, zhat, rstd, up.to(dev).clone())
+    # dLin alone: the batch-norm backward runs inside the product's operand loader instead of as a pass of its own (two
+    # fused multiply-adds there, four rounded operations in the pass); the upstream gradient is left untouched
+    gkeep = up.to(dev).clone()
+    only = ops.linear_bn_backward(x.to(dev), False, lin.to(dev), True, zhat, rstd, gkeep)
     assert only[0] is None and rel_err(only[1].cpu().double(), rdlin) <= 2e-5 * scale
+    assert torch.equal(gkeep.cpu(), up)
+    assert not torch.equal(gbuf.cpu(), up)  # (with the input gradient, it was overwritten with dL/dz)
 
 
 @pytest.mark.parametrize("shape", [(40000, 48, 300), (192, 40, 9000)], ids=["small layer, large batch", "wide layer, small batch"])
@@ -73,6 +78,9 @@ def test_split_reductions(dev, shape):
     runs = [ops.linear_bn_backward(x.to(dev), True, lin.to(dev), True, zhat, rstd, up.to(dev).clone()) for _ in range(2)]
     assert torch.equal(runs[0][1], runs[1][1]) and torch.equal(runs[0][0], runs[1][0])
     scale = max(float(rrstd.abs().max()), 1.0)
+    # dLin alone (batch-norm backward inside the product): reproducible as well
+    only = [ops.linear_bn_backward(x.to(dev), False, lin.to(dev), True, zhat, rstd, up.to(dev).clone()) for _ in range(2)]
+    assert torch.equal(only[0][1], only[1][1]) and rel_err(only[0][1].cpu().double(), rdlin) <= 2e-5 * scale
     assert rel_err(runs[0][1].cpu().double(), rdlin) <= 2e-5 * scale
     assert rel_err(runs[0][0].cpu().double(), rdx) <= 2e-5 * scale
 
