@@ -257,6 +257,8 @@ def bench_projection(torch, ops, dev, args):
     thr, ordn, w = thr.to(dev), ordn.to(dev), w.to(dev)
     gout = torch.randn([B, T, M], generator=torch.Generator(device=dev).manual_seed(6113), device=dev)
 
+    dense = bool(getattr(args, "dense_backward", False))
+
     def step(ev=None):
         if ev: ev[0].record()
         zhat, mean, rstd, var = ops.linear_bn_forward(x, lin, 1e-5)
@@ -264,9 +266,17 @@ def bench_projection(torch, ops, dev, args):
         # the training path of the autograd function: the forward keeps its walk records for the backward
         out, rec = ops.tree_forward_records(zhat, thr, ordn, w)
         if ev: ev[2].record()
-        dz, dthr, _, dw = ops.tree_backward_records(rec, False, zhat, True, thr, True, ordn, False, w, True, gout)
-        if ev: ev[3].record()
-        ops.linear_bn_backward(x, False, lin, True, zhat, rstd, dz)
+        if dense:
+            # dense route: the forest's input gradient as a [B, N] matrix, batch-norm backward, dLin = dz^T x
+            dz, dthr, _, dw = ops.tree_backward_records(rec, False, zhat, True, thr, True, ordn, False, w, True, gout)
+            if ev: ev[3].record()
+            ops.linear_bn_backward(x, False, lin, True, zhat, rstd, dz)
+        else:
+            # all three gradients from the walk records; the forest's input gradient (one non-zero per sample and
+            # tree) is never formed
+            if ev: ev[3].record()
+            got = ops.tree_linear_bn_backward_records(rec, x, lin, True, zhat, rstd, thr, True, ordn, w, True, gout)
+            assert got is not None
         if ev: ev[4].record()
 
     for _ in range(args.warmup):
@@ -292,9 +302,13 @@ def bench_projection(torch, ops, dev, args):
                    "T": T, "depth": depth, "extra_outputs": M},
         "projection_forward": {"ms": seg[0], "tflops": tf_fwd,
                                "note": "GEMM with fused batch sums + statistics + in-place normalisation"},
-        "forest_forward_ms": seg[1], "forest_backward_ms": seg[2],
-        "projection_backward": {"ms": seg[3], "tflops": tf_bwd,
-                                "note": "batch-norm backward (two passes over [B, N]) + dLin = dz^T x GEMM"},
+        "forest_forward_ms": seg[1], "forest_backward_ms": seg[2] if dense else None,
+        "projection_backward": {"ms": seg[3], "tflops": tf_bwd if dense else None,
+                                "note": "batch-norm backward sums + dLin = dz^T x GEMM with the normalisation's backward "
+                                        "in its operand loader" if dense else
+                                        "forest backward (dThr, dW) + dLin from the walk records: segment sums of centred "
+                                        "inputs per (tree, vertex), xc^T xc and lin * (xc^T xc) on the matrix cores "
+                                        "(--dense-backward times the dense route)"},
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (projection forward)", "achieved": tf_fwd,
                      "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf_fwd / MFMA_FP32_PEAK_TFLOPS,
                      "traffic": None, "flops": flops,
@@ -418,6 +432,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--dense-backward", action="store_true",
+                    help="c5: backward through a dense dL/dzhat (forest dX, batch-norm backward, dz^T x) instead of "
+                         "the records form")
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "c5", "f1", "f3"])
     ap.add_argument("--mode", default="atomic", choices=["atomic", "deterministic"])
     ap.add_argument("--path", default="train", choices=["train", "stateless"])

@@ -570,6 +570,33 @@ int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, cons
   return projection_backward(B, K, N, x, lin, zhat, rstd, g, dlin, dx, workspace, static_cast<hipStream_t>(stream));
 }
 
+size_t ht_projection_forest_backward_workspace(const ht_forest_shape *forest, int64_t K_in) {
+  ForestDims d;
+  if (!forest || forest->dtype != HT_F32 || make_dims(forest, &d) != HT_OK) return 0;
+  return projection_forest_backward_workspace(d, K_in);
+}
+
+int ht_projection_forest_backward(const ht_forest_shape *forest, int64_t K_in, const float *x, const float *lin,
+                                  const float *zhat, const float *rstd, const float *w, const float *gout,
+                                  const void *records, size_t records_bytes, float *dthr, float *dw, float *dlin,
+                                  void *workspace, size_t workspace_bytes, void *stream) {
+  ForestDims d;
+  if (!forest) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  int rc = make_dims(forest, &d);
+  if (rc != HT_OK) return rc;
+  if (forest->dtype != HT_F32) return fail(HT_ERR_INVALID_ARGUMENT, "Error: the projection supports float32 only.");
+  if (!projection_forest_backward_ok(d, K_in))
+    return fail(HT_ERR_INVALID_ARGUMENT,
+                "Error: this shape is not served by the records form of the projection backward "
+                "(ht_projection_forest_backward_workspace returns 0 for it).");
+  if (!x || !lin || !zhat || !rstd || !w || !gout || !records || !workspace)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (records_bytes < ht_forest_records_bytes(forest))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: records buffer too small.");
+  return projection_forest_backward(d, forest->kind == HT_FERN, K_in, x, lin, zhat, rstd, w, gout, records, dthr, dw,
+                                    dlin, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 int ht_gemm_tile_map(int32_t tiles_i, int32_t tiles_j, int32_t *tile_i, int32_t *tile_j, int64_t capacity) {
   if (tiles_i < 1 || tiles_j < 1) return fail(HT_ERR_INVALID_ARGUMENT, "Error: a tile grid needs at least one tile.");
   const long long slots = (long long)((tiles_i + kNumXCDs - 1) / kNumXCDs) * tiles_j * kNumXCDs;

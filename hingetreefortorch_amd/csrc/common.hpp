@@ -130,6 +130,14 @@ template <typename Real>
 int forest_backward_records(const ForestDims &d, bool fern, const Real *w, const Real *gout, const void *records,
                             Real *dx, Real *dthr, Real *dw, int mode, void *ws, size_t ws_bytes, hipStream_t stream);
 
+// ... for dThr / dW alone, leaving c = sign(margin) * sum_m w * g of every pair, tree major [T][S], at the start of the
+// workspace (*c) for a caller that goes on from the records itself; atomic mode, where forest_backward_keeps_c says so.
+template <typename Real>
+bool forest_backward_keeps_c(const ForestDims &d);
+template <typename Real>
+int forest_backward_records_keep_c(const ForestDims &d, bool fern, const Real *w, const Real *gout, const void *records,
+                                   Real *dthr, Real *dw, void *ws, size_t ws_bytes, hipStream_t stream, const Real **c);
+
 // The maps on the forward's row kernel walk (forest_forward.hip): bytes of packed vertices it wants (0: shape not
 // served), and the launch; keys16 (optional) receives the leaf keys as 16-bit values tree major.
 template <typename Real>
@@ -178,6 +186,14 @@ int projection_forward(long long B, long long K, long long N, const float *x, co
                        float *zhat, float *mean, float *rstd, float *var, void *ws, hipStream_t stream);
 int projection_backward(long long B, long long K, long long N, const float *x, const float *lin, const float *zhat,
                         const float *rstd, float *g, float *dlin, float *dx, void *ws, hipStream_t stream);
+// The same gradients for the whole Linear -> BatchNorm -> forest front from the forest's walk records: dThr, dW and
+// dLin without a dense dL/dzhat (d: the forest over the N = d.F projected features of B = d.S samples, K_in inputs).
+bool projection_forest_backward_ok(const ForestDims &d, long long K_in);
+size_t projection_forest_backward_workspace(const ForestDims &d, long long K_in);
+int projection_forest_backward(const ForestDims &d, bool fern, long long K_in, const float *x, const float *lin,
+                               const float *zhat, const float *rstd, const float *w, const float *gout,
+                               const void *records, float *dthr, float *dw, float *dlin, void *ws, size_t ws_bytes,
+                               hipStream_t stream);
 // Host-side view of the matrix-product kernel's workgroup -> result-tile map for tiles_i x tiles_j tiles: writes the
 // tile of every launch slot (-1, -1 for a slot without a tile) and returns the number of slots.
 int gemm_tile_map(int tiles_i, int tiles_j, int *tile_i, int *tile_j);

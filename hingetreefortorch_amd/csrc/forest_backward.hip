@@ -2056,12 +2056,12 @@ int launch_absmax(const Real *p, long long n, unsigned long long *slot, hipStrea
 template <typename Real, bool FERN, bool COMPACT, bool FIXED>
 int backward_staged(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, const Real *gout,
                     Real *dx, Real *dthr, Real *dw, Records<Real, COMPACT> rec, bool walk, void *fixed_ws,
-                    hipStream_t stream, const ImageStore *gout_image = nullptr) {
+                    hipStream_t stream, const ImageStore *gout_image = nullptr, bool keep_c = false) {
   int rc = HT_OK;
   if (FIXED && gout_image != nullptr)
     return fail(HT_ERR_RUNTIME, "Error: the deterministic mode cannot read the upstream gradient as an image.");
   if (walk && (rc = dispatch_records<Real, FERN, COMPACT>(d, x, nodes, rec, stream)) != HT_OK) return rc;
-  const bool need_c = dx || dthr;
+  const bool need_c = dx || dthr || keep_c;  // keep_c: the caller goes on from c itself
   const long long pairs = (long long)d.T * d.S;
   TreePlan plan;
   constexpr bool kLean = std::is_same<Real, float>::value && COMPACT;
@@ -2257,7 +2257,7 @@ size_t route_bytes(const ForestDims &d, Route r, bool need_dthr, bool need_dw, b
 template <typename Real>
 int run_route(const ForestDims &d, Route route, bool fern, const Real *x, const Node<Real> *nodes, const Real *w,
               const Real *gout, Real *dx, Real *dthr, Real *dw, void *saved, void *scratch, bool walk,
-              hipStream_t stream, const ImageStore *gout_image = nullptr) {
+              hipStream_t stream, const ImageStore *gout_image = nullptr, bool keep_c = false) {
   if (gout_image != nullptr && route != Route::kStaged)
     return fail(HT_ERR_RUNTIME, "Error: this shape cannot read the upstream gradient as an image.");
   void *fixed_ws = static_cast<unsigned char *>(scratch) + records_scratch_bytes<Real>(d);
@@ -2265,7 +2265,7 @@ int run_route(const ForestDims &d, Route route, bool fern, const Real *x, const 
 #define HT_STAGED(FERN_, COMPACT_, FIXED_)                                                            \
   backward_staged<Real, FERN_, COMPACT_, FIXED_>(d, x, nodes, w, gout, dx, dthr, dw,                  \
                                                  carve_records<Real, COMPACT_>(d, saved, scratch), walk, fixed_ws, stream, \
-                                                 gout_image)
+                                                 gout_image, keep_c)
 #define HT_SEQ(FERN_, COMPACT_)                                                                       \
   backward_sequential<Real, FERN_, COMPACT_>(d, x, nodes, w, gout, dx, dthr, dw,                      \
                                              carve_records<Real, COMPACT_>(d, saved, scratch), walk, stream)
@@ -2390,7 +2390,37 @@ int forest_backward_records(const ForestDims &d, bool fern, const Real *w, const
                          const_cast<void *>(records), ws, false, stream);
 }
 
+// The backward pass from records for dThr / dW alone that leaves c = sign(margin) * sum_m w * g of every pair, tree
+// major [T][S], at the start of the workspace: for callers inside the library that turn the records and c into an
+// input-side gradient of their own instead of a dense dX. Atomic mode on the staged kernels only --
+// forest_backward_keeps_c says whether a shape is served; workspace: forest_backward_records_workspace(d, atomic,
+// false, true, true).
+template <typename Real>
+bool forest_backward_keeps_c(const ForestDims &d) {
+  if (is_empty(d) || forest_records_bytes<Real>(d) == 0) return false;
+  return pick_route<Real>(d, HT_BACKWARD_ATOMIC, false, true, true) == Route::kStaged;
+}
+
+template <typename Real>
+int forest_backward_records_keep_c(const ForestDims &d, bool fern, const Real *w, const Real *gout, const void *records,
+                                   Real *dthr, Real *dw, void *ws, size_t ws_bytes, hipStream_t stream, const Real **c) {
+  int rc;
+  if (!forest_backward_keeps_c<Real>(d)) return fail(HT_ERR_RUNTIME, "Error: this shape keeps no c in its workspace.");
+  const Route route = Route::kStaged;
+  bool done;
+  if ((rc = clear_gradients<Real>(d, route, (Real *)nullptr, dthr, dw, stream, &done)) != HT_OK) return rc;
+  const size_t need = route_bytes<Real>(d, route, true, true, true);
+  if (ws == nullptr || ws_bytes < need)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the backward pass.");
+  *c = static_cast<const Real *>(ws);
+  return run_route<Real>(d, route, fern, (const Real *)nullptr, (const Node<Real> *)nullptr, w, gout, (Real *)nullptr,
+                         dthr, dw, const_cast<void *>(records), ws, false, stream, nullptr, true);
+}
+
 #define HT_INSTANTIATE(Real)                                                                                          \
+  template bool forest_backward_keeps_c<Real>(const ForestDims &);                                                    \
+  template int forest_backward_records_keep_c<Real>(const ForestDims &, bool, const Real *, const Real *, const void *, \
+                                                    Real *, Real *, void *, size_t, hipStream_t, const Real **);      \
   template size_t forest_backward_workspace<Real>(const ForestDims &, int, bool, bool, bool);                         \
   template int forest_backward<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,           \
                                      const Real *, const Real *, Real *, Real *, Real *, int, void *, size_t,         \

@@ -13,6 +13,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "records.hpp"
 
 namespace ht {
 namespace {
@@ -684,6 +685,327 @@ int projection_backward(long long B, long long K, long long N, const float *x, c
                                                                   nullptr, nullptr, stream, false, partials,
                                                                   reduction_shares(B, K, N))) != HT_OK)
     return rc;
+  return HT_OK;
+}
+
+namespace {
+
+// ---- dLin of Linear -> BatchNorm(affine = False) -> forest, from the forest's walk records ------------------------
+//
+// The upstream gradient of the normalisation, g = dL/dzhat [B x N], is the forest's dX: one non-zero per (sample, tree)
+// pair -- c at the feature the selected vertex looks at -- so B * T entries out of B * N (1.6 M of 208 M for the README
+// model). Instead of writing that matrix densely, summing its columns, normalising it and multiplying it by x as a dense
+// 2 * B * N * K product, the gradient is taken apart:
+//   dz = rstd * (g - m1 - zhat * m2),  m1 = mean_b g,  m2 = mean_b (g * zhat)            (batch-norm backward)
+//   dLin[n, k] = sum_b dz[b, n] * x[b, k]
+//              = rstd[n] * (sum_b g[b, n] * xc[b, k]  -  m2[n] * sum_b zhat[b, n] * xc[b, k])
+// with xc = x - mean_b x: the m1 term vanishes against the centring (sum_b xc = 0), and centring costs nothing on the
+// zhat term because sum_b zhat = 0. The second sum is rstd[n] * (lin * Gc)[n, k] with Gc = xc^T xc [K x K], since
+// zhat = (x lin^T - mean) * rstd: two small dense products (2 B K^2 + 2 N K^2 operations instead of 2 B N K).
+// The first sum is sparse: per (tree, vertex) the rows of xc of the samples that selected it, weighted by c. No term is
+// a difference of large numbers. m2 is sparse as well: c * zhat at the selected feature.
+//
+// Steps: column means of x and xc; per tree the samples bucketed by selected vertex (counting sort in LDS); one
+// wavefront per (tree, vertex) segment sums c * xc rows in registers (lanes along K) and c * zhat; the two products on
+// the matrix cores; an elementwise combination. The order of a segment's samples depends on scheduling (bucket cursors
+// are LDS atomics), so like every atomic-mode gradient the last bits can differ between runs.
+
+constexpr int kBucketThreads = 1024;
+constexpr int kMaxBucketVertices = 16384;  // LDS counters of the bucketing kernel
+
+// sums[k] += sum_b x[b, k] (fp64 atomics). A workgroup takes 64 column quads x a share of the rows, its four wavefronts
+// alternate rows and meet in LDS: one atomic per column and workgroup.
+__global__ __launch_bounds__(256) void col_sums_kernel(const float *__restrict__ x, long long B, int K, double *sums) {
+  __shared__ double part[3][kWave][4];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int k = (blockIdx.x * kWave + lane) * 4;
+  double s[4] = {0, 0, 0, 0};
+  if (k < K)
+    for (long long b = (long long)blockIdx.y * 4 + wave; b < B; b += (long long)gridDim.y * 4) {
+      const Vec4 v = *reinterpret_cast<const Vec4 *>(x + b * K + k);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] += double(v[e]);
+    }
+  if (wave > 0)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) part[wave - 1][lane][e] = s[e];
+  __syncthreads();
+  if (wave == 0 && k < K)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) atomicAdd(sums + k + e, s[e] + part[0][lane][e] + part[1][lane][e] + part[2][lane][e]);
+}
+
+// xc[b, k] = x[b, k] - float(sums[k] / B)
+__global__ __launch_bounds__(256) void center_kernel(const float *__restrict__ x, long long B, int K,
+                                                     const double *__restrict__ sums, float *__restrict__ xc) {
+  const int k = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (k >= K) return;
+  float m[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) m[e] = float(sums[k + e] / double(B));
+  for (long long b = blockIdx.y; b < B; b += gridDim.y) {
+    Vec4 v = *reinterpret_cast<const Vec4 *>(x + b * K + k);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] -= m[e];
+    *reinterpret_cast<Vec4 *>(xc + b * K + k) = v;
+  }
+}
+
+// One workgroup per tree: the tree's S samples ordered by the vertex they selected, as sample indices in perm[t][.].
+template <bool COMPACT>
+__global__ __launch_bounds__(kBucketThreads) void bucket_kernel(ForestDims d, Records<float, COMPACT> rec,
+                                                                uint32_t *__restrict__ perm) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint32_t *count = reinterpret_cast<uint32_t *>(smem);  // [V], then the segments' cursors
+  __shared__ uint32_t wave_total[kBucketThreads / kWave];
+  const int t = blockIdx.x;
+  const long long first = (long long)t * d.S;
+  for (int v = threadIdx.x; v < d.V; v += kBucketThreads) count[v] = 0u;
+  __syncthreads();
+  for (long long s = threadIdx.x; s < d.S; s += kBucketThreads) atomicAdd(&count[min(rec.vertex(first + s), uint32_t(d.V - 1))], 1u);
+  __syncthreads();
+  // exclusive scan over the V counters: a thread owns a run of `per` consecutive ones
+  const int per = (d.V + kBucketThreads - 1) / kBucketThreads;
+  const int v0 = min(int(threadIdx.x) * per, d.V), v1 = min(v0 + per, d.V);
+  uint32_t mine = 0u;
+  for (int v = v0; v < v1; ++v) mine += count[v];
+  uint32_t scan = mine;  // inclusive over the wavefront
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  for (int off = 1; off < kWave; off <<= 1) {
+    const uint32_t o = __shfl_up(scan, off, kWave);
+    if (lane >= off) scan += o;
+  }
+  if (lane == kWave - 1) wave_total[wave] = scan;
+  __syncthreads();
+  uint32_t before = scan - mine;
+  for (int wv = 0; wv < wave; ++wv) before += wave_total[wv];
+  __syncthreads();
+  for (int v = v0; v < v1; ++v) {
+    const uint32_t n = count[v];
+    count[v] = before;
+    before += n;
+  }
+  __syncthreads();
+  for (long long s = threadIdx.x; s < d.S; s += kBucketThreads) {
+    const uint32_t at = atomicAdd(&count[min(rec.vertex(first + s), uint32_t(d.V - 1))], 1u);
+    perm[first + at] = uint32_t(s);
+  }
+}
+
+constexpr int kSegmentQuads = 4;  // float4 accumulators per lane: 1024 columns per pass over a block
+constexpr int kSegmentRows = 4;   // rows of xc requested together
+
+// One wavefront per (tree, block of 64 entries of the tree's vertex-ordered sample list): acc[n, :] += sum_i c_i *
+// xc[s_i, :] and m2sum[n] += sum_i c_i * zhat[s_i, n], n the feature the entries' vertex looks at. A lane first takes one
+// entry (sample index, c, vertex, feature, c * zhat); the block falls into runs of equal vertices (the list is ordered
+// by vertex), and run by run every entry's row of xc is read by the whole wavefront, lanes along the row, four rows in
+// flight, and summed in registers; a run ends in atomic adds on its feature's row of acc (a run is a piece of a
+// segment: vertices that many samples select spread over many wavefronts instead of one long serial loop).
+template <bool COMPACT>
+__global__ __launch_bounds__(256) void segment_sums_kernel(ForestDims d, Records<float, COMPACT> rec,
+                                                           const float *__restrict__ c,
+                                                           const uint32_t *__restrict__ perm,
+                                                           const float *__restrict__ xc, int K,
+                                                           const float *__restrict__ zhat, float *acc_out,
+                                                           double *m2sum) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const long long blocks_per_tree = (d.S + kWave - 1) / kWave;
+  const long long id = (long long)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+  if (id >= (long long)d.T * blocks_per_tree) return;
+  const int t = int(id / blocks_per_tree);
+  const long long i0 = (id - (long long)t * blocks_per_tree) * kWave;
+  const int count = int(min<long long>(kWave, d.S - i0));
+  const long long first = (long long)t * d.S;
+  uint32_t s_mine = 0u, v_mine = 0xffffffffu, n_mine = 0u;
+  float c_mine = 0.f;
+  double p_mine = 0.0;
+  if (lane < count) {
+    s_mine = perm[first + i0 + lane];
+    c_mine = c[first + s_mine];
+    v_mine = rec.vertex(first + s_mine);
+    n_mine = min(rec.ord(first + s_mine), uint32_t(d.F - 1));
+    p_mine = double(c_mine) * double(zhat[(long long)s_mine * d.F + n_mine]);
+  }
+  // runs of equal vertices: bit l of `starts` says that entry l begins one
+  const uint32_t v_before = uint32_t(__shfl_up(int(v_mine), 1, kWave));
+  const unsigned long long starts = __ballot(lane < count && (lane == 0 || v_mine != v_before));
+  const int quads = K / 4;
+  auto lane_value = [&](uint32_t mine, int j) { return uint32_t(__builtin_amdgcn_readlane(int(mine), j)); };
+  for (int q0 = 0; q0 < quads; q0 += kSegmentQuads * kWave) {
+    unsigned long long left = starts;
+    while (left) {
+      const int a = __builtin_ctzll(left);
+      left &= left - 1;
+      const int b = left ? __builtin_ctzll(left) : count;  // the run is entries a .. b - 1
+      const long long n = lane_value(n_mine, a);
+      Vec4 acc[kSegmentQuads];
+#pragma unroll
+      for (int q = 0; q < kSegmentQuads; ++q) acc[q] = Vec4{0.f, 0.f, 0.f, 0.f};
+      double m2 = 0.0;
+      for (int j0 = a; j0 < b; j0 += kSegmentRows) {
+        Vec4 xv[kSegmentRows][kSegmentQuads];
+        float cj[kSegmentRows];
+#pragma unroll
+        for (int r = 0; r < kSegmentRows; ++r) {
+          const int j = min(j0 + r, b - 1);  // (past the run's end: its last row again, weight 0)
+          const float *row = xc + (long long)lane_value(s_mine, j) * K;
+          cj[r] = j0 + r < b ? __uint_as_float(lane_value(__float_as_uint(c_mine), j)) : 0.f;
+#pragma unroll
+          for (int q = 0; q < kSegmentQuads; ++q) {
+            const int col = q0 + q * kWave + lane;
+            xv[r][q] = col < quads ? *reinterpret_cast<const Vec4 *>(row + 4 * col) : Vec4{0.f, 0.f, 0.f, 0.f};
+          }
+          if (q0 == 0 && j0 + r < b)
+            m2 += __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(p_mine), j),
+                                   __builtin_amdgcn_readlane(__double2loint(p_mine), j));
+        }
+#pragma unroll
+        for (int r = 0; r < kSegmentRows; ++r)
+#pragma unroll
+          for (int q = 0; q < kSegmentQuads; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[q][e] += cj[r] * xv[r][q][e];
+      }
+#pragma unroll
+      for (int q = 0; q < kSegmentQuads; ++q) {
+        const int col = q0 + q * kWave + lane;
+        if (col < quads) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (acc[q][e] != 0.f) atomicAdd(acc_out + n * K + 4 * col + e, acc[q][e]);
+        }
+      }
+      if (q0 == 0 && lane == 0 && m2 != 0.0) atomicAdd(m2sum + n, m2);
+    }
+  }
+}
+
+// dlin[n, k] = rstd[n] * (sparse[n, k] - (m2sum[n] / B) * rstd[n] * dense[n, k])
+__global__ __launch_bounds__(256) void combine_dlin_kernel(long long N, int K, double B, const float *__restrict__ sparse,
+                                                           const float *__restrict__ dense,
+                                                           const float *__restrict__ rstd,
+                                                           const double *__restrict__ m2sum, float *__restrict__ dlin) {
+  const long long quads = N * (K / 4);
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < quads; i += (long long)gridDim.x * 256) {
+    const long long n = i / (K / 4);
+    const float r = rstd[n], f = float(m2sum[n] / B) * r;
+    const Vec4 a = *reinterpret_cast<const Vec4 *>(sparse + 4 * i), b = *reinterpret_cast<const Vec4 *>(dense + 4 * i);
+    Vec4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = r * (a[e] - f * b[e]);
+    *reinterpret_cast<Vec4 *>(dlin + 4 * i) = o;
+  }
+}
+
+struct ProjectionForestLayout {
+  size_t forest, colsum, m2sum, xc, gram, partials, dense, sparse, perm, total;
+};
+
+ProjectionForestLayout projection_forest_layout(const ForestDims &d, long long K) {
+  ProjectionForestLayout l;
+  size_t at = 0;
+  auto take = [&](size_t bytes) {
+    const size_t here = at;
+    at += align_up(bytes, 256);
+    return here;
+  };
+  l.forest = take(forest_backward_records_workspace<float>(d, HT_BACKWARD_ATOMIC, false, true, true));
+  l.colsum = take(size_t(K) * sizeof(double));
+  l.m2sum = take(size_t(d.F) * sizeof(double));
+  l.xc = take(size_t(d.S) * K * sizeof(float));
+  l.gram = take(size_t(K) * K * sizeof(float));
+  const int shares = reduction_shares(K, K, d.S);
+  l.partials = take(shares > 1 ? size_t(shares) * K * K * sizeof(float) : 0);
+  l.dense = take(size_t(d.F) * K * sizeof(float));
+  l.sparse = take(size_t(d.F) * K * sizeof(float));
+  l.perm = take(size_t(d.T) * d.S * sizeof(uint32_t));
+  l.total = at;
+  return l;
+}
+
+template <bool COMPACT>
+int projection_forest_sparse(const ForestDims &d, long long K, const void *records, const float *c, const float *xc,
+                             const float *zhat, uint32_t *perm, float *sparse, double *m2sum,
+                             hipStream_t stream) {
+  // (the records are only read here; c comes from the forest pass)
+  const Records<float, COMPACT> rec = carve_records<float, COMPACT>(d, const_cast<void *>(records), nullptr);
+  auto bucket = bucket_kernel<COMPACT>;
+  hipLaunchKernelGGL(bucket, dim3((unsigned)d.T), dim3(kBucketThreads), size_t(d.V) * sizeof(uint32_t), stream, d, rec,
+                     perm);
+  HT_LAUNCH_CHECK("projection + forest backward (samples by vertex)");
+  const long long waves = (long long)d.T * ((d.S + kWave - 1) / kWave);
+  hipLaunchKernelGGL(segment_sums_kernel<COMPACT>, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, d, rec, c,
+                     perm, xc, int(K), zhat, sparse, m2sum);
+  HT_LAUNCH_CHECK("projection + forest backward (segment sums)");
+  return HT_OK;
+}
+
+}  // namespace
+
+// Whether projection_forest_backward serves a forest [B x N features, K = 1] behind a projection from K_in inputs.
+bool projection_forest_backward_ok(const ForestDims &d, long long K) {
+  if (is_empty(d) || d.K != 1 || K <= 0 || K % 4 != 0 || d.V > kMaxBucketVertices) return false;
+  if ((long long)d.T * d.V > 0x7fffffffLL * 4 || d.S > 0xffffffffLL) return false;
+  return forest_backward_keeps_c<float>(d);
+}
+
+size_t projection_forest_backward_workspace(const ForestDims &d, long long K) {
+  return projection_forest_backward_ok(d, K) ? projection_forest_layout(d, K).total : 0;
+}
+
+// dThr, dW of the forest and dLin of the projection in front of it, from the forest's walk records and upstream
+// gradient gout; no dense dL/dzhat is formed. x [B x K], lin [N x K], zhat [B x N], rstd [N] as projection_forward left
+// them; dthr / dw / dlin may be null.
+int projection_forest_backward(const ForestDims &d, bool fern, long long K, const float *x, const float *lin,
+                               const float *zhat, const float *rstd, const float *w, const float *gout,
+                               const void *records, float *dthr, float *dw, float *dlin, void *ws, size_t ws_bytes,
+                               hipStream_t stream) {
+  int rc;
+  if (!projection_forest_backward_ok(d, K))
+    return fail(HT_ERR_RUNTIME, "Error: this shape is not served by the records form of the projection backward.");
+  const ProjectionForestLayout l = projection_forest_layout(d, K);
+  if (ws == nullptr || ws_bytes < l.total)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the backward pass.");
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(lin) % 16 != 0 ||
+      (dlin && reinterpret_cast<uintptr_t>(dlin) % 16 != 0) || reinterpret_cast<uintptr_t>(ws) % 16 != 0)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: x, lin, dlin and the workspace must be 16-byte aligned.");
+  unsigned char *base = static_cast<unsigned char *>(ws);
+  const float *c = nullptr;
+  const size_t forest_bytes = l.colsum - l.forest;
+  if ((rc = forest_backward_records_keep_c<float>(d, fern, w, gout, records, dthr, dw, base + l.forest, forest_bytes,
+                                                  stream, &c)) != HT_OK)
+    return rc;
+  if (!dlin) return HT_OK;
+  const long long B = d.S, N = d.F;
+  double *colsum = reinterpret_cast<double *>(base + l.colsum), *m2sum = reinterpret_cast<double *>(base + l.m2sum);
+  float *xc = reinterpret_cast<float *>(base + l.xc), *gram = reinterpret_cast<float *>(base + l.gram);
+  float *partials = reinterpret_cast<float *>(base + l.partials), *dense = reinterpret_cast<float *>(base + l.dense);
+  float *sparse = reinterpret_cast<float *>(base + l.sparse);
+  uint32_t *perm = reinterpret_cast<uint32_t *>(base + l.perm);
+  // colsum and m2sum are neighbours: one clear
+  if ((rc = zero_fill(colsum, l.xc - l.colsum, stream)) != HT_OK) return rc;
+  if ((rc = zero_fill(sparse, size_t(N) * K * sizeof(float), stream)) != HT_OK) return rc;
+  // (x is small beside the matrices of the forward pass: shares of 16 rows or more, enough of them to fill the device)
+  const dim3 grid((unsigned)((K + 1023) / 1024), (unsigned)(B < 16 ? 1 : (B / 16 < 1024 ? B / 16 : 1024)));
+  const dim3 sums_grid((unsigned)((K / 4 + kWave - 1) / kWave), (unsigned)(B < 64 ? 1 : (B / 64 < 256 ? B / 64 : 256)));
+  hipLaunchKernelGGL(col_sums_kernel, sums_grid, dim3(256), 0, stream, x, B, int(K), colsum);
+  HT_LAUNCH_CHECK("projection + forest backward (column means)");
+  hipLaunchKernelGGL(center_kernel, grid, dim3(256), 0, stream, x, B, int(K), colsum, xc);
+  HT_LAUNCH_CHECK("projection + forest backward (centring)");
+  // Gc = xc^T xc (reduction over the batch, shares summed in a fixed order), dense = lin * Gc (Gc is symmetric: its
+  // rows serve as the columns the product wants, reduction index contiguous)
+  if ((rc = launch_gemm_batched<false, false, false, false>(xc, K, 0, xc, K, 0, gram, K, 0, K, K, B, 1, nullptr, nullptr,
+                                                            nullptr, stream, false, partials,
+                                                            reduction_shares(K, K, B))) != HT_OK)
+    return rc;
+  if ((rc = launch_gemm<true, true, false>(lin, K, gram, K, dense, K, N, K, K, nullptr, stream)) != HT_OK) return rc;
+  rc = compact_ok(d) ? projection_forest_sparse<true>(d, K, records, c, xc, zhat, perm, sparse, m2sum, stream)
+                     : projection_forest_sparse<false>(d, K, records, c, xc, zhat, perm, sparse, m2sum, stream);
+  if (rc != HT_OK) return rc;
+  const long long quads = N * (K / 4);
+  hipLaunchKernelGGL(combine_dlin_kernel, dim3((unsigned)((quads + 255) / 256 < 8192 ? (quads + 255) / 256 : 8192)),
+                     dim3(256), 0, stream, N, int(K), double(B), sparse, dense, rstd, m2sum, dlin);
+  HT_LAUNCH_CHECK("projection + forest backward (dLin)");
   return HT_OK;
 }
 

@@ -224,6 +224,55 @@ class LinearBatchNorm(torch.autograd.Function):
         return dx, dlin, None
 
 
+class LinearBatchNormForest(torch.autograd.Function):
+    """Linear(bias=False) -> BatchNorm1d(affine=False, training) -> HingeTree / HingeFern as one operator: the whole
+    README model (README.md:117-129). forward(ctx, inData, inLinearWeights, eps, inThresholds, inOrdinals, inWeights,
+    fern) returns (out, mean, var). Forward values are those of LinearBatchNorm followed by the forest function; what
+    the fusion buys is the backward pass: when inData wants no gradient (a first layer), the gradient of the linear
+    weights comes straight from the forest's walk records -- the forest's input gradient has one non-zero per sample
+    and tree, so its dense [batch, features] form, the batch-norm backward over it and the dense product with the inputs
+    are all skipped (tree_linear_bn_backward_records). Deterministic mode, inputs that want gradients and shapes the
+    library does not serve that way take the two separate backward passes."""
+
+    @staticmethod
+    def forward(ctx, inData, inLinearWeights, eps, inThresholds, inOrdinals, inWeights, fern):
+        pre = "fern" if fern else "tree"
+        zhat, mean, rstd, var = _ops.linear_bn_forward(inData, inLinearWeights, eps)
+        records = None
+        if any(ctx.needs_input_grad):
+            out, records = getattr(_ops, pre + "_forward_records")(zhat, inThresholds, inOrdinals, inWeights)
+        else:
+            out = getattr(_ops, pre + "_forward")(zhat, inThresholds, inOrdinals, inWeights)
+        ctx.pre = pre
+        ctx.has_records = records is not None
+        saved = [inData, inLinearWeights, zhat, rstd, inThresholds, inOrdinals, inWeights]
+        ctx.save_for_backward(*(saved + ([records] if records is not None else [])))
+        ctx.mark_non_differentiable(mean, var)
+        return out, mean, var
+
+    @staticmethod
+    def backward(ctx, outDataGrad, _mean_grad, _var_grad):
+        inData, inLinearWeights, zhat, rstd, inThresholds, inOrdinals, inWeights = ctx.saved_tensors[:7]
+        need_x, need_lin, _, need_thr, need_ord, need_w, _ = ctx.needs_input_grad
+        up = outDataGrad.contiguous()
+        deterministic = _is_deterministic()
+        if ctx.has_records and not need_x and not deterministic:
+            got = getattr(_ops, ctx.pre + "_linear_bn_backward_records")(
+                ctx.saved_tensors[7], inData, inLinearWeights, need_lin, zhat, rstd, inThresholds, need_thr, inOrdinals,
+                inWeights, need_w, up)
+            if got is not None:
+                return None, got[0], None, got[1], None, got[2], None
+        args = (zhat, need_x or need_lin, inThresholds, need_thr, inOrdinals, need_ord, inWeights, need_w, up)
+        if ctx.has_records:
+            dz, dthr, _, dw = getattr(_ops, ctx.pre + "_backward_records")(ctx.saved_tensors[7], deterministic, *args)
+        else:
+            dz, dthr, _, dw = getattr(_ops, ctx.pre + ("_backward_deterministic" if deterministic else "_backward"))(*args)
+        dx = dlin = None
+        if dz is not None:
+            dx, dlin = _ops.linear_bn_backward(inData, need_x, inLinearWeights, need_lin, zhat, rstd, dz)
+        return dx, dlin, None, dthr, None, dw, None
+
+
 def contract(inData, window, padding=0):
     """HingeTree/_HingeTree.py:32-39."""
     if isinstance(window, int):

@@ -412,6 +412,63 @@ def linear_bn_backward(inData, bInDataGrad, inLinearWeights, bInLinearWeightsGra
     return [dx, dlin]
 
 
+def _linear_bn_backward_records(kind, records, inData, inLinearWeights, bInLinearWeightsGrad, zhat, rstd, inThresholds,
+                                bInThresholdsGrad, inOrdinals, inWeights, bInWeightsGrad, outDataGrad):
+    """Backward of the whole front linear_bn_forward -> *_forward_records(zhat, ...) for an upstream gradient on the
+    forest's output, when no gradient of inData is wanted: [dLinearWeights | None, dThresholds | None, dWeights | None]
+    from the forest's walk records, without forming the dense gradient on zhat (it has one non-zero per sample and
+    tree). Returns None where the library does not serve the shape this way (the caller then runs *_backward_records
+    and linear_bn_backward)."""
+    if not isinstance(records, torch.Tensor) or records.dtype != torch.uint8 or not records.is_contiguous():
+        _invalid("Error: records must be the contiguous uint8 tensor a *_forward_records call returned.")
+    for t in (inData, inLinearWeights, zhat, rstd, inThresholds, inWeights, outDataGrad):
+        if t.dtype != torch.float32:
+            _invalid("Error: the projection supports torch.float32 only.")
+    for t in (inData, inLinearWeights, zhat, rstd, records):
+        if not t.is_contiguous():
+            _invalid("Error: All tensors are expected to be contiguous.")
+        if t.device != inData.device:
+            _invalid("Error: All tensors are expected to be on the same device.")
+    if not inData.is_cuda:
+        _runtime("Error: this build has no CPU back-end; tensors must be on a GPU.")
+    _common_checks([zhat, inThresholds, inWeights, outDataGrad], inOrdinals, True)
+    if inData.dim() != 2 or inLinearWeights.dim() != 2 or zhat.dim() != 2:
+        _invalid("Error: inData must be [batch, in_features], inLinearWeights [out_features, in_features], zhat "
+                 "[batch, out_features].")
+    B, K = inData.shape
+    N = inLinearWeights.shape[0]
+    if inLinearWeights.shape[1] != K or zhat.shape != (B, N) or rstd.shape != (N,):
+        _invalid("Error: shapes of zhat / rstd do not match the projection.")
+    shape, _ = _forest_shape(kind, zhat, inThresholds, inOrdinals, inWeights, outDataGrad)
+    lib = L.load()
+    if records.numel() != lib.ht_forest_records_bytes(ctypes.byref(shape)):
+        _invalid("Error: records do not belong to a forest of this shape.")
+    nbytes = lib.ht_projection_forest_backward_workspace(ctypes.byref(shape), K)
+    if nbytes == 0:
+        return None
+    with torch.cuda.device(inData.device):
+        dlin = torch.empty_like(inLinearWeights) if bInLinearWeightsGrad else None
+        dthr = torch.empty_like(inThresholds) if bInThresholdsGrad else None
+        dw = torch.empty_like(inWeights) if bInWeightsGrad else None
+        ws = _workspace(nbytes, inData.device)
+        L.check(lib.ht_projection_forest_backward(ctypes.byref(shape), K, _ptr(inData), _ptr(inLinearWeights), _ptr(zhat),
+                                                  _ptr(rstd), _ptr(inWeights), _ptr(outDataGrad), _ptr(records),
+                                                  records.numel(), _ptr(dthr), _ptr(dw), _ptr(dlin), _ptr(ws), nbytes,
+                                                  _stream(inData.device)))
+    return [dlin, dthr, dw]
+
+
+def tree_linear_bn_backward_records(*args):
+    return _linear_bn_backward_records(L.HT_TREE, *args)
+
+
+def fern_linear_bn_backward_records(*args):
+    return _linear_bn_backward_records(L.HT_FERN, *args)
+
+
+tree_linear_bn_backward_records.__doc__ = fern_linear_bn_backward_records.__doc__ = _linear_bn_backward_records.__doc__
+
+
 # ---- forest / fern ------------------------------------------------------------------------------------------------
 def _common_checks(tensors, ordinals, with_grad):
     data = tensors[0]

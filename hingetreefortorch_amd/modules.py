@@ -281,7 +281,9 @@ class LinearHingeForest(nn.Module):
     def forward(self, x):
         if not self.training or not x.is_cuda or x.dtype != torch.float32:
             return self.forest(self.bn(self.fc(x)))
-        zhat, mean, var = _fn.LinearBatchNorm.apply(x.contiguous(), self.fc.weight, self.bn.eps)
+        out, mean, var = _fn.LinearBatchNormForest.apply(x.contiguous(), self.fc.weight, self.bn.eps,
+                                                         self.forest.thresholds, self.forest.ordinals,
+                                                         self.forest.weights, False)
         if self.bn.track_running_stats:
             with torch.no_grad():
                 n = x.shape[0]
@@ -289,4 +291,4 @@ class LinearHingeForest(nn.Module):
                 m = self.bn.momentum if self.bn.momentum is not None else 1.0 / float(self.bn.num_batches_tracked)
                 self.bn.running_mean.mul_(1 - m).add_(mean, alpha=m)
                 self.bn.running_var.mul_(1 - m).add_(var * (n / max(n - 1, 1)), alpha=m)
-        return self.forest(zhat)
+        return out

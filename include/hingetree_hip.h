@@ -189,6 +189,27 @@ int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, cons
                            const float *rstd, float *g, float *dlin, float *dx, void *workspace,
                            size_t workspace_bytes, void *stream);
 
+/* The backward pass of the whole front -- Linear(bias = False) -> BatchNorm1d(affine = False) -> forest in training
+ * mode -- from the walk records of ht_forest_forward_records run on zhat: dthr [T, V], dw [T, L, M] of the forest and
+ * dlin [N, K_in] of the projection (each may be NULL), for a caller that wants no gradient of the projection's input.
+ * No counterpart in the reference, whose composition multiplies a dense dL/dzhat [B, N] by the inputs; here that
+ * matrix is never formed: it holds one non-zero per (sample, tree), so
+ *   dlin[n, :] = rstd[n] * (sum over the pairs that selected feature n of c * xc[sample, :]
+ *                           - mean_b(g * zhat)[n] * rstd[n] * (lin * xc^T xc)[n, :]),   xc = x - mean_b x,
+ * with c the forest's input gradient at the selected vertex: a sparse sum over the records plus two small dense
+ * products, which agrees with the dense form to rounding (sums reordered, nothing cancelled).
+ *   forest: the forest's shape with B = batch, F = N (the projected features), K = 1, dtype HT_F32; x [B, K_in],
+ *   lin [N, K_in], zhat [B, N], rstd [N] as ht_projection_forward took / left them; w, gout, records as for
+ *   ht_forest_backward_records. Atomic accumulation (the order of additions, hence the last bits, can differ between
+ *   runs). ht_projection_forest_backward_workspace returns 0 where the shape is not served (K_in not a multiple of 4,
+ *   K > 1, more than 16384 vertices per tree, shapes whose records the staged kernels do not take): call
+ *   ht_forest_backward_records + ht_projection_backward there. */
+size_t ht_projection_forest_backward_workspace(const ht_forest_shape *forest, int64_t K_in);
+int ht_projection_forest_backward(const ht_forest_shape *forest, int64_t K_in, const float *x, const float *lin,
+                                  const float *zhat, const float *rstd, const float *w, const float *gout,
+                                  const void *records, size_t records_bytes, float *dthr, float *dw, float *dlin,
+                                  void *workspace, size_t workspace_bytes, void *stream);
+
 /* Diagnostic, host only, no counterpart in the reference: the matrix-product kernel's launch-slot -> result-tile map
  * for a grid of tiles_i x tiles_j result tiles (slots are dealt to the 8 L2 domains round robin; each domain walks a
  * band of tile rows in panels of 8 tile columns). tile_i / tile_j receive one entry per launch slot, (-1, -1) for a

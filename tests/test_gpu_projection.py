@@ -130,3 +130,67 @@ def test_linear_hinge_forest_matches_composition(dev):
     assert rel_err(model.fc.weight.grad.double().cpu(), dz.t() @ x.double().cpu()) <= 5e-5
     model.eval()
     assert model(x).shape == out.shape
+
+
+RECORD_CASES = [
+    # B, K_in, N features, trees, depth, outputs per leaf, fern, private features (the README model's sequential ordinals)
+    (200, 36, 42, 6, 3, 4, False, True),
+    (333, 40, 50, 9, 4, 1, False, False),     # features shared by vertices of several trees
+    (96, 8, 30, 5, 5, 3, True, False),        # ferns: a vertex is a level
+    (1000, 100, 310, 10, 5, 10, False, True),
+    (77, 4, 7, 3, 2, 2, False, False),
+]
+
+
+@pytest.mark.parametrize("case", RECORD_CASES, ids=[f"c{i}" for i in range(len(RECORD_CASES))])
+def test_front_backward_from_records(dev, case):
+    """tree_linear_bn_backward_records (dLin from the forest's walk records: sparse segment sums + two small products)
+    against the dense route -- forest backward to a dense dL/dzhat, batch-norm backward, dz^T x -- and against the fp64
+    closed form of that route; dThr and dW are the forest's own."""
+    B, K, N, T, depth, M, fern, private = case
+    g = torch.Generator().manual_seed(31)
+    V = depth if fern else 2 ** depth - 1
+    x = torch.rand([B, K], generator=g)
+    lin = torch.randn([N, K], generator=g) / K ** 0.5
+    thr = 3.0 * torch.rand([T, V], generator=g) - 1.5
+    ordn = (torch.arange(T * V).reshape(T, V) % N) if private else torch.randint(0, N, (T, V), generator=g)
+    w = torch.randn([T, 2 ** depth, M], generator=g)
+    up = torch.randn([B, T, M], generator=g)
+    pre = "fern" if fern else "tree"
+    dx_, dlin_, dthr_, dw_ = None, None, None, None
+    gx, glin, gthr, gord, gw, gup = (t.to(dev) for t in (x, lin, thr, ordn, w, up))
+    zhat, mean, rstd, var = ops.linear_bn_forward(gx, glin, 1e-5)
+    out, rec = getattr(ops, pre + "_forward_records")(zhat, gthr, gord, gw)
+    dz, dthr_, _, dw_ = getattr(ops, pre + "_backward_records")(rec, True, zhat, True, gthr, True, gord, False, gw, True, gup)
+    gz = dz.clone()
+    _, dlin_ = ops.linear_bn_backward(gx, False, glin, True, zhat, rstd, dz)
+    got = getattr(ops, pre + "_linear_bn_backward_records")(rec, gx, glin, True, zhat, rstd, gthr, True, gord, gw, True, gup)
+    assert got is not None, "shape not served by the records form"
+    dlin, dthr, dw = got
+    # closed form in fp64 from the dense dL/dzhat
+    gd, rz, r64 = gz.double().cpu(), zhat.double().cpu(), rstd.double().cpu()
+    want = (r64 * (gd - gd.mean(0) - rz * (gd * rz).mean(0))).t() @ x.double()
+    scale = max(float(r64.abs().max()), 1.0)
+    assert rel_err(dlin.cpu().double(), want) <= 2e-5 * scale
+    assert rel_err(dlin_.cpu().double(), want) <= 2e-5 * scale
+    assert rel_err(dthr.cpu(), dthr_.cpu()) <= 1e-5 and rel_err(dw.cpu(), dw_.cpu()) <= 1e-5
+    # single gradients
+    only = getattr(ops, pre + "_linear_bn_backward_records")(rec, gx, glin, True, zhat, rstd, gthr, False, gord, gw, False, gup)
+    assert only[1] is None and only[2] is None and rel_err(only[0].cpu().double(), want) <= 2e-5 * scale
+    only = getattr(ops, pre + "_linear_bn_backward_records")(rec, gx, glin, False, zhat, rstd, gthr, True, gord, gw, True, gup)
+    assert only[0] is None and rel_err(only[1].cpu(), dthr_.cpu()) <= 1e-5 and rel_err(only[2].cpu(), dw_.cpu()) <= 1e-5
+
+
+def test_front_backward_from_records_rejects(dev):
+    g = torch.Generator().manual_seed(3)
+    B, K, N, T, depth, M = 64, 6, 14, 2, 3, 2    # 6 inputs: not a multiple of 4 -> not served, the caller falls back
+    x, lin = torch.rand([B, K], generator=g).to(dev), torch.randn([N, K], generator=g).to(dev)
+    thr, ordn = torch.rand([T, 7], generator=g).to(dev), torch.randint(0, N, (T, 7), generator=g).to(dev)
+    w, up = torch.randn([T, 8, M], generator=g).to(dev), torch.randn([B, T, M], generator=g).to(dev)
+    zhat, mean, rstd, var = ops.linear_bn_forward(x, lin, 1e-5)
+    out, rec = ops.tree_forward_records(zhat, thr, ordn, w)
+    assert ops.tree_linear_bn_backward_records(rec, x, lin, True, zhat, rstd, thr, True, ordn, w, True, up) is None
+    with pytest.raises(ValueError):
+        ops.tree_linear_bn_backward_records(rec[:-1].contiguous(), x, lin, True, zhat, rstd, thr, True, ordn, w, True, up)
+    with pytest.raises(ValueError):
+        ops.tree_linear_bn_backward_records(rec, x.double(), lin, True, zhat, rstd, thr, True, ordn, w, True, up)
