@@ -14,7 +14,7 @@ HT_F32, HT_F64 = 0, 1
 HT_TREE, HT_FERN = 0, 1
 HT_BACKWARD_ATOMIC, HT_BACKWARD_DETERMINISTIC = 0, 1
 HT_MAX_CONV_DIMS = 3
-HT_ABI_VERSION = 2  # of include/hingetree_hip.h as this file mirrors it; load() refuses a library built from another
+HT_ABI_VERSION = 3  # of include/hingetree_hip.h as this file mirrors it; load() refuses a library built from another
 
 
 class ForestShape(ctypes.Structure):

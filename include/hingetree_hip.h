@@ -62,7 +62,7 @@ const char *ht_last_error(void);
  * (what a workspace or records size covers, what a later call expects an earlier one to have written there).
  * ht_abi_version() returns the value the library was built with; a host compiled against this header compares it with
  * HT_ABI_VERSION and refuses a library built from another one. */
-#define HT_ABI_VERSION 2
+#define HT_ABI_VERSION 3
 int ht_abi_version(void);
 /* HT_OK if GPU `device` can run this library's code object (gfx950), else an error that names what it is. The tile
  * sizes assume that part's 160 KB of LDS per workgroup, 256 compute units and 8 L2 domains; hosts call this once per
