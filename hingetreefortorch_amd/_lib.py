@@ -82,8 +82,11 @@ SIGNATURES = {
     "ht_projection_backward": (_I, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _P, _P, _P, _P, _P, _P, _P, _P,
                                     _SZ, _P]),
     "ht_projection_forest_backward_workspace": (_SZ, [_P, ctypes.c_int64]),
-    "ht_projection_forest_backward": (_I, [_P, ctypes.c_int64, _P, _P, _P, _P, _P, _P, _P, _SZ, _P, _P, _P, _P, _SZ,
-                                           _P]),
+    "ht_projection_forest_backward": (_I, [_P, ctypes.c_int64, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P, _P, _P, _P,
+                                           _SZ, _P]),
+    "ht_projection_forest_forward_workspace": (_SZ, [_P]),
+    "ht_projection_forest_forward": (_I, [_P, ctypes.c_int64, _P, _P, ctypes.c_double, _P, _P, _P, _P, _P, _P, _P, _P,
+                                          _P, _SZ, _P, _SZ, _P]),
     "ht_gemm_tile_map": (_I, [ctypes.c_int32, ctypes.c_int32, _P, _P, ctypes.c_int64]),
     "ht_check_thresholds": (_I, [_P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),
     "ht_fix_thresholds": (_I, [_P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),

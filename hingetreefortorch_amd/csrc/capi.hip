@@ -576,8 +576,38 @@ size_t ht_projection_forest_backward_workspace(const ht_forest_shape *forest, in
   return projection_forest_backward_workspace(d, K_in);
 }
 
+size_t ht_projection_forest_forward_workspace(const ht_forest_shape *forest) {
+  ForestDims d;
+  if (!forest || forest->dtype != HT_F32 || forest->K != 1 || make_dims(forest, &d) != HT_OK) return 0;
+  return projection_forest_forward_workspace(d);
+}
+
+int ht_projection_forest_forward(const ht_forest_shape *forest, int64_t K_in, const float *x, const float *lin, double eps,
+                                 const float *thr, const int64_t *ord, const float *w, float *out, float *z, float *mean,
+                                 float *rstd, float *var, void *records, size_t records_bytes, void *workspace,
+                                 size_t workspace_bytes, void *stream) {
+  ForestDims d;
+  if (!forest) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  int rc = make_dims(forest, &d);
+  if (rc != HT_OK) return rc;
+  if (forest->dtype != HT_F32) return fail(HT_ERR_INVALID_ARGUMENT, "Error: the projection supports float32 only.");
+  if (forest->K != 1 || K_in < 0)
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: the projection's forest has no inner data dimensions.");
+  if (d.F > 0 && (!mean || !rstd || !workspace)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (d.S > 0 && d.F > 0 && (!z || (K_in > 0 && (!x || !lin)))) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (!is_empty(d) && (!thr || !ord || !w || !out)) return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
+  if (records) {
+    const size_t need = ht_forest_records_bytes(forest);
+    if (need == 0 && !is_empty(d))
+      return fail(HT_ERR_INVALID_ARGUMENT, "Error: walk records are not offered for this shape.");
+    if (records_bytes < need) return fail(HT_ERR_INVALID_ARGUMENT, "Error: records buffer too small.");
+  }
+  return projection_forest_forward(d, forest->kind == HT_FERN, K_in, x, lin, eps, thr, ord, w, out, z, mean, rstd, var,
+                                   records, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 int ht_projection_forest_backward(const ht_forest_shape *forest, int64_t K_in, const float *x, const float *lin,
-                                  const float *zhat, const float *rstd, const float *w, const float *gout,
+                                  const float *zhat, const float *mean, const float *rstd, const float *w, const float *gout,
                                   const void *records, size_t records_bytes, float *dthr, float *dw, float *dlin,
                                   void *workspace, size_t workspace_bytes, void *stream) {
   ForestDims d;
@@ -593,7 +623,7 @@ int ht_projection_forest_backward(const ht_forest_shape *forest, int64_t K_in, c
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: null pointer.");
   if (records_bytes < ht_forest_records_bytes(forest))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: records buffer too small.");
-  return projection_forest_backward(d, forest->kind == HT_FERN, K_in, x, lin, zhat, rstd, w, gout, records, dthr, dw,
+  return projection_forest_backward(d, forest->kind == HT_FERN, K_in, x, lin, zhat, mean, rstd, w, gout, records, dthr, dw,
                                     dlin, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 

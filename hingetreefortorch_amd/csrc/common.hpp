@@ -101,14 +101,22 @@ template <typename Real>
 int pack_nodes(const ForestDims &d, const Real *thr, const int64_t *ord, void *dst, hipStream_t stream,
                unsigned long long *zero_slots = nullptr);
 
+// Optional normalisation of the features on their way into the forward pass: feature f of every sample is read as
+// (x - mean[f]) * rstd[f] (two rounded operations, like a separate elementwise pass would do them). Null: x as it is.
+template <typename Real>
+struct FeatureNorm {
+  const Real *mean = nullptr, *rstd = nullptr;
+};
+
 template <typename Real>
 size_t forest_forward_workspace(const ForestDims &d);
 // `records` (optional): forest_records_bytes() bytes that receive the walk records for forest_backward_records().
 // `image` (optional): store the result as that image instead of [B, T, K, M]; needs K > 1.
+// `norm` (optional): the features are normalised as they are read (FeatureNorm).
 template <typename Real>
 int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
                    Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream,
-                   const ImageStore *image = nullptr);
+                   const ImageStore *image = nullptr, const FeatureNorm<Real> *norm = nullptr);
 
 template <typename Real>
 size_t forest_backward_workspace(const ForestDims &d, int mode, bool need_dx, bool need_dthr, bool need_dw);
@@ -188,10 +196,16 @@ int projection_backward(long long B, long long K, long long N, const float *x, c
                         const float *rstd, float *g, float *dlin, float *dx, void *ws, hipStream_t stream);
 // The same gradients for the whole Linear -> BatchNorm -> forest front from the forest's walk records: dThr, dW and
 // dLin without a dense dL/dzhat (d: the forest over the N = d.F projected features of B = d.S samples, K_in inputs).
+// (mean given: `zhat` is the un-normalised product z of projection_forest_forward)
 bool projection_forest_backward_ok(const ForestDims &d, long long K_in);
+// The forward pass of the front with the forest reading the un-normalised product z through FeatureNorm.
+size_t projection_forest_forward_workspace(const ForestDims &d);
+int projection_forest_forward(const ForestDims &d, bool fern, long long K_in, const float *x, const float *lin, double eps,
+                              const float *thr, const int64_t *ord, const float *w, float *out, float *z, float *mean,
+                              float *rstd, float *var, void *records, void *ws, size_t ws_bytes, hipStream_t stream);
 size_t projection_forest_backward_workspace(const ForestDims &d, long long K_in);
 int projection_forest_backward(const ForestDims &d, bool fern, long long K_in, const float *x, const float *lin,
-                               const float *zhat, const float *rstd, const float *w, const float *gout,
+                               const float *zhat, const float *mean, const float *rstd, const float *w, const float *gout,
                                const void *records, float *dthr, float *dw, float *dlin, void *ws, size_t ws_bytes,
                                hipStream_t stream);
 // Host-side view of the matrix-product kernel's workgroup -> result-tile map for tiles_i x tiles_j tiles: writes the

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
                                                      const Node<Real> *__restrict__ nodes,
                                                      const Real *__restrict__ w, Real *__restrict__ out,
                                                      Records<Real, COMPACT> rec, int trees_per_block,
-                                                     FastDiv div_m, ImageStore img) {
+                                                     FastDiv div_m, ImageStore img, FeatureNorm<Real> norm) {
   typedef Real Vec __attribute__((ext_vector_type(VW)));
   constexpr int TC = NT / BT;        // tree slots per walk round
   constexpr int kIlp = ILP;
@@ -60,13 +60,14 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
 
   const long long s0 = (long long)blockIdx.x * BT;
   if (XLDS) {
-    load_tile<Real, BT, NT>(xs, x, d, s0);
+    load_tile<Real, BT, NT>(xs, x, d, s0, norm);
     __syncthreads();
   }
   const int j = threadIdx.x % BT, tt = threadIdx.x / BT;
   const long long s = s0 + j;
   const bool live = s < d.S;
   const long long xbase = live ? (s / d.K) * d.FK + (s % d.K) : 0;
+  const bool normalise = norm.mean != nullptr;
 
   const int t_begin = blockIdx.y * trees_per_block;
   const int t_end = min(d.T, t_begin + trees_per_block);
@@ -83,7 +84,13 @@ __global__ __launch_bounds__(NT) void forward_kernel(ForestDims d, const Real *_
       if (XLDS)
         walk_many<Real, FERN, kIlp>(d.depth, nd, [&](int, int f) { return xs[f * BT + j]; }, r);
       else
-        walk_many<Real, FERN, kIlp>(d.depth, nd, [&](int, int f) { return x[xbase + (long long)f * d.K]; }, r);
+        walk_many<Real, FERN, kIlp>(
+            d.depth, nd,
+            [&](int, int f) {
+              const Real v = x[xbase + (long long)f * d.K];
+              return normalise ? (v - norm.mean[f]) * norm.rstd[f] : v;
+            },
+            r);
 #pragma unroll
       for (int i = 0; i < kIlp; ++i) {
         r_abs[j * LDR + tt + i * TC] = ht_abs(r[i].margin);
@@ -948,11 +955,11 @@ int dispatch_rows(const ForestDims &d, const Real *x, const void *vertices, cons
 
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
 int launch_forward_rec(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                       void *records, hipStream_t stream, const ImageStore &img);
+                       void *records, hipStream_t stream, const ImageStore &img, const FeatureNorm<Real> &norm);
 
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW, bool RECORD, bool COMPACT>
 int launch_forward_vw(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                      void *records, hipStream_t stream, const ImageStore &img) {
+                      void *records, hipStream_t stream, const ImageStore &img, const FeatureNorm<Real> &norm) {
   constexpr int NT = kForestThreads;
   constexpr int TP = NT / BT * ILP;
   const size_t lds = (XLDS ? size_t(d.F) * BT * sizeof(Real) : 0) + size_t(TP + 1) * BT * (sizeof(Real) + sizeof(KeyT));
@@ -965,26 +972,27 @@ int launch_forward_vw(const ForestDims &d, const Real *x, const Node<Real> *node
   if (RECORD) rec = carve_records<Real, COMPACT>(d, records, nullptr);
   HT_HIP_CHECK(grant_lds(reinterpret_cast<const void *>(kernel)));
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)gy), dim3(NT), lds, stream, d, x, nodes, w, out, rec,
-                     trees_per_block, FastDiv(d.M), img);
+                     trees_per_block, FastDiv(d.M), img, norm);
   HT_LAUNCH_CHECK("forest forward");
   return HT_OK;
 }
 
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT, int VW>
 int launch_forward_rec(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                       void *records, hipStream_t stream, const ImageStore &img) {
+                       void *records, hipStream_t stream, const ImageStore &img, const FeatureNorm<Real> &norm) {
   if (!records)
     return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, false, true>(d, x, nodes, w, out, records, stream,
-                                                                               img);
+                                                                               img, norm);
   if (compact_ok(d))
     return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, true, true>(d, x, nodes, w, out, records, stream,
-                                                                              img);
-  return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, true, false>(d, x, nodes, w, out, records, stream, img);
+                                                                              img, norm);
+  return launch_forward_vw<Real, FERN, BT, XLDS, ILP, KeyT, VW, true, false>(d, x, nodes, w, out, records, stream, img,
+                                                                             norm);
 }
 
 template <typename Real, bool FERN, int BT, bool XLDS, int ILP, typename KeyT>
 int launch_forward_as(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                      void *records, hipStream_t stream, const ImageStore &img) {
+                      void *records, hipStream_t stream, const ImageStore &img, const FeatureNorm<Real> &norm) {
   // widest output vector that M and the pointers allow (inner dimensions shorter than the tile keep scalar outputs);
   // into an image, a vector must also stay inside one window row and keep the image rows aligned
   const uintptr_t pw = reinterpret_cast<uintptr_t>(w), po = reinterpret_cast<uintptr_t>(out);
@@ -993,24 +1001,26 @@ int launch_forward_as(const ForestDims &d, const Real *x, const Node<Real> *node
     if (!runs || d.M % vw != 0 || pw % (vw * sizeof(Real)) != 0 || po % (vw * sizeof(Real)) != 0) return false;
     return img.nd == 0 || (img.win[2] % vw == 0 && img.pad[2] % vw == 0 && img.size[2] % vw == 0);
   };
-  if (fits(4)) return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 4>(d, x, nodes, w, out, records, stream, img);
-  if (fits(2)) return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 2>(d, x, nodes, w, out, records, stream, img);
-  return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 1>(d, x, nodes, w, out, records, stream, img);
+  if (fits(4))
+    return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 4>(d, x, nodes, w, out, records, stream, img, norm);
+  if (fits(2))
+    return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 2>(d, x, nodes, w, out, records, stream, img, norm);
+  return launch_forward_rec<Real, FERN, BT, XLDS, ILP, KeyT, 1>(d, x, nodes, w, out, records, stream, img, norm);
 }
 
 // Four trees per thread with 16-bit parked keys where the depth allows it, else two trees with 32-bit keys: both keep
 // the per-pass results of a 1024-thread workgroup under the LDS left beside a 128 KB sample tile.
 template <typename Real, bool FERN, int BT, bool XLDS>
 int launch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                   void *records, hipStream_t stream, const ImageStore &img) {
+                   void *records, hipStream_t stream, const ImageStore &img, const FeatureNorm<Real> &norm) {
   if (d.depth <= 16)
-    return launch_forward_as<Real, FERN, BT, XLDS, 4, uint16_t>(d, x, nodes, w, out, records, stream, img);
-  return launch_forward_as<Real, FERN, BT, XLDS, 2, uint32_t>(d, x, nodes, w, out, records, stream, img);
+    return launch_forward_as<Real, FERN, BT, XLDS, 4, uint16_t>(d, x, nodes, w, out, records, stream, img, norm);
+  return launch_forward_as<Real, FERN, BT, XLDS, 2, uint32_t>(d, x, nodes, w, out, records, stream, img, norm);
 }
 
 template <typename Real, bool FERN>
 int dispatch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes, const Real *w, Real *out,
-                     void *records, hipStream_t stream, const ImageStore &img) {
+                     void *records, hipStream_t stream, const ImageStore &img, const FeatureNorm<Real> &norm) {
   // room for the per-pass results: (4 trees x 1024 threads + one pad column) x (|margin| + key)
   const size_t reserve = size_t(4) * kForestThreads * (sizeof(Real) + sizeof(uint32_t));
   int bt = pick_tile<Real>(d.F, reserve);
@@ -1018,11 +1028,11 @@ int dispatch_forward(const ForestDims &d, const Real *x, const Node<Real> *nodes
   // pass (longer contiguous row segments per store burst, half the barriers) and one row per wavefront.
   if (d.M >= 8 && bt >= 32) bt /= 2;
   switch (bt) {
-    case 64: return launch_forward<Real, FERN, 64, true>(d, x, nodes, w, out, records, stream, img);
-    case 32: return launch_forward<Real, FERN, 32, true>(d, x, nodes, w, out, records, stream, img);
-    case 16: return launch_forward<Real, FERN, 16, true>(d, x, nodes, w, out, records, stream, img);
-    case 8: return launch_forward<Real, FERN, 8, true>(d, x, nodes, w, out, records, stream, img);
-    default: return launch_forward<Real, FERN, 64, false>(d, x, nodes, w, out, records, stream, img);
+    case 64: return launch_forward<Real, FERN, 64, true>(d, x, nodes, w, out, records, stream, img, norm);
+    case 32: return launch_forward<Real, FERN, 32, true>(d, x, nodes, w, out, records, stream, img, norm);
+    case 16: return launch_forward<Real, FERN, 16, true>(d, x, nodes, w, out, records, stream, img, norm);
+    case 8: return launch_forward<Real, FERN, 8, true>(d, x, nodes, w, out, records, stream, img, norm);
+    default: return launch_forward<Real, FERN, 64, false>(d, x, nodes, w, out, records, stream, img, norm);
   }
 }
 
@@ -1121,8 +1131,11 @@ __global__ __launch_bounds__(256) void pad_rows_pairs_kernel(const Real *__restr
 
 template <typename Real>
 int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *thr, const int64_t *ord, const Real *w,
-                   Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream, const ImageStore *image) {
+                   Real *out, void *records, void *ws, size_t ws_bytes, hipStream_t stream, const ImageStore *image,
+                   const FeatureNorm<Real> *norm_in) {
   if (is_empty(d)) return HT_OK;
+  FeatureNorm<Real> norm;
+  if (norm_in) norm = *norm_in;
   if (ws == nullptr || ws_bytes < forest_forward_workspace<Real>(d))
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the forward pass.");
   ImageStore img{};
@@ -1131,7 +1144,8 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
   unsigned long long *slots = records ? records_bound_slots<Real>(d, records) : nullptr;
   if (img.nd && d.K == 1)
     return fail(HT_ERR_INVALID_ARGUMENT, "Error: an image result needs inner data positions (inData of 3 or more dimensions).");
-  if (rows_ok<Real>(d)) {
+  // (the row kernels read the features as they lie in memory: a normalising call takes the tile kernels below)
+  if (rows_ok<Real>(d) && norm.mean == nullptr) {
     int wpitch = weight_pitch<Real>(d);
     const bool shifted =
         odd_pairs_ok<Real>(d, wpitch, out) &&
@@ -1173,8 +1187,8 @@ int forest_forward(const ForestDims &d, bool fern, const Real *x, const Real *th
   int rc = pack_nodes<Real>(d, thr, ord, ws, stream, slots);
   if (rc != HT_OK) return rc;
   const Node<Real> *nodes = static_cast<const Node<Real> *>(ws);
-  return fern ? dispatch_forward<Real, true>(d, x, nodes, w, out, records, stream, img)
-              : dispatch_forward<Real, false>(d, x, nodes, w, out, records, stream, img);
+  return fern ? dispatch_forward<Real, true>(d, x, nodes, w, out, records, stream, img, norm)
+              : dispatch_forward<Real, false>(d, x, nodes, w, out, records, stream, img, norm);
 }
 
 // ---- maps on the row kernel's walk ----------------------------------------------------------------------------------
@@ -1248,7 +1262,8 @@ int forest_maps_rows(const ForestDims &d, bool fern, const Real *x, const Real *
                                 unsigned long long *);                                                                \
   template size_t forest_forward_workspace<Real>(const ForestDims &);                                                 \
   template int forest_forward<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,            \
-                                    const Real *, Real *, void *, void *, size_t, hipStream_t, const ImageStore *);   \
+                                    const Real *, Real *, void *, void *, size_t, hipStream_t, const ImageStore *,    \
+                                    const FeatureNorm<Real> *);                                                       \
   template size_t forest_maps_rows_workspace<Real>(const ForestDims &);                                               \
   template int forest_maps_rows<Real>(const ForestDims &, bool, const Real *, const Real *, const int64_t *,          \
                                       int64_t *, uint16_t *, Real *, int64_t *, void *, hipStream_t);

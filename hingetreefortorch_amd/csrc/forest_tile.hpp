@@ -24,7 +24,8 @@ static inline int pick_tile(int F, size_t reserve) {
 // wave * CPW ... (wave + 1) * CPW), so the 128-byte lines of a row are requested by consecutive loads of one wavefront
 // and reach L2 as one request each, rather than once from each of four wavefronts.
 template <typename Real, int BT, int NT>
-__device__ __forceinline__ void load_tile(Real *xs, const Real *__restrict__ x, const ForestDims &d, long long s0) {
+__device__ __forceinline__ void load_tile(Real *xs, const Real *__restrict__ x, const ForestDims &d, long long s0,
+                                          const FeatureNorm<Real> norm = FeatureNorm<Real>()) {
   typedef Real Vec4 __attribute__((ext_vector_type(4)));
   const int j = threadIdx.x % BT;
   const long long s = s0 + j;
@@ -41,13 +42,20 @@ __device__ __forceinline__ void load_tile(Real *xs, const Real *__restrict__ x, 
     for (int c = span * cpw + r; c < c_end; c += R) {
       Vec4 v = {Real(0), Real(0), Real(0), Real(0)};
       if (live) v = *reinterpret_cast<const Vec4 *>(x + base + 4 * c);
+      if (norm.mean != nullptr && live) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (v[i] - norm.mean[4 * c + i]) * norm.rstd[4 * c + i];
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) xs[(4 * c + i) * BT + j] = v[i];
     }
     return;
   }
-  for (int f = threadIdx.x / BT; f < d.F; f += NT / BT)
-    xs[f * BT + j] = live ? x[base + (long long)f * d.K] : Real(0);
+  for (int f = threadIdx.x / BT; f < d.F; f += NT / BT) {
+    Real v = live ? x[base + (long long)f * d.K] : Real(0);
+    if (norm.mean != nullptr && live) v = (v - norm.mean[f]) * norm.rstd[f];
+    xs[f * BT + j] = v;
+  }
 }
 
 // Flat offset of element (sample s, tree t, output m) of the [B, T, K, M] output / upstream-gradient tensors.

@@ -806,7 +806,9 @@ __global__ __launch_bounds__(256) void segment_sums_kernel(ForestDims d, Records
                                                            const float *__restrict__ c,
                                                            const uint32_t *__restrict__ perm,
                                                            const float *__restrict__ xc, int K,
-                                                           const float *__restrict__ zhat, float *acc_out,
+                                                           const float *__restrict__ zhat,
+                                                           const float *__restrict__ z_mean,
+                                                           const float *__restrict__ z_rstd, float *acc_out,
                                                            double *m2sum) {
   const int lane = threadIdx.x & (kWave - 1);
   const long long blocks_per_tree = (d.S + kWave - 1) / kWave;
@@ -824,7 +826,10 @@ __global__ __launch_bounds__(256) void segment_sums_kernel(ForestDims d, Records
     c_mine = c[first + s_mine];
     v_mine = rec.vertex(first + s_mine);
     n_mine = min(rec.ord(first + s_mine), uint32_t(d.F - 1));
-    p_mine = double(c_mine) * double(zhat[(long long)s_mine * d.F + n_mine]);
+    // (z_mean given: `zhat` holds the product before its normalisation, which is applied here as the forward applied it)
+    float zh = zhat[(long long)s_mine * d.F + n_mine];
+    if (z_mean != nullptr) zh = (zh - z_mean[n_mine]) * z_rstd[n_mine];
+    p_mine = double(c_mine) * double(zh);
   }
   // runs of equal vertices: bit l of `starts` says that entry l begins one
   const uint32_t v_before = uint32_t(__shfl_up(int(v_mine), 1, kWave));
@@ -925,8 +930,8 @@ ProjectionForestLayout projection_forest_layout(const ForestDims &d, long long K
 
 template <bool COMPACT>
 int projection_forest_sparse(const ForestDims &d, long long K, const void *records, const float *c, const float *xc,
-                             const float *zhat, uint32_t *perm, float *sparse, double *m2sum,
-                             hipStream_t stream) {
+                             const float *zhat, const float *z_mean, const float *z_rstd, uint32_t *perm, float *sparse,
+                             double *m2sum, hipStream_t stream) {
   // (the records are only read here; c comes from the forest pass)
   const Records<float, COMPACT> rec = carve_records<float, COMPACT>(d, const_cast<void *>(records), nullptr);
   auto bucket = bucket_kernel<COMPACT>;
@@ -935,12 +940,42 @@ int projection_forest_sparse(const ForestDims &d, long long K, const void *recor
   HT_LAUNCH_CHECK("projection + forest backward (samples by vertex)");
   const long long waves = (long long)d.T * ((d.S + kWave - 1) / kWave);
   hipLaunchKernelGGL(segment_sums_kernel<COMPACT>, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, d, rec, c,
-                     perm, xc, int(K), zhat, sparse, m2sum);
+                     perm, xc, int(K), zhat, z_mean, z_rstd, sparse, m2sum);
   HT_LAUNCH_CHECK("projection + forest backward (segment sums)");
   return HT_OK;
 }
 
 }  // namespace
+
+size_t projection_forest_forward_workspace(const ForestDims &d) {
+  return align_up(projection_workspace(d.F), 256) + forest_forward_workspace<float>(d);
+}
+
+// The forward pass of the whole front: z [B x N] = x [B x K] * lin [N x K]^T with its batch statistics (mean, rstd, var
+// [N] out), then the forest over the normalised product -- which is never written: the forest's kernels normalise z as
+// they read it ((z - mean) * rstd, the arithmetic of bn_apply_kernel), one pass over [B x N] less than
+// projection_forward + forest_forward. records (optional) as for forest_forward.
+int projection_forest_forward(const ForestDims &d, bool fern, long long K, const float *x, const float *lin, double eps,
+                              const float *thr, const int64_t *ord, const float *w, float *out, float *z, float *mean,
+                              float *rstd, float *var, void *records, void *ws, size_t ws_bytes, hipStream_t stream) {
+  int rc;
+  if (d.K != 1) return fail(HT_ERR_INVALID_ARGUMENT, "Error: the projection's forest has no inner data dimensions.");
+  if (ws == nullptr || ws_bytes < projection_forest_forward_workspace(d))
+    return fail(HT_ERR_INVALID_ARGUMENT, "Error: workspace too small for the forward pass.");
+  const long long B = d.S, N = d.F;
+  double *stats = static_cast<double *>(ws);
+  if ((rc = zero_fill(stats, size_t(2) * N * sizeof(double), stream)) != HT_OK) return rc;
+  if (B == 0 || N == 0) return HT_OK;
+  if ((rc = launch_gemm<true, true, true>(x, K, lin, K, z, N, B, N, K, stats, stream)) != HT_OK) return rc;
+  hipLaunchKernelGGL(bn_finalize_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, stats, int(N), B, eps,
+                     mean, rstd, var);
+  HT_LAUNCH_CHECK("batch statistics");
+  FeatureNorm<float> norm;
+  norm.mean = mean, norm.rstd = rstd;
+  unsigned char *forest_ws = static_cast<unsigned char *>(ws) + align_up(projection_workspace(N), 256);
+  return forest_forward<float>(d, fern, z, thr, ord, w, out, records, forest_ws,
+                               ws_bytes - align_up(projection_workspace(N), 256), stream, nullptr, &norm);
+}
 
 // Whether projection_forest_backward serves a forest [B x N features, K = 1] behind a projection from K_in inputs.
 bool projection_forest_backward_ok(const ForestDims &d, long long K) {
@@ -955,9 +990,10 @@ size_t projection_forest_backward_workspace(const ForestDims &d, long long K) {
 
 // dThr, dW of the forest and dLin of the projection in front of it, from the forest's walk records and upstream
 // gradient gout; no dense dL/dzhat is formed. x [B x K], lin [N x K], zhat [B x N], rstd [N] as projection_forward left
-// them; dthr / dw / dlin may be null.
+// them -- or, with mean [N] given, `zhat` is the product before its normalisation as projection_forest_forward left it;
+// dthr / dw / dlin may be null.
 int projection_forest_backward(const ForestDims &d, bool fern, long long K, const float *x, const float *lin,
-                               const float *zhat, const float *rstd, const float *w, const float *gout,
+                               const float *zhat, const float *mean, const float *rstd, const float *w, const float *gout,
                                const void *records, float *dthr, float *dw, float *dlin, void *ws, size_t ws_bytes,
                                hipStream_t stream) {
   int rc;
@@ -999,8 +1035,8 @@ int projection_forest_backward(const ForestDims &d, bool fern, long long K, cons
                                                             reduction_shares(K, K, B))) != HT_OK)
     return rc;
   if ((rc = launch_gemm<true, true, false>(lin, K, gram, K, dense, K, N, K, K, nullptr, stream)) != HT_OK) return rc;
-  rc = compact_ok(d) ? projection_forest_sparse<true>(d, K, records, c, xc, zhat, perm, sparse, m2sum, stream)
-                     : projection_forest_sparse<false>(d, K, records, c, xc, zhat, perm, sparse, m2sum, stream);
+  rc = compact_ok(d) ? projection_forest_sparse<true>(d, K, records, c, xc, zhat, mean, rstd, perm, sparse, m2sum, stream)
+                     : projection_forest_sparse<false>(d, K, records, c, xc, zhat, mean, rstd, perm, sparse, m2sum, stream);
   if (rc != HT_OK) return rc;
   const long long quads = N * (K / 4);
   hipLaunchKernelGGL(combine_dlin_kernel, dim3((unsigned)((quads + 255) / 256 < 8192 ? (quads + 255) / 256 : 8192)),

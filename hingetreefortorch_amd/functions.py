@@ -237,34 +237,34 @@ class LinearBatchNormForest(torch.autograd.Function):
     @staticmethod
     def forward(ctx, inData, inLinearWeights, eps, inThresholds, inOrdinals, inWeights, fern):
         pre = "fern" if fern else "tree"
-        zhat, mean, rstd, var = _ops.linear_bn_forward(inData, inLinearWeights, eps)
-        records = None
-        if any(ctx.needs_input_grad):
-            out, records = getattr(_ops, pre + "_forward_records")(zhat, inThresholds, inOrdinals, inWeights)
-        else:
-            out = getattr(_ops, pre + "_forward")(zhat, inThresholds, inOrdinals, inWeights)
+        # one call: the forest reads the un-normalised product z and normalises it on the way (no pass over [batch,
+        # features] to write zhat); the walk records are kept when a backward pass will follow
+        out, records, z, mean, rstd, var = getattr(_ops, pre + "_linear_bn_forward_records")(
+            inData, inLinearWeights, eps, inThresholds, inOrdinals, inWeights, want_records=any(ctx.needs_input_grad))
         ctx.pre = pre
         ctx.has_records = records is not None
-        saved = [inData, inLinearWeights, zhat, rstd, inThresholds, inOrdinals, inWeights]
+        saved = [inData, inLinearWeights, z, mean, rstd, inThresholds, inOrdinals, inWeights]
         ctx.save_for_backward(*(saved + ([records] if records is not None else [])))
         ctx.mark_non_differentiable(mean, var)
         return out, mean, var
 
     @staticmethod
     def backward(ctx, outDataGrad, _mean_grad, _var_grad):
-        inData, inLinearWeights, zhat, rstd, inThresholds, inOrdinals, inWeights = ctx.saved_tensors[:7]
+        inData, inLinearWeights, z, mean, rstd, inThresholds, inOrdinals, inWeights = ctx.saved_tensors[:8]
         need_x, need_lin, _, need_thr, need_ord, need_w, _ = ctx.needs_input_grad
         up = outDataGrad.contiguous()
         deterministic = _is_deterministic()
         if ctx.has_records and not need_x and not deterministic:
             got = getattr(_ops, ctx.pre + "_linear_bn_backward_records")(
-                ctx.saved_tensors[7], inData, inLinearWeights, need_lin, zhat, rstd, inThresholds, need_thr, inOrdinals,
-                inWeights, need_w, up)
+                ctx.saved_tensors[8], inData, inLinearWeights, need_lin, z, rstd, inThresholds, need_thr, inOrdinals,
+                inWeights, need_w, up, mean=mean)
             if got is not None:
                 return None, got[0], None, got[1], None, got[2], None
+        # the two separate backward passes, on the normalised product
+        zhat = (z - mean) * rstd
         args = (zhat, need_x or need_lin, inThresholds, need_thr, inOrdinals, need_ord, inWeights, need_w, up)
         if ctx.has_records:
-            dz, dthr, _, dw = getattr(_ops, ctx.pre + "_backward_records")(ctx.saved_tensors[7], deterministic, *args)
+            dz, dthr, _, dw = getattr(_ops, ctx.pre + "_backward_records")(ctx.saved_tensors[8], deterministic, *args)
         else:
             dz, dthr, _, dw = getattr(_ops, ctx.pre + ("_backward_deterministic" if deterministic else "_backward"))(*args)
         dx = dlin = None

@@ -412,23 +412,78 @@ def linear_bn_backward(inData, bInDataGrad, inLinearWeights, bInLinearWeightsGra
     return [dx, dlin]
 
 
+def _linear_bn_forward_records(kind, inData, inLinearWeights, eps, inThresholds, inOrdinals, inWeights,
+                               want_records=True):
+    """The forward pass of the whole front in one call: z = inData @ inLinearWeights.T with its batch statistics, then the
+    forest over (z - mean) * rstd, which is not written out (the forest's kernels normalise z as they read it; values
+    equal those of linear_bn_forward + *_forward_records bit for bit, the records hold the same walks). Returns [out, records | None, z,
+    mean, rstd, var]; z, mean, rstd go to *_linear_bn_backward_records (zhat = z, mean = mean). want_records=False: no
+    backward pass will follow."""
+    for t in (inData, inLinearWeights, inThresholds, inWeights):
+        if t.dtype != torch.float32:
+            _invalid("Error: the projection supports torch.float32 only.")
+    for t in (inData, inLinearWeights):
+        if not t.is_contiguous():
+            _invalid("Error: All tensors are expected to be contiguous.")
+    if inData.device != inLinearWeights.device:
+        _invalid("Error: All tensors are expected to be on the same device.")
+    if not inData.is_cuda:
+        _runtime("Error: this build has no CPU back-end; tensors must be on a GPU.")
+    if inData.dim() != 2 or inLinearWeights.dim() != 2 or inData.shape[1] != inLinearWeights.shape[1]:
+        _invalid("Error: inData must be [batch, in_features] and inLinearWeights [out_features, in_features].")
+    B, K = inData.shape
+    N = inLinearWeights.shape[0]
+    if B == 0:
+        _invalid("Error: batch statistics need at least one sample.")
+    lib = L.load()
+    dev = inData.device
+    with torch.cuda.device(dev):
+        z = torch.empty([B, N], dtype=torch.float32, device=dev)
+        _common_checks([z, inThresholds, inWeights], inOrdinals, False)
+        shape, out_sizes = _forest_shape(kind, z, inThresholds, inOrdinals, inWeights)
+        mean, rstd, var = (torch.empty([N], dtype=torch.float32, device=dev) for _ in range(3))
+        out = torch.empty(out_sizes, dtype=torch.float32, device=dev)
+        rbytes = lib.ht_forest_records_bytes(ctypes.byref(shape)) if want_records else 0
+        records = torch.empty([rbytes], dtype=torch.uint8, device=dev) if rbytes else None
+        nbytes = lib.ht_projection_forest_forward_workspace(ctypes.byref(shape))
+        ws = _workspace(nbytes, dev)
+        L.check(lib.ht_projection_forest_forward(ctypes.byref(shape), K, _ptr(inData), _ptr(inLinearWeights), float(eps),
+                                                 _ptr(inThresholds), _ptr(inOrdinals), _ptr(inWeights), _ptr(out), _ptr(z),
+                                                 _ptr(mean), _ptr(rstd), _ptr(var), _ptr(records), rbytes, _ptr(ws), nbytes,
+                                                 _stream(dev)))
+    return [out, records, z, mean, rstd, var]
+
+
+def tree_linear_bn_forward_records(*args, **kwargs):
+    return _linear_bn_forward_records(L.HT_TREE, *args, **kwargs)
+
+
+def fern_linear_bn_forward_records(*args, **kwargs):
+    return _linear_bn_forward_records(L.HT_FERN, *args, **kwargs)
+
+
+tree_linear_bn_forward_records.__doc__ = fern_linear_bn_forward_records.__doc__ = _linear_bn_forward_records.__doc__
+
+
 def _linear_bn_backward_records(kind, records, inData, inLinearWeights, bInLinearWeightsGrad, zhat, rstd, inThresholds,
-                                bInThresholdsGrad, inOrdinals, inWeights, bInWeightsGrad, outDataGrad):
+                                bInThresholdsGrad, inOrdinals, inWeights, bInWeightsGrad, outDataGrad, mean=None):
     """Backward of the whole front linear_bn_forward -> *_forward_records(zhat, ...) for an upstream gradient on the
     forest's output, when no gradient of inData is wanted: [dLinearWeights | None, dThresholds | None, dWeights | None]
     from the forest's walk records, without forming the dense gradient on zhat (it has one non-zero per sample and
-    tree). Returns None where the library does not serve the shape this way (the caller then runs *_backward_records
-    and linear_bn_backward)."""
+    tree). With `mean`, `zhat` is the un-normalised product z of *_linear_bn_forward_records. Returns None where the
+    library does not serve the shape this way (the caller then runs *_backward_records and linear_bn_backward)."""
     if not isinstance(records, torch.Tensor) or records.dtype != torch.uint8 or not records.is_contiguous():
         _invalid("Error: records must be the contiguous uint8 tensor a *_forward_records call returned.")
     for t in (inData, inLinearWeights, zhat, rstd, inThresholds, inWeights, outDataGrad):
         if t.dtype != torch.float32:
             _invalid("Error: the projection supports torch.float32 only.")
-    for t in (inData, inLinearWeights, zhat, rstd, records):
+    for t in (inData, inLinearWeights, zhat, rstd, records) + (() if mean is None else (mean,)):
         if not t.is_contiguous():
             _invalid("Error: All tensors are expected to be contiguous.")
         if t.device != inData.device:
             _invalid("Error: All tensors are expected to be on the same device.")
+    if mean is not None and (mean.dtype != torch.float32 or mean.shape != rstd.shape):
+        _invalid("Error: shapes of zhat / rstd do not match the projection.")
     if not inData.is_cuda:
         _runtime("Error: this build has no CPU back-end; tensors must be on a GPU.")
     _common_checks([zhat, inThresholds, inWeights, outDataGrad], inOrdinals, True)
@@ -452,18 +507,18 @@ def _linear_bn_backward_records(kind, records, inData, inLinearWeights, bInLinea
         dw = torch.empty_like(inWeights) if bInWeightsGrad else None
         ws = _workspace(nbytes, inData.device)
         L.check(lib.ht_projection_forest_backward(ctypes.byref(shape), K, _ptr(inData), _ptr(inLinearWeights), _ptr(zhat),
-                                                  _ptr(rstd), _ptr(inWeights), _ptr(outDataGrad), _ptr(records),
+                                                  _ptr(mean), _ptr(rstd), _ptr(inWeights), _ptr(outDataGrad), _ptr(records),
                                                   records.numel(), _ptr(dthr), _ptr(dw), _ptr(dlin), _ptr(ws), nbytes,
                                                   _stream(inData.device)))
     return [dlin, dthr, dw]
 
 
-def tree_linear_bn_backward_records(*args):
-    return _linear_bn_backward_records(L.HT_TREE, *args)
+def tree_linear_bn_backward_records(*args, **kwargs):
+    return _linear_bn_backward_records(L.HT_TREE, *args, **kwargs)
 
 
-def fern_linear_bn_backward_records(*args):
-    return _linear_bn_backward_records(L.HT_FERN, *args)
+def fern_linear_bn_backward_records(*args, **kwargs):
+    return _linear_bn_backward_records(L.HT_FERN, *args, **kwargs)
 
 
 tree_linear_bn_backward_records.__doc__ = fern_linear_bn_backward_records.__doc__ = _linear_bn_backward_records.__doc__

@@ -203,10 +203,23 @@ int ht_projection_backward(int64_t B, int64_t K, int64_t N, const float *x, cons
  *   ht_forest_backward_records. Atomic accumulation (the order of additions, hence the last bits, can differ between
  *   runs). ht_projection_forest_backward_workspace returns 0 where the shape is not served (K_in not a multiple of 4,
  *   K > 1, more than 16384 vertices per tree, shapes whose records the staged kernels do not take): call
- *   ht_forest_backward_records + ht_projection_backward there. */
+ *   ht_forest_backward_records + ht_projection_backward there.
+ *   mean [N]: NULL when `zhat` is the normalised product; when `zhat` is the product z before its normalisation, as
+ *   ht_projection_forest_forward leaves it, its batch means (the normalisation is then applied where zhat is read).
+ * ht_projection_forest_forward is the matching forward pass: z [B, N] = x * lin^T on the matrix cores with its batch
+ * statistics (mean, rstd [N]; var [N], biased, may be NULL), then the forest over (z - mean) * rstd, which is not
+ * written out -- the forest's kernels normalise z as they read it, with the two rounded operations a separate pass
+ * would use, so `out` equals that of ht_projection_forward + ht_forest_forward_records bit for bit and the records hold
+ * the same walks.
+ * records may be NULL (no backward pass will follow). */
+size_t ht_projection_forest_forward_workspace(const ht_forest_shape *forest);
+int ht_projection_forest_forward(const ht_forest_shape *forest, int64_t K_in, const float *x, const float *lin, double eps,
+                                 const float *thr, const int64_t *ord, const float *w, float *out, float *z, float *mean,
+                                 float *rstd, float *var, void *records, size_t records_bytes, void *workspace,
+                                 size_t workspace_bytes, void *stream);
 size_t ht_projection_forest_backward_workspace(const ht_forest_shape *forest, int64_t K_in);
 int ht_projection_forest_backward(const ht_forest_shape *forest, int64_t K_in, const float *x, const float *lin,
-                                  const float *zhat, const float *rstd, const float *w, const float *gout,
+                                  const float *zhat, const float *mean, const float *rstd, const float *w, const float *gout,
                                   const void *records, size_t records_bytes, float *dthr, float *dw, float *dlin,
                                   void *workspace, size_t workspace_bytes, void *stream);
 

@@ -194,3 +194,52 @@ def test_front_backward_from_records_rejects(dev):
         ops.tree_linear_bn_backward_records(rec[:-1].contiguous(), x, lin, True, zhat, rstd, thr, True, ordn, w, True, up)
     with pytest.raises(ValueError):
         ops.tree_linear_bn_backward_records(rec, x.double(), lin, True, zhat, rstd, thr, True, ordn, w, True, up)
+
+
+FUSED_FORWARD_CASES = [
+    # B, K_in, N features, trees, depth, outputs per leaf, fern
+    (200, 36, 42, 6, 3, 4, False),       # a tile of samples holds all features in LDS
+    (96, 8, 30, 5, 5, 3, True),
+    (70, 12, 5200, 40, 7, 2, False),     # more features than any tile holds: the walk reads them from memory
+    (33, 5, 9, 2, 2, 1, False),
+]
+
+
+@pytest.mark.parametrize("case", FUSED_FORWARD_CASES, ids=[f"c{i}" for i in range(len(FUSED_FORWARD_CASES))])
+def test_front_forward_in_one_call(dev, case):
+    """tree_linear_bn_forward_records (the forest normalises the product as it reads it) against linear_bn_forward +
+    tree_forward_records: statistics, forest output and walk records bit for bit, z such that (z - mean) * rstd is the
+    separate call's zhat bit for bit; then the backward from the records with the un-normalised product."""
+    B, K, N, T, depth, M, fern = case
+    g = torch.Generator().manual_seed(41)
+    V = depth if fern else 2 ** depth - 1
+    x = torch.rand([B, K], generator=g).to(dev)
+    lin = (torch.randn([N, K], generator=g) / K ** 0.5).to(dev)
+    thr = (3.0 * torch.rand([T, V], generator=g) - 1.5).to(dev)
+    ordn = torch.randint(0, N, (T, V), generator=g).to(dev)
+    w = torch.randn([T, 2 ** depth, M], generator=g).to(dev)
+    up = torch.randn([B, T, M], generator=g).to(dev)
+    pre = "fern" if fern else "tree"
+    zhat, mean, rstd, var = ops.linear_bn_forward(x, lin, 1e-5)
+    out, rec = getattr(ops, pre + "_forward_records")(zhat, thr, ordn, w)
+    fout, frec, z, fmean, frstd, fvar = getattr(ops, pre + "_linear_bn_forward_records")(x, lin, 1e-5, thr, ordn, w)
+    assert torch.equal(fmean, mean) and torch.equal(frstd, rstd) and torch.equal(fvar, var)
+    assert torch.equal((z - fmean) * frstd, zhat)
+    assert torch.equal(fout, out)
+    assert (frec is None) == (rec is None)
+    if rec is None:
+        return
+    # the same walks recorded: the packed words of all (tree, sample) pairs lead the buffer (what follows has alignment
+    # gaps and per-workgroup slots of a bound, which differ between the kernels that can write records)
+    assert torch.equal(frec[:4 * T * B], rec[:4 * T * B])
+    dense_a = getattr(ops, pre + "_backward_records")(rec, False, zhat, True, thr, True, ordn, False, w, True, up)
+    dense_b = getattr(ops, pre + "_backward_records")(frec, False, zhat, True, thr, True, ordn, False, w, True, up)
+    assert torch.equal(dense_a[0], dense_b[0])  # dX has one writer per element: no atomics, so bit for bit
+    if K % 4:
+        return
+    a = getattr(ops, pre + "_linear_bn_backward_records")(rec, x, lin, True, zhat, rstd, thr, True, ordn, w, True, up)
+    b = getattr(ops, pre + "_linear_bn_backward_records")(frec, x, lin, True, z, frstd, thr, True, ordn, w, True, up,
+                                                          mean=fmean)
+    assert a is not None and b is not None
+    for got, want in zip(b, a):
+        assert rel_err(got.cpu(), want.cpu()) <= 1e-5
