@@ -139,6 +139,7 @@ struct GemmArgs {
   int splits;                          // > 1: blockIdx.y takes a share of the reduction and adds into a zeroed C ...
   long long split_stride;              // ... or, if not 0, stores its share at C + blockIdx.y * split_stride
   bool vec_a, vec_b;
+  bool symmetric;  // A and B are the same operand: tiles below the diagonal are not computed but mirrored from above
   double *stats;
   const float *bias_i, *bias_j;
   // A_BN: operand A is not read as it lies in memory but as the batch-norm backward of it, element (i, r) =
@@ -174,7 +175,13 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(3,
   __shared__ float Bs[2][kRed * kPitch];
   const int n_i = g.n_i, n_j = g.n_j, n_r = g.n_r;
   int tile_i, tile_j;
-  if (!gemm_tile_of(int(blockIdx.x), g.tiles_i, g.tiles_j, g.rows_per_xcd, &tile_i, &tile_j)) return;
+  // A launch slot runs on XCD slot % 8 whatever its share of a split reduction is (the grid's x extent is a multiple
+  // of 8), and the tile map gives every XCD a band of tile rows: with few tile rows -- or a symmetric product, whose
+  // upper rows hold more tiles -- the shares would pile their work on the same XCDs, so share y takes the band of the
+  // XCD y places further on.
+  const int slot = int(blockIdx.x) - int(blockIdx.x) % kNumXCDs + (int(blockIdx.x) + int(blockIdx.y)) % kNumXCDs;
+  if (!gemm_tile_of(slot, g.tiles_i, g.tiles_j, g.rows_per_xcd, &tile_i, &tile_j)) return;
+  if (g.symmetric && tile_j < tile_i) return;
   const int i0 = tile_i * kTile, j0 = tile_j * kTile;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wavefront's 64 x 64 corner
@@ -340,10 +347,12 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(3,
           float v = acc[a][b][e];
           if (g.bias_i && first) v += g.bias_i[i];
           v += bj;
-          if (g.splits > 1 && g.split_stride == 0)
+          if (g.splits > 1 && g.split_stride == 0) {
             atomicAdd(C + (long long)i * g.ldc + j, v);
-          else
+          } else {
             C[(long long)i * g.ldc + j] = v;
+            if (g.symmetric && tile_i != tile_j) C[(long long)j * g.ldc + i] = v;
+          }
           if (STATS) {
             s1 += double(v);
             s2 += double(v) * double(v);
@@ -499,7 +508,7 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
                         long long stride_b, float *C, long long ldc, long long stride_c, long long n_i, long long n_j,
                         long long n_r, long long batches, double *stats, const float *bias_i, const float *bias_j,
                         hipStream_t stream, bool allow_split = false, float *partials = nullptr, int ordered_splits = 0,
-                        const BnOperand *bn = nullptr) {
+                        const BnOperand *bn = nullptr, bool symmetric = false) {
   if (n_i <= 0 || n_j <= 0 || batches <= 0) return HT_OK;
   if (!SUM_BATCHES && batches > kMaxGridZ) {
     // one result per batch rides on blockIdx.z: longer batch lists go out in several launches
@@ -527,6 +536,8 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
   if (slots > 0x7fffffffLL) return fail(HT_ERR_RUNTIME, "Error: matrix product too large for this build.");
   g.vec_a = aligned16(A, lda, stride_a), g.vec_b = aligned16(B, ldb, stride_b);
   g.stats = stats, g.bias_i = bias_i, g.bias_j = bias_j;
+  // (mirrored stores are plain stores: not with atomic shares, statistics or biases)
+  g.symmetric = symmetric && A == B && lda == ldb && n_i == n_j && ldc == n_j && !STATS && !bias_i && !bias_j && batches == 1;
   g.bn_zhat = g.bn_rstd = nullptr, g.bn_sums = nullptr, g.bn_count = 1.0;
   if (A_BN) {
     if (!bn || batches != 1) return fail(HT_ERR_RUNTIME, "Error: fused batch-norm operand needs its statistics.");
@@ -555,6 +566,7 @@ int launch_gemm_batched(const float *A, long long lda, long long stride_a, const
     HT_LAUNCH_CHECK("matrix product (sum of the shares)");
     return HT_OK;
   }
+  if (allow_split) g.symmetric = false;
   if (allow_split && !STATS && ldc == n_j && (SUM_BATCHES || batches == 1) && gi * gj < kNumCUs && all_steps >= 64) {
     long long want = (2 * kNumCUs + gi * gj - 1) / (gi * gj);
     if (want > all_steps / 16) want = all_steps / 16;
@@ -600,8 +612,9 @@ int reduction_shares(long long rows, long long cols, long long red) {
   if (tiles <= 0 || steps < 64) return 1;
   long long want;
   if (tiles < kNumCUs / 2) {
-    // a handful of tiles: enough shares to put two workgroups on every CU
-    want = (2 * kNumCUs + tiles - 1) / tiles;
+    // a handful of tiles: enough shares to put four workgroups on every CU (a workgroup alone on a CU waits out every
+    // operand latency by itself: xc^T xc of the README model, 49 tiles over 16 384 rows, 0.32 ms with 11 shares)
+    want = (4 * kNumCUs + tiles - 1) / tiles;
     if (want > steps / 16) want = steps / 16;
   } else {
     // A few tiles per CU: tiles are equal pieces of work, so 700 of them leave some CUs with three and some with two
@@ -1032,7 +1045,7 @@ int projection_forest_backward(const ForestDims &d, bool fern, long long K, cons
   // rows serve as the columns the product wants, reduction index contiguous)
   if ((rc = launch_gemm_batched<false, false, false, false>(xc, K, 0, xc, K, 0, gram, K, 0, K, K, B, 1, nullptr, nullptr,
                                                             nullptr, stream, false, partials,
-                                                            reduction_shares(K, K, B))) != HT_OK)
+                                                            reduction_shares(K, K, B), nullptr, true)) != HT_OK)
     return rc;
   if ((rc = launch_gemm<true, true, false>(lin, K, gram, K, dense, K, N, K, K, nullptr, stream)) != HT_OK) return rc;
   rc = compact_ok(d) ? projection_forest_sparse<true>(d, K, records, c, xc, zhat, mean, rstd, perm, sparse, m2sum, stream)
