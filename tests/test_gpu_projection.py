@@ -243,3 +243,35 @@ def test_front_forward_in_one_call(dev, case):
     assert a is not None and b is not None
     for got, want in zip(b, a):
         assert rel_err(got.cpu(), want.cpu()) <= 1e-5
+
+
+def test_linear_hinge_forest_routes_agree(dev):
+    """LinearHingeForest's training step by its three backward routes: from the walk records (inputs without gradient),
+    through a dense dL/dzhat (inputs with gradient), and in deterministic mode (dense, reproducible): the same parameter
+    gradients within fp32 tolerance, the deterministic ones bit for bit twice."""
+    torch.manual_seed(9)
+    B, K, T, depth, M = 160, 24, 7, 4, 3
+    model = LinearHingeForest(K, T, depth, extra_outputs=M).to(dev)
+    model.train()
+    x = torch.rand([B, K], device=dev)
+    up = torch.randn([B, T, M], device=dev)
+
+    def grads(requires_input_grad, deterministic):
+        model.zero_grad()
+        xi = x.clone().requires_grad_(requires_input_grad)
+        torch.use_deterministic_algorithms(deterministic)
+        try:
+            out = model(xi)
+            out.backward(up)
+        finally:
+            torch.use_deterministic_algorithms(False)
+        return [p.grad.clone() for p in (model.fc.weight, model.forest.thresholds, model.forest.weights)], out.detach()
+
+    rec, out_a = grads(False, False)
+    dense, out_b = grads(True, False)
+    det1, out_c = grads(False, True)
+    det2, _ = grads(False, True)
+    assert torch.equal(out_a, out_b) and torch.equal(out_a, out_c)
+    for a, b, c, d in zip(rec, dense, det1, det2):
+        assert rel_err(a.cpu(), b.cpu()) <= 2e-5 and rel_err(c.cpu(), b.cpu()) <= 2e-5
+        assert torch.equal(c, d)
