@@ -272,8 +272,10 @@ __device__ inline void det_pick_scale(double bound, double count, double *scale,
   frexp(bound, &e);  // bound < 2^e
   int bits = 0;
   while (ldexp(1.0, bits) < count) ++bits;
-  // a product rounded to Real can exceed the bound by an ulp: 61, not 62, keeps every sum inside int64
+  // a product rounded to Real can exceed the bound by an ulp: 61, not 62, keeps every sum inside int64; and a single
+  // term stays below 2^50 whatever the count (to_fixed)
   int k = 61 - e - bits;
+  if (k > 50 - e) k = 50 - e;
   k = k > 1000 ? 1000 : (k < -1000 ? -1000 : k);
   *scale = ldexp(1.0, k);
   *inv = ldexp(1.0, -k);
@@ -325,8 +327,12 @@ __global__ __launch_bounds__(256) void zero_if_kernel(unsigned long long *p, lon
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) p[i] = 0ull;
 }
 
+// round(v * scale) as a 64-bit integer, for |v * scale| < 2^51 (det_pick_scale keeps every term below 2^50): adding
+// 1.5 * 2^52 leaves the rounded integer, as a two's complement offset, in the low bits of the double -- one fused
+// multiply-add and one 64-bit subtraction where a conversion instruction sequence takes a dozen; same rounding (to
+// nearest, ties to even). Larger products (a sampled bound that did not hold: the run is repeated) give some integer.
 __device__ __forceinline__ unsigned long long to_fixed(double v, double scale) {
-  return (unsigned long long)__double2ll_rn(v * scale);
+  return (unsigned long long)(__double_as_longlong(__builtin_fma(v, scale, 0x1.8p52)) - 0x4338000000000000LL);
 }
 template <typename Real>
 __device__ __forceinline__ Real from_fixed(unsigned long long q, double inv) {
