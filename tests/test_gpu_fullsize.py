@@ -145,6 +145,20 @@ def test_projection_full_size(dev):
         assert rel_err(dlin[cs].double(), want) <= 2e-5, cs
     # dLin alone: the batch-norm backward ran inside the product's operand loader, the gradient buffer is as it came
     assert torch.equal(dz_in, up)
+    # the route the module takes: forward of the whole front in one call (the forest normalises the product as it reads
+    # it), backward from the walk records (no dense gradient on zhat): same outputs bit for bit, same gradients
+    print("case projection full size: one-call forward, backward from records", flush=True)
+    fout, frec, z, fmean, frstd, fvar = ops.tree_linear_bn_forward_records(x, lin, eps, gthr, gord, gw)
+    assert torch.equal(fmean, mean) and torch.equal(frstd, rstd) and torch.equal(fout, out)
+    assert torch.equal((z[rows] - fmean) * frstd, zhat[rows])
+    got = ops.tree_linear_bn_backward_records(frec, x, lin, True, z, frstd, gthr, True, gord, gw, True, gout, mean=fmean)
+    assert got is not None
+    rlin, rthr, rw = got
+    assert rel_err(rthr.cpu(), dthr.cpu()) <= 1e-5 and rel_err(rw.cpu(), dw.cpu()) <= 1e-5
+    for cs in col_sets:
+        gd, rz = up[:, cs].double(), zhat[:, cs].double()
+        dz = rstd[cs].double() * (gd - gd.mean(0) - rz * (gd * rz).mean(0))
+        assert rel_err(rlin[cs].double(), dz.t() @ x64) <= 2e-5, cs
 
 
 def test_conv_full_size(dev):
