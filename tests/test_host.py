@@ -289,3 +289,27 @@ def test_library_sources_never_allocate_device_memory():
     for f in files:
         text = open(f).read()
         assert not banned.search(text), f
+
+
+def test_front_operators_validate_on_cpu_tensors():
+    """The operators of the Linear -> BatchNorm -> forest front refuse what they cannot serve before they touch the
+    library's kernels: other dtypes, records that are not a forward pass's byte buffer, and CPU tensors (this build has
+    no CPU back-end)."""
+    g = torch.Generator().manual_seed(2)
+    B, K, N, T, depth, M = 16, 8, 14, 2, 3, 2
+    x, lin = torch.rand([B, K], generator=g), torch.randn([N, K], generator=g)
+    thr, ordn = torch.rand([T, 7], generator=g), torch.randint(0, N, (T, 7), generator=g)
+    w, up = torch.randn([T, 8, M], generator=g), torch.randn([B, T, M], generator=g)
+    zhat, rstd = torch.randn([B, N], generator=g), torch.rand([N], generator=g)
+    records = torch.zeros([64], dtype=torch.uint8)
+    with pytest.raises(ValueError, match="float32"):
+        ops.tree_linear_bn_forward_records(x.double(), lin, 1e-5, thr, ordn, w)
+    with pytest.raises(RuntimeError, match="no CPU back-end"):
+        ops.tree_linear_bn_forward_records(x, lin, 1e-5, thr, ordn, w)
+    with pytest.raises(ValueError, match="records must be"):
+        ops.tree_linear_bn_backward_records(records.float(), x, lin, True, zhat, rstd, thr, True, ordn, w, True, up)
+    with pytest.raises(ValueError, match="float32"):
+        ops.fern_linear_bn_backward_records(records, x, lin.double(), True, zhat, rstd, thr, True, ordn, w, True, up)
+    with pytest.raises(RuntimeError, match="no CPU back-end"):
+        ops.tree_linear_bn_backward_records(records, x, lin, True, zhat, rstd, thr, True, ordn, w, True, up)
+    assert HingeTree.LinearBatchNormForest is not None and hasattr(ops, "fern_linear_bn_forward_records")
