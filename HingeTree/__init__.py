@@ -10,6 +10,7 @@ from hingetreefortorch_amd.functions import (  # noqa: F401
     HingeFernConv2d,
     HingeFernConv3d,
     LinearBatchNorm,
+    LinearBatchNormForest,
     HingeTreeFusedLinear,
     HingeFernFusedLinear,
     HingeTreeExpanded,

@@ -6,7 +6,7 @@
     hingetreefortorch_amd.build           hipcc build of libhingetree_hip.so (csrc/, include/hingetree_hip.h)
 """
 from . import hingetree_cpp  # noqa: F401
-from .functions import HingeFern, HingeTree, LinearBatchNorm  # noqa: F401
+from .functions import HingeFern, HingeTree, LinearBatchNorm, LinearBatchNormForest  # noqa: F401
 from .modules import (  # noqa: F401
     HingeFernConv1d,
     HingeFernConv2d,
