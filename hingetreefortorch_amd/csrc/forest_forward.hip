@@ -540,6 +540,17 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
   const int t_end = min(d.T, t_begin + trees_per_block);
   const uint32_t TM = uint32_t(d.T) * uint32_t(d.M);
   MarginBits margin_bound;  // RECORD: bound on the |margin| this lane recorded
+  // Single-output rows: a wavefront step's run of a sample is TPW * 4 bytes, half a 64-byte sector or less, and the
+  // other half is written by another wavefront at another time. Streaming stores send each half to memory by itself
+  // (the fern benchmark wrote 922 MB for 786 MB); ordinary stores let the L2 put the halves together first (forward
+  // 0.458 -> 0.430 ms there). Wider rows fill their sectors and stream (ordinary stores: 0.89 -> 1.39 ms at 10 outputs).
+  const bool narrow_rows = d.M == 1;
+  auto store_out = [&](Vec v, Real *at) {
+    if (GW == 1 && narrow_rows)
+      *reinterpret_cast<Vec *>(at) = v;
+    else
+      __builtin_nontemporal_store(v, reinterpret_cast<Vec *>(at));
+  };
 
   // Output phase, lane constants of burst slot q for `un` slots per burst and u vectors per sample: where the parked
   // walk result of the vector's pair lies, the vector's column in the leaf table of the step's first tree, and its
@@ -664,7 +675,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
             o[1] = a[q] * wv[q][1];
             const Real from_next = value_of_next_lane(o[1]);
             if (odd_role == 1) o[1] = from_next;
-            if (live_q[q] && odd_role != 2) __builtin_nontemporal_store(o, reinterpret_cast<Vec *>(obase + off[q]));
+            if (live_q[q] && odd_role != 2) store_out(o, obase + off[q]);
             park[q] += samples * LDP;
             off[q] += samples * TM;
             g[q] += per_iteration;
@@ -702,7 +713,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
           if (odd_role == 1) o[q][1] = from_next;
           // (ordinary stores for the pairs in sectors that the step's run covers only in part -- an odd run of 8 M
           // elements is not a whole number of 64-byte sectors -- were measured and cost 15 %)
-          if (live_q[q] && odd_role != 2) __builtin_nontemporal_store(o[q], reinterpret_cast<Vec *>(obase + off[q]));
+          if (live_q[q] && odd_role != 2) store_out(o[q], obase + off[q]);
         }
       }
       __builtin_amdgcn_wave_barrier();
@@ -739,7 +750,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
           Vec o;
 #pragma unroll
           for (int i = 0; i < GW; ++i) o[i] = a[q] * wv[q][i];
-          __builtin_nontemporal_store(o, reinterpret_cast<Vec *>(obase + off[q]));
+          store_out(o, obase + off[q]);
           park[q] += park_step;
           off[q] += off_step;
         }
@@ -776,7 +787,7 @@ __global__ __launch_bounds__(kForestThreads) void forward_rows_kernel(ForestDims
             // streaming store: the output is written once and not read here, so it should not displace the vertices
             // and leaf weights that the gathers keep re-reading from L2 (measured: 1.45 -> 1.17 ms at the headline
             // shape)
-            __builtin_nontemporal_store(o, reinterpret_cast<Vec *>(obase + off[q]));
+            store_out(o, obase + off[q]);
           }
         }
       }
